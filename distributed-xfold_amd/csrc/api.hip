@@ -1,0 +1,318 @@
+// C ABI of libaf3hip.so (declared in include/af3_hip.h): argument checks,
+// workspace carving and kernel sequencing.  No allocation, no synchronisation.
+#include "../../include/af3_hip.h"
+#include "kernels.h"
+
+namespace {
+
+constexpr int C_PAIR = 128;
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+inline int64_t pad8(int64_t n) { return (n + 7) / 8 * 8; }
+
+// bump allocator over the caller's workspace
+struct Carver {
+  char* base;
+  size_t size, used = 0;
+  bool ok = true;
+  Carver(void* p, size_t n) : base(static_cast<char*>(p)), size(n) {}
+  template <typename T> T* take(size_t count) {
+    const size_t bytes = align_up(count * sizeof(T), 256);
+    if (!base || used + bytes > size) { ok = false; return nullptr; }
+    T* r = reinterpret_cast<T*>(base + used);
+    used += bytes;
+    return r;
+  }
+};
+
+inline bool bad_dtype(int d) { return d != AF3_BF16 && d != AF3_F32; }
+inline bool misaligned(const void* p) { return ((uintptr_t)p & 15) != 0; }
+
+}  // namespace
+
+extern "C" {
+
+int af3_abi_version(void) { return 1; }
+
+const char* af3_error_string(int code) {
+  switch (code) {
+    case AF3_OK: return "ok";
+    case AF3_ERR_BAD_ARG: return "bad argument (null/misaligned pointer, shape or dtype)";
+    case AF3_ERR_WORKSPACE: return "workspace missing or too small";
+    case AF3_ERR_LAUNCH: return "kernel launch failed";
+    case AF3_ERR_UNSUPPORTED: return "unsupported shape (channels / head dimension)";
+    default: return "unknown error";
+  }
+}
+
+// ------------------------------------------------------ triangle multiplication
+size_t af3_triangle_multiplication_workspace_bytes(int64_t n) {
+  if (n <= 0) return 0;
+  return 3 * align_up((size_t)C_PAIR * n * pad8(n) * sizeof(bf16_t), 256);
+}
+
+int af3_triangle_multiplication_forward(
+    const void* act, int io_dtype, const float* mask, int equation_flag,
+    const float* ln_in_w, const float* ln_in_b, const uint16_t* w_proj_gate,
+    const float* ln_c_w, const float* ln_c_b, const uint16_t* w_out, const uint16_t* w_gl,
+    void* out, int residual, int64_t n, void* workspace, size_t workspace_bytes, af3_stream_t stream) {
+  if (!act || !out || !ln_in_w || !ln_in_b || !w_proj_gate || !ln_c_w || !ln_c_b || !w_out || !w_gl)
+    return AF3_ERR_BAD_ARG;
+  if (bad_dtype(io_dtype) || n <= 0 || n > 8192 || (equation_flag != 0 && equation_flag != 1)) return AF3_ERR_BAD_ARG;
+  if (misaligned(act) || misaligned(out) || misaligned(mask)) return AF3_ERR_BAD_ARG;
+  const int64_t np = pad8(n);
+  Carver ws(workspace, workspace_bytes);
+  bf16_t* a_buf = ws.take<bf16_t>((size_t)C_PAIR * n * np);
+  bf16_t* b_buf = ws.take<bf16_t>((size_t)C_PAIR * n * np);
+  bf16_t* t_buf = ws.take<bf16_t>((size_t)C_PAIR * n * np);
+  if (!ws.ok) return AF3_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+
+  TriMulArgs a;
+  a.pair = act; a.mask = mask; a.out = out;
+  a.io_f32 = io_dtype == AF3_F32; a.N = (int)n; a.Np = (int)np;
+  a.outgoing = equation_flag == 0; a.residual = residual != 0;
+  a.ln_in_w = ln_in_w; a.ln_in_b = ln_in_b; a.ln_c_w = ln_c_w; a.ln_c_b = ln_c_b;
+  a.w_pg = w_proj_gate; a.w_gl = w_gl; a.w_out = w_out;
+  a.a_buf = a_buf; a.b_buf = b_buf; a.t_buf = t_buf;
+  int rc = launch_trimul_prologue(a, s);
+  if (rc) return rc;
+
+  // outgoing: t[c][i][j] = sum_k a'[c][i][k] b'[c][j][k]
+  // incoming: t[c][i][j] = sum_k b'[c][i][k] a'[c][j][k]  (a', b' stored transposed by the prologue)
+  GemmArgs g;
+  g.A = a.outgoing ? a_buf : b_buf;
+  g.B = a.outgoing ? b_buf : a_buf;
+  g.C = t_buf;
+  g.M = g.N = (int)n; g.K = (int)np; g.batch = C_PAIR;
+  g.lda = g.ldb = g.ldc = np;
+  g.sA = g.sB = g.sC = n * np;
+  rc = launch_gemm_nt(g, s);
+  if (rc) return rc;
+  return launch_trimul_epilogue(a, s);
+}
+
+// ------------------------------------------------------------ triangle attention
+size_t af3_grid_self_attn_workspace_bytes(int64_t n, int num_head) {
+  if (n <= 0 || num_head <= 0) return 0;
+  return align_up((size_t)n * n * 4 * C_PAIR * sizeof(bf16_t), 256) +
+         align_up((size_t)n * n * C_PAIR * sizeof(bf16_t), 256) +
+         align_up((size_t)num_head * n * n * sizeof(float), 256);
+}
+
+int af3_grid_self_attn_forward(
+    const void* pair, int io_dtype, const float* mask, int transpose,
+    const float* ln_w, const float* ln_b, const uint16_t* w_pair_bias, const float* nonbatched_bias,
+    const uint16_t* w_qkvg, const uint16_t* w_output, int num_head,
+    void* out, int residual, int64_t n, void* workspace, size_t workspace_bytes, af3_stream_t stream) {
+  if (!pair || !out || !w_qkvg || !w_output) return AF3_ERR_BAD_ARG;
+  if (bad_dtype(io_dtype) || n <= 0 || n > 8192 || num_head <= 0 || C_PAIR % num_head) return AF3_ERR_BAD_ARG;
+  if ((ln_w == nullptr) != (ln_b == nullptr)) return AF3_ERR_BAD_ARG;
+  if (w_pair_bias && nonbatched_bias) return AF3_ERR_BAD_ARG;
+  if (misaligned(pair) || misaligned(out) || misaligned(mask) || misaligned(nonbatched_bias)) return AF3_ERR_BAD_ARG;
+  const int d = C_PAIR / num_head;
+  if (d != 32) return AF3_ERR_UNSUPPORTED;
+  Carver ws(workspace, workspace_bytes);
+  bf16_t* qkvg = ws.take<bf16_t>((size_t)n * n * 4 * C_PAIR);
+  bf16_t* og = ws.take<bf16_t>((size_t)n * n * C_PAIR);
+  float* nb = ws.take<float>((size_t)num_head * n * n);
+  if (!ws.ok) return AF3_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+
+  AttnProjArgs p;
+  p.pair = pair; p.io_f32 = io_dtype == AF3_F32; p.N = (int)n; p.transpose = transpose != 0;
+  p.ln_w = ln_w; p.ln_b = ln_b;
+  p.w_main = w_qkvg; p.n_chunks = 4;
+  p.chunk_ops = SEG_BIAS_SCALE | (SEG_PLAIN << 4) | (SEG_PLAIN << 8) | (SEG_SIGMOID << 12);
+  p.q_scale = 1.0f / sqrtf((float)d);
+  p.out_main = qkvg; p.ld_main = 4 * C_PAIR;
+  p.w_bias = w_pair_bias; p.n_bias = w_pair_bias ? num_head : 0; p.out_bias = nb;
+  p.skip_ln = ln_w == nullptr;
+  int rc = launch_attn_proj(p, s);
+  if (rc) return rc;
+
+  FlashArgs f;
+  f.q = qkvg; f.k = qkvg + C_PAIR; f.v = qkvg + 2 * C_PAIR; f.g = qkvg + 3 * C_PAIR;
+  f.q_ss = f.k_ss = f.v_ss = f.g_ss = 4 * C_PAIR;
+  f.q_sb = f.k_sb = f.v_sb = f.g_sb = n * 4 * C_PAIR;
+  f.out = og; f.out_f32 = 0; f.o_ss = C_PAIR; f.o_sb = n * C_PAIR;
+  f.B = (int)n; f.H = num_head; f.Sq = f.Sk = (int)n; f.d = d;
+  f.bias = w_pair_bias ? nb : nonbatched_bias;
+  f.bias_sb = 0; f.bias_sh = n * n; f.bias_sq = n;
+  f.key_mask = mask; f.km_sb = n;
+  rc = launch_flash_attention(f, s);
+  if (rc) return rc;
+
+  AttnOutArgs o;
+  o.og = og; o.ld_og = C_PAIR; o.w_out = w_output; o.pair = pair; o.out = out;
+  o.io_f32 = p.io_f32; o.N = (int)n; o.transpose = p.transpose; o.residual = residual != 0;
+  return launch_attn_out(o, s);
+}
+
+// -------------------------------------------------------------------- transition
+int af3_transition_forward(
+    const void* act, int io_dtype, const float* ln_w, const float* ln_b,
+    const uint16_t* w1_packed, const uint16_t* w2, int hidden,
+    void* out, int residual, int64_t rows, af3_stream_t stream) {
+  if (!act || !out || !ln_w || !ln_b || !w1_packed || !w2) return AF3_ERR_BAD_ARG;
+  if (bad_dtype(io_dtype) || rows <= 0 || rows > 0x7fffffff || hidden <= 0 || (hidden & 63)) return AF3_ERR_BAD_ARG;
+  TransitionArgs t;
+  t.x = act; t.out = out; t.io_f32 = io_dtype == AF3_F32; t.N = (int)rows; t.hidden = hidden;
+  t.residual = residual != 0; t.ln_w = ln_w; t.ln_b = ln_b; t.w1 = w1_packed; t.w2 = w2;
+  return launch_transition(t, static_cast<hipStream_t>(stream));
+}
+
+// ------------------------------------------- pair-biased self-attention (single / diffusion)
+size_t af3_batch_diffusion_self_attention_workspace_bytes(int64_t batch, int64_t seq, int channels) {
+  if (batch <= 0 || seq <= 0 || channels <= 0) return 0;
+  return align_up((size_t)batch * seq * 4 * channels * sizeof(bf16_t), 256);
+}
+
+int af3_batch_diffusion_self_attention_forward(
+    const uint16_t* q_data, const float* key_mask, const float* nonbatched_bias,
+    const uint16_t* w_qkvg, const float* query_b, int num_head,
+    void* out, int out_dtype, int64_t batch, int64_t seq, int channels,
+    void* workspace, size_t workspace_bytes, af3_stream_t stream) {
+  if (!q_data || !w_qkvg || !out) return AF3_ERR_BAD_ARG;
+  if (bad_dtype(out_dtype) || batch <= 0 || seq <= 0 || channels <= 0 || (channels & 7) || num_head <= 0 ||
+      channels % num_head)
+    return AF3_ERR_BAD_ARG;
+  if (batch * seq > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  const int d = channels / num_head;
+  if (d != 24 && d != 32 && d != 48) return AF3_ERR_UNSUPPORTED;
+  Carver ws(workspace, workspace_bytes);
+  bf16_t* qkvg = ws.take<bf16_t>((size_t)batch * seq * 4 * channels);
+  if (!ws.ok) return AF3_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+
+  GemmArgs g;
+  g.A = q_data; g.B = w_qkvg; g.C = qkvg;
+  g.M = (int)(batch * seq); g.N = 4 * channels; g.K = channels;
+  g.lda = channels; g.ldb = channels; g.ldc = 4 * channels;
+  g.epi = EPI_SEGMENTED; g.seg_len = channels;
+  g.seg_ops = SEG_BIAS_SCALE | (SEG_PLAIN << 4) | (SEG_PLAIN << 8) | (SEG_SIGMOID << 12);
+  g.alpha = 1.0f / sqrtf((float)d);
+  g.bias = query_b;
+  int rc = launch_gemm_nt(g, s);
+  if (rc) return rc;
+
+  FlashArgs f;
+  f.q = qkvg; f.k = qkvg + channels; f.v = qkvg + 2 * channels; f.g = qkvg + 3 * channels;
+  f.q_ss = f.k_ss = f.v_ss = f.g_ss = 4 * channels;
+  f.q_sb = f.k_sb = f.v_sb = f.g_sb = seq * 4 * channels;
+  f.out = out; f.out_f32 = out_dtype == AF3_F32; f.o_ss = channels; f.o_sb = seq * channels;
+  f.B = (int)batch; f.H = num_head; f.Sq = f.Sk = (int)seq; f.d = d;
+  f.bias = nonbatched_bias; f.bias_sb = 0; f.bias_sh = seq * seq; f.bias_sq = seq;
+  f.key_mask = key_mask; f.km_sb = 0;
+  return launch_flash_attention(f, s);
+}
+
+// --------------------------------------------------- windowed (atom) cross-attention
+size_t af3_batch_diffusion_cross_attention_workspace_bytes(int64_t batch, int64_t sq, int64_t sk, int channels) {
+  if (batch <= 0 || sq <= 0 || sk <= 0 || channels <= 0) return 0;
+  return align_up((size_t)batch * sq * 2 * channels * sizeof(bf16_t), 256) +
+         align_up((size_t)batch * sk * 2 * channels * sizeof(bf16_t), 256);
+}
+
+int af3_batch_diffusion_cross_attention_forward(
+    const uint16_t* q_data, const uint16_t* m_data,
+    const float* pair_logits, const float* mask_q, const float* mask_k, int64_t bias_batches,
+    const uint16_t* w_qg, const uint16_t* w_kv, const float* query_b, int num_head,
+    void* out, int out_dtype, int64_t batch, int64_t sq, int64_t sk, int channels,
+    void* workspace, size_t workspace_bytes, af3_stream_t stream) {
+  if (!q_data || !m_data || !w_qg || !w_kv || !out) return AF3_ERR_BAD_ARG;
+  if (bad_dtype(out_dtype) || batch <= 0 || sq <= 0 || sk <= 0 || channels <= 0 || (channels & 7) ||
+      num_head <= 0 || channels % num_head)
+    return AF3_ERR_BAD_ARG;
+  if ((mask_q == nullptr) != (mask_k == nullptr)) return AF3_ERR_BAD_ARG;
+  if ((pair_logits || mask_q) && (bias_batches <= 0 || batch % bias_batches)) return AF3_ERR_BAD_ARG;
+  if (batch * sq > 0x7fffffff || batch * sk > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  const int d = channels / num_head;
+  if (d != 24 && d != 32 && d != 48) return AF3_ERR_UNSUPPORTED;
+  Carver ws(workspace, workspace_bytes);
+  bf16_t* qg = ws.take<bf16_t>((size_t)batch * sq * 2 * channels);
+  bf16_t* kv = ws.take<bf16_t>((size_t)batch * sk * 2 * channels);
+  if (!ws.ok) return AF3_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+
+  GemmArgs g;
+  g.A = q_data; g.B = w_qg; g.C = qg;
+  g.M = (int)(batch * sq); g.N = 2 * channels; g.K = channels;
+  g.lda = channels; g.ldb = channels; g.ldc = 2 * channels;
+  g.epi = EPI_SEGMENTED; g.seg_len = channels;
+  g.seg_ops = SEG_BIAS_SCALE | (SEG_SIGMOID << 4);
+  g.alpha = 1.0f / sqrtf((float)d);
+  g.bias = query_b;
+  int rc = launch_gemm_nt(g, s);
+  if (rc) return rc;
+  GemmArgs g2;
+  g2.A = m_data; g2.B = w_kv; g2.C = kv;
+  g2.M = (int)(batch * sk); g2.N = 2 * channels; g2.K = channels;
+  g2.lda = channels; g2.ldb = channels; g2.ldc = 2 * channels;
+  rc = launch_gemm_nt(g2, s);
+  if (rc) return rc;
+
+  FlashArgs f;
+  f.q = qg; f.g = qg + channels; f.k = kv; f.v = kv + channels;
+  f.q_ss = f.g_ss = f.k_ss = f.v_ss = 2 * channels;
+  f.q_sb = f.g_sb = sq * 2 * channels;
+  f.k_sb = f.v_sb = sk * 2 * channels;
+  f.out = out; f.out_f32 = out_dtype == AF3_F32; f.o_ss = channels; f.o_sb = sq * channels;
+  f.B = (int)batch; f.H = num_head; f.Sq = (int)sq; f.Sk = (int)sk; f.d = d;
+  f.bias = pair_logits; f.bias_sb = (int64_t)num_head * sq * sk; f.bias_sh = sq * sk; f.bias_sq = sk;
+  f.qpad = mask_q; f.kpad = mask_k; f.qp_sb = sq; f.kp_sb = sk;
+  f.bias_mod = (pair_logits || mask_q) ? (int)bias_batches : 0;
+  return launch_flash_attention(f, s);
+}
+
+// ------------------------------------------------------------------ pair logits
+int af3_pair_logits_forward(
+    const void* pair, int io_dtype, const float* norm_weight, const float* norm_bias,
+    const uint16_t* w, int n_out, float* out, int64_t n, af3_stream_t stream) {
+  if (!pair || !w || !out || !norm_weight) return AF3_ERR_BAD_ARG;
+  if (bad_dtype(io_dtype) || n <= 0 || n > 8192 || n_out <= 0) return AF3_ERR_BAD_ARG;
+  AttnProjArgs p;
+  p.pair = pair; p.io_f32 = io_dtype == AF3_F32; p.N = (int)n;
+  p.ln_w = norm_weight; p.ln_b = norm_bias;
+  p.w_bias = w; p.n_bias = n_out; p.out_bias = out;
+  return launch_attn_proj(p, static_cast<hipStream_t>(stream));
+}
+
+// ------------------------------------------------------------------- row norm
+int af3_layer_norm_forward(
+    const void* x, int x_dtype, uint16_t* y, int64_t rows, int channels,
+    const float* weight, const float* bias, const float* scale, const float* shift,
+    int64_t cond_rows, int64_t cond_ld, af3_stream_t stream) {
+  if (!x || !y || bad_dtype(x_dtype)) return AF3_ERR_BAD_ARG;
+  RowNormArgs a;
+  a.x = x; a.x_f32 = x_dtype == AF3_F32; a.y = y; a.rows = rows; a.ldx = a.ldy = channels; a.C = channels;
+  a.weight = weight; a.bias = bias; a.scale = scale; a.shift = shift;
+  a.cond_rows = cond_rows; a.ld_cond = cond_ld;
+  return launch_row_norm(a, static_cast<hipStream_t>(stream));
+}
+
+// --------------------------------------------------------------------- linear
+int af3_linear_forward(
+    const uint16_t* x, const uint16_t* w, const float* bias, void* y, int y_dtype,
+    int64_t m, int n, int k, int mode, float alpha, int sigmoid,
+    const float* gate, int64_t gate_rows, const void* residual, int res_dtype, af3_stream_t stream) {
+  if (!x || !w || !y || bad_dtype(y_dtype) || m <= 0 || m > 0x7fffffff || n <= 0 || k <= 0) return AF3_ERR_BAD_ARG;
+  if (mode != AF3_LINEAR_PLAIN && mode != AF3_LINEAR_SWIGLU && mode != AF3_LINEAR_GATE_RES) return AF3_ERR_BAD_ARG;
+  if (residual && bad_dtype(res_dtype)) return AF3_ERR_BAD_ARG;
+  GemmArgs g;
+  g.A = x; g.B = w; g.C = y;
+  g.M = (int)m; g.N = n; g.K = k;
+  g.lda = k; g.ldb = k;
+  g.ldc = mode == AF3_LINEAR_SWIGLU ? n / 2 : n;
+  g.out_f32 = y_dtype == AF3_F32;
+  g.epi = mode; g.alpha = alpha; g.bias = bias; g.act_sigmoid = sigmoid;
+  g.gate = gate; g.gate_rows = (int)gate_rows; g.ld_gate = n;
+  if (residual) {
+    if (res_dtype == AF3_F32) g.res_f32 = static_cast<const float*>(residual);
+    else g.res_bf16 = static_cast<const bf16_t*>(residual);
+    g.ld_res = n;
+  }
+  return launch_gemm_nt(g, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,127 @@
+// Shared device helpers for the gfx950 (CDNA4) kernels: bf16 conversion, MFMA
+// fragment conventions, wave reductions and LDS tile geometry.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define AF3_OK 0
+#define AF3_ERR_BAD_ARG (-1)
+#define AF3_ERR_WORKSPACE (-2)
+#define AF3_ERR_LAUNCH (-3)
+#define AF3_ERR_UNSUPPORTED (-4)
+
+typedef uint16_t bf16_t;  // raw bf16 bits in memory
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+#define WAVE 64
+
+// ----------------------------------------------------------------------------
+// bf16 <-> fp32 (round to nearest even; NaN kept quiet)
+// ----------------------------------------------------------------------------
+__device__ __forceinline__ float bf2f(bf16_t h) {
+  return __uint_as_float(((uint32_t)h) << 16);
+}
+__device__ __forceinline__ bf16_t f2bf(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+__device__ __forceinline__ uint32_t pack2bf(float lo, float hi) {
+  return (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
+}
+__device__ __forceinline__ float bflo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bfhi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// 8 consecutive bf16 (16 bytes) <-> 8 floats
+__device__ __forceinline__ void unpack8(const u32x4 v, float* f) {
+  f[0] = bflo(v.x); f[1] = bfhi(v.x); f[2] = bflo(v.y); f[3] = bfhi(v.y);
+  f[4] = bflo(v.z); f[5] = bfhi(v.z); f[6] = bflo(v.w); f[7] = bfhi(v.w);
+}
+__device__ __forceinline__ u32x4 pack8(const float* f) {
+  u32x4 v;
+  v.x = pack2bf(f[0], f[1]); v.y = pack2bf(f[2], f[3]);
+  v.z = pack2bf(f[4], f[5]); v.w = pack2bf(f[6], f[7]);
+  return v;
+}
+
+// Load / store 8 consecutive channels of the residual stream, which may be
+// held as bf16 or fp32.
+template <typename T> struct Elem;
+template <> struct Elem<bf16_t> {
+  static __device__ __forceinline__ void load8(const bf16_t* p, float* f) {
+    unpack8(*reinterpret_cast<const u32x4*>(p), f);
+  }
+  static __device__ __forceinline__ void store8(bf16_t* p, const float* f) {
+    *reinterpret_cast<u32x4*>(p) = pack8(f);
+  }
+  static __device__ __forceinline__ float load(const bf16_t* p) { return bf2f(*p); }
+  static __device__ __forceinline__ void store(bf16_t* p, float v) { *p = f2bf(v); }
+};
+template <> struct Elem<float> {
+  static __device__ __forceinline__ void load8(const float* p, float* f) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p);
+    const f32x4 b = *reinterpret_cast<const f32x4*>(p + 4);
+    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w;
+    f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+  }
+  static __device__ __forceinline__ void store8(float* p, const float* f) {
+    f32x4 a = {f[0], f[1], f[2], f[3]}, b = {f[4], f[5], f[6], f[7]};
+    *reinterpret_cast<f32x4*>(p) = a;
+    *reinterpret_cast<f32x4*>(p + 4) = b;
+  }
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+};
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+// ----------------------------------------------------------------------------
+// MFMA 32x32x16 bf16 (D = A[32xK16] * B[K16x32] + C), wave64.
+//   A fragment: lane l holds A[row = l & 31][k = 8*(l >> 5) .. +7]
+//   B fragment: lane l holds B[k = 8*(l >> 5) .. +7][col = l & 31]
+//   C/D       : lane l, register r holds D[row = 8*(r >> 2) + 4*(l >> 5) + (r & 3)][col = l & 31]
+// Both fragments are "8 consecutive k of one row/col", so an operand stored
+// k-contiguous ([row][k]) is read with one 16-byte load per fragment.
+// ----------------------------------------------------------------------------
+__device__ __forceinline__ f32x16 mfma32(const bf16x8 a, const bf16x8 b, const f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ bf16x8 as_frag(const u32x4 v) {
+  return __builtin_bit_cast(bf16x8, v);
+}
+__device__ __forceinline__ int acc_row(int r, int lane) {
+  return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+}
+
+// 16-byte fragment read from an LDS tile stored [row][ld] (bf16, k-contiguous)
+__device__ __forceinline__ bf16x8 lds_frag(const bf16_t* tile, int ld, int row0, int k0, int lane) {
+  const bf16_t* p = tile + (row0 + (lane & 31)) * ld + k0 + 8 * (lane >> 5);
+  return as_frag(*reinterpret_cast<const u32x4*>(p));
+}
+
+// ----------------------------------------------------------------------------
+// reductions over groups of 16 / 64 lanes
+// ----------------------------------------------------------------------------
+__device__ __forceinline__ float group16_sum(float v) {
+  v += __shfl_xor(v, 1); v += __shfl_xor(v, 2);
+  v += __shfl_xor(v, 4); v += __shfl_xor(v, 8);
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  v = group16_sum(v);
+  v += __shfl_xor(v, 16); v += __shfl_xor(v, 32);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+  for (int m = 1; m < 64; m <<= 1) v = fmaxf(v, __shfl_xor(v, m));
+  return v;
+}
+
+#define LN_EPS 1e-5f

@@ -1,0 +1,118 @@
+// Host-side launch interface of the kernels (internal; the public C ABI is in
+// include/af3_hip.h and implemented in api.hip).
+#pragma once
+#include "common.h"
+
+// ------------------------------------------------------------------ gemm.hip
+enum { EPI_PLAIN = 0, EPI_SEGMENTED = 1, EPI_SWIGLU = 2, EPI_GATE_RES = 3 };
+enum { SEG_PLAIN = 0, SEG_BIAS_SCALE = 1, SEG_SIGMOID = 2 };
+
+struct GemmArgs {
+  const bf16_t* A = nullptr;  // [batch][M][lda]
+  const bf16_t* B = nullptr;  // [batch][N][ldb]   (C = A * B^T)
+  void* C = nullptr;          // [batch][M][ldc]   bf16 or fp32
+  int M = 0, N = 0, K = 0, batch = 1;
+  int64_t lda = 0, ldb = 0, ldc = 0, sA = 0, sB = 0, sC = 0;
+  int out_f32 = 0;
+  int epi = EPI_PLAIN;
+  float alpha = 1.f;            // PLAIN: (acc + bias) * alpha ; SEG_BIAS_SCALE likewise
+  const float* bias = nullptr;  // [N]
+  int act_sigmoid = 0;          // PLAIN only
+  int seg_len = 0, seg_ops = 0; // SEGMENTED: op of column segment s in bits [4s, 4s+4)
+  const float* gate = nullptr;  // GATE_RES: multiply by gate[m % gate_rows][n]
+  int gate_rows = 0;
+  int64_t ld_gate = 0;
+  const float* res_f32 = nullptr;   // GATE_RES: residual added last (either dtype)
+  const bf16_t* res_bf16 = nullptr;
+  int64_t ld_res = 0, sRes = 0;
+};
+int launch_gemm_nt(const GemmArgs& g, hipStream_t stream);
+
+// ---------------------------------------------------------------- rowops.hip
+// y = LN(x) [* weight + bias] ; then, if scale: y = sigmoid(scale[r]) * y + shift[r]
+// with r = row % cond_rows (conditioning shared by the sample batch).
+struct RowNormArgs {
+  const void* x = nullptr;  // [rows][ldx] bf16 or fp32
+  int x_f32 = 0;
+  bf16_t* y = nullptr;      // [rows][ldy]
+  int64_t rows = 0, ldx = 0, ldy = 0;
+  int C = 0;
+  const float* weight = nullptr;  // [C] or null
+  const float* bias = nullptr;    // [C] or null
+  const float* scale = nullptr;   // [cond_rows][ld_cond] pre-sigmoid, or null
+  const float* shift = nullptr;
+  int64_t cond_rows = 0, ld_cond = 0;
+};
+int launch_row_norm(const RowNormArgs& a, hipStream_t stream);
+
+// -------------------------------------------------------------- pair_tile.hip
+// Residual-stream tensors (`pair`, `out`, `x`) are bf16 or fp32 (io_f32).
+struct TriMulArgs {
+  const void* pair = nullptr;   // [N][N][128]
+  const float* mask = nullptr;  // [N][N] 0/1 or null
+  void* out = nullptr;          // [N][N][128]; may alias pair when residual
+  int io_f32 = 0, N = 0, Np = 0, outgoing = 1, residual = 0;
+  const float *ln_in_w = nullptr, *ln_in_b = nullptr, *ln_c_w = nullptr, *ln_c_b = nullptr;
+  const bf16_t* w_pg = nullptr;   // [4][128][128]: per chunk 64 projection rows + 64 gate rows
+  const bf16_t* w_gl = nullptr;   // [128][128] gating_linear
+  const bf16_t* w_out = nullptr;  // [128][128] output_projection
+  bf16_t *a_buf = nullptr, *b_buf = nullptr;  // [128][N][Np] channel-major operands
+  const bf16_t* t_buf = nullptr;              // [128][N][Np] contraction result
+};
+int launch_trimul_prologue(const TriMulArgs& a, hipStream_t s);
+int launch_trimul_epilogue(const TriMulArgs& a, hipStream_t s);
+
+struct AttnProjArgs {
+  const void* pair = nullptr;  // [N][N][128]
+  int io_f32 = 0, N = 0, transpose = 0;
+  int skip_ln = 0;  // pair is already normalised
+  const float *ln_w = nullptr, *ln_b = nullptr;
+  const bf16_t* w_main = nullptr;  // [n_chunks][128][128]
+  int n_chunks = 0, chunk_ops = 0; // SEG_* per chunk, 4 bits each
+  float q_scale = 1.f;
+  bf16_t* out_main = nullptr;      // [(b*N + s)][ld_main], chunk c at columns 128c..
+  int64_t ld_main = 0;
+  const bf16_t* w_bias = nullptr;  // [roundup(n_bias, 32)][128]
+  int n_bias = 0;
+  float* out_bias = nullptr;       // [n_bias][N][N]
+};
+int launch_attn_proj(const AttnProjArgs& a, hipStream_t s);
+
+struct AttnOutArgs {
+  const bf16_t* og = nullptr;  // [(b*N + s)][ld_og] gated attention output
+  int64_t ld_og = 0;
+  const bf16_t* w_out = nullptr;  // [128][128]
+  const void* pair = nullptr;     // residual source
+  void* out = nullptr;
+  int io_f32 = 0, N = 0, transpose = 0, residual = 0;
+};
+int launch_attn_out(const AttnOutArgs& a, hipStream_t s);
+
+struct TransitionArgs {
+  const void* x = nullptr;  // [N][128]
+  void* out = nullptr;
+  int io_f32 = 0, N = 0, hidden = 0, residual = 0;
+  const float *ln_w = nullptr, *ln_b = nullptr;
+  const bf16_t* w1 = nullptr;  // [hidden/64][128][128]: 64 a rows then 64 b rows per slab
+  const bf16_t* w2 = nullptr;  // [128][hidden]
+};
+int launch_transition(const TransitionArgs& a, hipStream_t s);
+
+// -------------------------------------------------------------- attention.hip
+// q/k/v/g/out are addressed as base + batch * sb + position * ss + head * d.
+struct FlashArgs {
+  const bf16_t *q = nullptr, *k = nullptr, *v = nullptr, *g = nullptr;  // g: output gate or null
+  int64_t q_sb = 0, q_ss = 0, k_sb = 0, k_ss = 0, v_sb = 0, v_ss = 0, g_sb = 0, g_ss = 0;
+  void* out = nullptr;
+  int out_f32 = 0;
+  int64_t o_sb = 0, o_ss = 0;
+  int B = 0, H = 0, Sq = 0, Sk = 0, d = 0;
+  const float* bias = nullptr;  // [.][H][Sq][Sk], key stride 1
+  int64_t bias_sb = 0, bias_sh = 0, bias_sq = 0;
+  const float* key_mask = nullptr;  // [B][Sk] (km_sb may be 0): 0 -> logit replaced by -1e9
+  int64_t km_sb = 0;
+  const float *qpad = nullptr, *kpad = nullptr;  // [B][Sq], [B][Sk]: +1e9 where both are 0
+  int64_t qp_sb = 0, kp_sb = 0;
+  int bias_mod = 0;  // > 0: bias, qpad and kpad are indexed by batch % bias_mod
+};
+int launch_flash_attention(const FlashArgs& a, hipStream_t stream);

@@ -1,0 +1,543 @@
+// Row-tile kernels of the 128-channel pair path.
+//
+// Every kernel here walks the [N, N, 128] pair tensor in tiles of 128
+// consecutive positions along one axis (a row segment, or a column segment for
+// the transposed operators), keeps the tile's LayerNorm-ed activations in LDS /
+// registers as bf16 MFMA fragments and multiplies them with 128x128 weight
+// chunks streamed through LDS.  They are HBM-bound (one read of the pair tensor,
+// one write of each product) except the SwiGLU transition, which is MFMA-bound.
+//
+//   trimul_prologue  LN -> [proj|gate] -> mask * sigmoid -> a, b channel-major
+//   trimul_epilogue  channel-major contraction result -> LN -> out-proj ->
+//                    * sigmoid(LN(x) Wgl^T) -> (+ residual)
+//   attn_proj        LN -> q (scaled), k, v, sigmoid gate, + pair-bias heads
+//   attn_out         gated attention output -> out-proj -> (+ residual)
+//   transition       LN -> W1 -> silu(a) * b -> W2 -> (+ residual), hidden in registers
+//
+// MFMA orientation: "D form" computes out[px][ch] with the pixel fragments as
+// the A operand (a lane then owns one channel and 16 pixels), "T form" computes
+// out^T[ch][px] with the weight rows as A (a lane owns one pixel and groups of
+// 4 consecutive channels).  D form feeds channel-major stores, T form feeds
+// pixel-major stores; the fragments are the same registers in both.
+#include "common.h"
+#include "kernels.h"
+
+namespace {
+
+constexpr int C = 128;    // pair channels
+constexpr int TM = 128;   // positions per tile
+constexpr int LDX = 136;  // LDS row stride (bf16) for [row][128] tiles: 272 B
+constexpr int LDS_F = 132;  // LDS row stride (fp32) for staged output tiles
+
+struct Tile {
+  int o, r0, N;
+  int64_t so, sr;  // pixel index = o * so + r * sr
+  __device__ __forceinline__ int64_t pix(int p) const { return (int64_t)o * so + (int64_t)(r0 + p) * sr; }
+  __device__ __forceinline__ bool valid(int p) const { return r0 + p < N; }
+};
+
+__device__ __forceinline__ Tile make_tile(int N, bool column_mode) {
+  const int tiles_r = (N + TM - 1) / TM;
+  Tile t;
+  t.N = N;
+  t.o = blockIdx.x / tiles_r;
+  t.r0 = (blockIdx.x % tiles_r) * TM;
+  t.so = column_mode ? 1 : N;
+  t.sr = column_mode ? N : 1;
+  return t;
+}
+
+// LayerNorm of a tile of pixels from global memory into sX[p][c] (bf16).
+// Thread (prow = tid / 16, chunk = tid % 16) handles channels 8*chunk..+7 of
+// pixels prow, prow + 16, ...; 16 lanes cooperate on one pixel's statistics.
+// Out-of-range pixels become zero rows.
+template <typename TIO>
+__device__ __forceinline__ void load_ln_tile(const TIO* x, const Tile& t, const float* lnw,
+                                             const float* lnb, bf16_t* sX, int tid, bool skip_ln = false) {
+  const int chunk = tid & 15, prow = tid >> 4;
+  float w[8], b[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    w[e] = lnw ? lnw[chunk * 8 + e] : 1.f;
+    b[e] = lnb ? lnb[chunk * 8 + e] : 0.f;
+  }
+  float v[8][8];
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int p = it * 16 + prow;
+    if (t.valid(p)) {
+      Elem<TIO>::load8(x + t.pix(p) * C + chunk * 8, v[it]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[it][e] = 0.f;
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int p = it * 16 + prow;
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += v[it][e];
+    const float mean = group16_sum(s) * (1.f / C);
+    float q = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { const float d = v[it][e] - mean; q += d * d; }
+    const float rstd = rsqrtf(group16_sum(q) * (1.f / C) + LN_EPS);
+    float o[8];
+    const bool ok = t.valid(p);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = ok ? (skip_ln ? v[it][e] : (v[it][e] - mean) * rstd * w[e] + b[e]) : 0.f;
+    *reinterpret_cast<u32x4*>(sX + p * LDX + chunk * 8) = pack8(o);
+  }
+}
+
+// In-place LayerNorm of the rows of sX (bf16 in LDS), same thread mapping.
+__device__ __forceinline__ void ln_inplace_tile(bf16_t* sX, const float* lnw, const float* lnb, int tid) {
+  const int chunk = tid & 15, prow = tid >> 4;
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int p = it * 16 + prow;
+    float v[8];
+    unpack8(*reinterpret_cast<const u32x4*>(sX + p * LDX + chunk * 8), v);
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += v[e];
+    const float mean = group16_sum(s) * (1.f / C);
+    float q = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { const float d = v[e] - mean; q += d * d; }
+    const float rstd = rsqrtf(group16_sum(q) * (1.f / C) + LN_EPS);
+    float o[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (v[e] - mean) * rstd * lnw[chunk * 8 + e] + lnb[chunk * 8 + e];
+    *reinterpret_cast<u32x4*>(sX + p * LDX + chunk * 8) = pack8(o);
+  }
+}
+
+// Copy `rows` x 128 bf16 weights (row-major, contiguous) into sW[row][LDX].
+__device__ __forceinline__ void load_w_rows(const bf16_t* gW, bf16_t* sW, int rows, int tid) {
+  for (int idx = tid; idx < rows * 16; idx += 256) {
+    const int row = idx >> 4, ch = idx & 15;
+    *reinterpret_cast<u32x4*>(sW + row * LDX + ch * 8) =
+        *reinterpret_cast<const u32x4*>(gW + row * C + ch * 8);
+  }
+}
+
+// The wave's 32 pixels as 8 k-step fragments (k = 128 channels).
+__device__ __forceinline__ void load_x_frags(const bf16_t* sX, int wave, int lane, bf16x8* xf) {
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) xf[ks] = lds_frag(sX, LDX, wave * 32, ks * 16, lane);
+}
+
+// acc[nt] = tile nt (32 weight rows) of  X * W^T  (D form) or  W * X^T  (T form)
+template <bool TFORM, int NT>
+__device__ __forceinline__ void mfma_chunk(const bf16x8* xf, const bf16_t* sW, int lane, f32x16* acc) {
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[nt][r] = 0.f;
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const bf16x8 wf = lds_frag(sW, LDX, nt * 32, ks * 16, lane);
+      acc[nt] = TFORM ? mfma32(wf, xf[ks], acc[nt]) : mfma32(xf[ks], wf, acc[nt]);
+    }
+}
+
+// T-form accumulators (lane = pixel, 4 consecutive channels per register
+// quad) -> fp32 staging tile sS[px][LDS_F].
+__device__ __forceinline__ void stage_t_f32(const f32x16* acc, float* sS, int wave, int lane) {
+  const int px = wave * 32 + (lane & 31);
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int ch = nt * 32 + 8 * g + 4 * (lane >> 5);
+      f32x4 v = {acc[nt][4 * g], acc[nt][4 * g + 1], acc[nt][4 * g + 2], acc[nt][4 * g + 3]};
+      *reinterpret_cast<f32x4*>(sS + px * LDS_F + ch) = v;
+    }
+}
+
+// T-form accumulators -> bf16 staging tile sS[px][LDX]
+__device__ __forceinline__ void stage_t_bf16(const f32x16* acc, bf16_t* sS, int wave, int lane) {
+  const int px = wave * 32 + (lane & 31);
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int ch = nt * 32 + 8 * g + 4 * (lane >> 5);
+      u32x2 v;
+      v.x = pack2bf(acc[nt][4 * g], acc[nt][4 * g + 1]);
+      v.y = pack2bf(acc[nt][4 * g + 2], acc[nt][4 * g + 3]);
+      *reinterpret_cast<u32x2*>(sS + px * LDX + ch) = v;
+    }
+}
+
+// Staged fp32 tile -> residual stream: out[pix] = (res ? res[pix] : 0) + tile
+template <typename TIO>
+__device__ __forceinline__ void store_tile_f32(const float* sS, const Tile& t, TIO* out, const TIO* res, int tid) {
+  const int chunk = tid & 15, prow = tid >> 4;
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int p = it * 16 + prow;
+    if (!t.valid(p)) continue;
+    float v[8];
+    const f32x4 a = *reinterpret_cast<const f32x4*>(sS + p * LDS_F + chunk * 8);
+    const f32x4 b = *reinterpret_cast<const f32x4*>(sS + p * LDS_F + chunk * 8 + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    const int64_t off = t.pix(p) * C + chunk * 8;
+    if (res) {
+      float rr[8];
+      Elem<TIO>::load8(res + off, rr);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] += rr[e];
+    }
+    Elem<TIO>::store8(out + off, v);
+  }
+}
+
+// ============================================================================
+// triangle multiplication, prologue
+// ============================================================================
+template <typename TIO>
+__global__ __launch_bounds__(256) void trimul_prologue_kernel(TriMulArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t sX[TM * LDX];
+  __shared__ __attribute__((aligned(16))) bf16_t sW[TM * LDX];
+  __shared__ float sMask[TM];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // outgoing: tiles run along k for fixed i (a[c][i][k]); incoming: along k for
+  // fixed j, i.e. a column segment of the pair tensor (a'[c][j][k] = a[k][j][c]).
+  const Tile t = make_tile(a.N, !a.outgoing);
+  const TIO* x = reinterpret_cast<const TIO*>(a.pair);
+
+  if (tid < TM) sMask[tid] = (t.valid(tid) ? (a.mask ? a.mask[t.pix(tid)] : 1.f) : 0.f);
+  load_ln_tile<TIO>(x, t, a.ln_in_w, a.ln_in_b, sX, tid);
+  __syncthreads();
+  bf16x8 xf[8];
+  load_x_frags(sX, wave, lane, xf);
+
+  // weight chunks: [P(64 ch) | G(64 ch)] for a ch 0-63, a ch 64-127, b ch 0-63, b ch 64-127
+  for (int chunk = 0; chunk < 4; ++chunk) {
+    load_w_rows(a.w_pg + (int64_t)chunk * TM * C, sW, TM, tid);
+    __syncthreads();
+    f32x16 acc[4];
+    mfma_chunk<false, 4>(xf, sW, lane, acc);
+    __syncthreads();  // sW is free: reuse it as the [64 ch][LDX px] staging tile
+    // D form: lane owns channel (lane & 31) of tiles 0/1 (P) and 2/3 (G)
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int ch = nt * 32 + (lane & 31);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int p0 = wave * 32 + 8 * g + 4 * (lane >> 5);
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          v[e] = acc[nt][4 * g + e] * sMask[p0 + e] * sigmoidf_(acc[nt + 2][4 * g + e]);
+        u32x2 pk;
+        pk.x = pack2bf(v[0], v[1]);
+        pk.y = pack2bf(v[2], v[3]);
+        *reinterpret_cast<u32x2*>(sW + ch * LDX + p0) = pk;
+      }
+    }
+    __syncthreads();
+    bf16_t* dst = (chunk < 2 ? a.a_buf : a.b_buf) + ((int64_t)(chunk & 1) * 64 * a.N + t.o) * a.Np;
+    for (int idx = tid; idx < 64 * 16; idx += 256) {
+      const int ch = idx >> 4, pc = idx & 15;
+      const int r = t.r0 + pc * 8;
+      if (r < a.Np)
+        *reinterpret_cast<u32x4*>(dst + (int64_t)ch * a.N * a.Np + r) =
+            *reinterpret_cast<const u32x4*>(sW + ch * LDX + pc * 8);
+    }
+    __syncthreads();
+  }
+}
+
+// ============================================================================
+// triangle multiplication, epilogue
+// ============================================================================
+template <typename TIO>
+__global__ __launch_bounds__(256) void trimul_epilogue_kernel(TriMulArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t smem[2 * TM * LDX];
+  bf16_t* sX = smem;
+  bf16_t* sW = smem + TM * LDX;
+  float* sS = reinterpret_cast<float*>(smem);  // [TM][LDS_F] fp32 over both, after the last MFMA
+  static_assert(TM * LDS_F * 4 <= 2 * TM * LDX * 2, "staging tile must fit");
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const Tile t = make_tile(a.N, false);
+  const TIO* x = reinterpret_cast<const TIO*>(a.pair);
+
+  // 1. output gate from the LayerNorm-ed input: sigmoid(LN(x) Wgl^T), T form, kept in registers
+  load_ln_tile<TIO>(x, t, a.ln_in_w, a.ln_in_b, sX, tid);
+  load_w_rows(a.w_gl, sW, TM, tid);
+  __syncthreads();
+  bf16x8 xf[8];
+  load_x_frags(sX, wave, lane, xf);
+  f32x16 gate[4];
+  mfma_chunk<true, 4>(xf, sW, lane, gate);
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) gate[nt][r] = sigmoidf_(gate[nt][r]);
+  __syncthreads();
+
+  // 2. contraction result t[c][i][j0..] -> sX[j][c], then center LayerNorm
+  {
+    const int pc = tid & 15, crow = tid >> 4;
+    const int nvalid = min(max(a.N - (t.r0 + pc * 8), 0), 8);
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int c = it * 16 + crow;
+      u32x4 raw = {0, 0, 0, 0};
+      if (nvalid > 0)
+        raw = *reinterpret_cast<const u32x4*>(a.t_buf + ((int64_t)c * a.N + t.o) * a.Np + t.r0 + pc * 8);
+      const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        bf16_t h = (bf16_t)((e & 1) ? (w4[e >> 1] >> 16) : (w4[e >> 1] & 0xffffu));
+        if (e >= nvalid) h = 0;
+        sX[(pc * 8 + e) * LDX + c] = h;
+      }
+    }
+  }
+  load_w_rows(a.w_out, sW, TM, tid);
+  __syncthreads();
+  ln_inplace_tile(sX, a.ln_c_w, a.ln_c_b, tid);
+  __syncthreads();
+  load_x_frags(sX, wave, lane, xf);
+  f32x16 acc[4];
+  mfma_chunk<true, 4>(xf, sW, lane, acc);
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[nt][r] *= gate[nt][r];
+  __syncthreads();
+  stage_t_f32(acc, sS, wave, lane);
+  __syncthreads();
+  store_tile_f32<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), a.residual ? x : nullptr, tid);
+}
+
+// ============================================================================
+// triangle attention: projections
+// ============================================================================
+template <typename TIO>
+__global__ __launch_bounds__(256) void attn_proj_kernel(AttnProjArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t sX[TM * LDX];
+  __shared__ __attribute__((aligned(16))) bf16_t sW[TM * LDX];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // (b, s) = (o, r): for the transposed operator a tile is a column segment
+  const Tile t = make_tile(a.N, a.transpose != 0);
+  const TIO* x = reinterpret_cast<const TIO*>(a.pair);
+  load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0);
+  __syncthreads();
+  bf16x8 xf[8];
+  load_x_frags(sX, wave, lane, xf);
+
+  for (int chunk = 0; chunk < a.n_chunks; ++chunk) {
+    load_w_rows(a.w_main + (int64_t)chunk * TM * C, sW, TM, tid);
+    __syncthreads();
+    f32x16 acc[4];
+    mfma_chunk<true, 4>(xf, sW, lane, acc);
+    const int op = (a.chunk_ops >> (4 * chunk)) & 15;
+    if (op == SEG_BIAS_SCALE) {
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[nt][r] *= a.q_scale;
+    } else if (op == SEG_SIGMOID) {
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[nt][r] = sigmoidf_(acc[nt][r]);
+    }
+    __syncthreads();
+    stage_t_bf16(acc, sW, wave, lane);
+    __syncthreads();
+    const int ck = tid & 15, prow = tid >> 4;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int p = it * 16 + prow;
+      if (t.valid(p))
+        *reinterpret_cast<u32x4*>(a.out_main + ((int64_t)t.o * a.N + t.r0 + p) * a.ld_main + chunk * C + ck * 8) =
+            *reinterpret_cast<const u32x4*>(sW + p * LDX + ck * 8);
+    }
+    __syncthreads();
+  }
+
+  // pair-bias heads: out_bias[h][q][k] with (q, k) the pixel's own (row, col)
+  for (int h0 = 0; h0 < a.n_bias; h0 += 32) {
+    load_w_rows(a.w_bias + (int64_t)h0 * C, sW, 32, tid);  // host pads w_bias to a multiple of 32 rows
+    __syncthreads();
+    f32x16 acc[1];
+    mfma_chunk<true, 1>(xf, sW, lane, acc);
+    const int p = wave * 32 + (lane & 31);
+    if (t.valid(p)) {
+      const int64_t pixel = t.pix(p);  // = q * N + k
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int h = h0 + acc_row(r, lane);
+        if (h < a.n_bias) a.out_bias[(int64_t)h * a.N * a.N + pixel] = acc[0][r];
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// ============================================================================
+// triangle attention: output projection
+// ============================================================================
+template <typename TIO>
+__global__ __launch_bounds__(256) void attn_out_kernel(AttnOutArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t smem[2 * TM * LDX];
+  bf16_t* sX = smem;
+  bf16_t* sW = smem + TM * LDX;
+  float* sS = reinterpret_cast<float*>(smem);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const Tile t = make_tile(a.N, a.transpose != 0);  // where the result lands in the pair tensor
+  {
+    const int ck = tid & 15, prow = tid >> 4;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int p = it * 16 + prow;
+      u32x4 v = {0, 0, 0, 0};
+      if (t.valid(p))
+        v = *reinterpret_cast<const u32x4*>(a.og + ((int64_t)t.o * a.N + t.r0 + p) * a.ld_og + ck * 8);
+      *reinterpret_cast<u32x4*>(sX + p * LDX + ck * 8) = v;
+    }
+  }
+  load_w_rows(a.w_out, sW, TM, tid);
+  __syncthreads();
+  bf16x8 xf[8];
+  load_x_frags(sX, wave, lane, xf);
+  f32x16 acc[4];
+  mfma_chunk<true, 4>(xf, sW, lane, acc);
+  __syncthreads();
+  stage_t_f32(acc, sS, wave, lane);
+  __syncthreads();
+  store_tile_f32<TIO>(sS, t, reinterpret_cast<TIO*>(a.out),
+                      a.residual ? reinterpret_cast<const TIO*>(a.pair) : nullptr, tid);
+}
+
+// ============================================================================
+// SwiGLU transition, c = 128, hidden = 128 * factor, all in one kernel
+// ============================================================================
+constexpr int LDW2 = 72;  // LDS row stride (bf16) of a [128 out][64 hidden] W2 slab
+
+template <typename TIO>
+__global__ __launch_bounds__(256) void transition_kernel(TransitionArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t smem[2 * TM * LDX];
+  bf16_t* sX = smem;              // phase 0: LN tile;   later: W1 slab [128][LDX]
+  bf16_t* sW1 = smem;
+  bf16_t* sW2 = smem + TM * LDX;  // W2 slab [128][LDW2]
+  float* sS = reinterpret_cast<float*>(smem);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const Tile t = make_tile(a.N, false);
+  const TIO* x = reinterpret_cast<const TIO*>(a.x);
+  load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid);
+  __syncthreads();
+  bf16x8 xf[8];
+  load_x_frags(sX, wave, lane, xf);
+  __syncthreads();
+
+  f32x16 out[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) out[nt][r] = 0.f;
+
+  const int n_slabs = a.hidden / 64;
+  for (int hs = 0; hs < n_slabs; ++hs) {
+    // W1 slab: 64 "a" rows then the 64 matching "b" rows (host-packed), K = 128
+    load_w_rows(a.w1 + (int64_t)hs * 128 * C, sW1, 128, tid);
+    // W2 slab: all 128 output rows, hidden columns 64*hs .. +63
+    for (int idx = tid; idx < 128 * 8; idx += 256) {
+      const int row = idx >> 3, ck = idx & 7;
+      *reinterpret_cast<u32x4*>(sW2 + row * LDW2 + ck * 8) =
+          *reinterpret_cast<const u32x4*>(a.w2 + (int64_t)row * a.hidden + hs * 64 + ck * 8);
+    }
+    __syncthreads();
+    // GEMM1, T form: acc[0..1] = a^T (64 hidden x 32 px), acc[2..3] = b^T
+    f32x16 acc[4];
+    mfma_chunk<true, 4>(xf, sW1, lane, acc);
+    // h^T = silu(a) * b; registers 8s..8s+7 of tile nt are, as they stand, the
+    // B fragment of k-step s of GEMM2 provided W2's k index is permuted alike:
+    // element e of lane-half hh is hidden unit 32*nt + 16*s + 8*(e >> 2) + 4*hh + (e & 3).
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        float hv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float av = acc[nt][8 * s + e], bv = acc[nt + 2][8 * s + e];
+          hv[e] = av * sigmoidf_(av) * bv;
+        }
+        const bf16x8 hf = as_frag(pack8(hv));
+        const int kbase = 32 * nt + 16 * s + 4 * (lane >> 5);
+#pragma unroll
+        for (int ot = 0; ot < 4; ++ot) {
+          const bf16_t* wp = sW2 + (ot * 32 + (lane & 31)) * LDW2 + kbase;
+          u32x4 wv;
+          const u32x2 lo = *reinterpret_cast<const u32x2*>(wp);
+          const u32x2 hi = *reinterpret_cast<const u32x2*>(wp + 8);
+          wv.x = lo.x; wv.y = lo.y; wv.z = hi.x; wv.w = hi.y;
+          out[ot] = mfma32(as_frag(wv), hf, out[ot]);
+        }
+      }
+    }
+    __syncthreads();
+  }
+  stage_t_f32(out, sS, wave, lane);
+  __syncthreads();
+  store_tile_f32<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), a.residual ? x : nullptr, tid);
+}
+
+template <typename K, typename A>
+int launch_tiles(K kern, const A& a, int64_t n_outer, int N, hipStream_t stream) {
+  const int64_t tiles = n_outer * ((N + TM - 1) / TM);
+  if (tiles <= 0 || tiles > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(256), 0, stream, a);
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+}  // namespace
+
+int launch_trimul_prologue(const TriMulArgs& a, hipStream_t s) {
+  if (a.N <= 0 || a.Np < a.N || (a.Np & 7) || !a.pair || !a.a_buf || !a.b_buf || !a.w_pg) return AF3_ERR_BAD_ARG;
+  if (!aligned16(a.pair) || !aligned16(a.a_buf) || !aligned16(a.b_buf) || !aligned16(a.w_pg)) return AF3_ERR_BAD_ARG;
+  return a.io_f32 ? launch_tiles(trimul_prologue_kernel<float>, a, a.N, a.N, s)
+                  : launch_tiles(trimul_prologue_kernel<bf16_t>, a, a.N, a.N, s);
+}
+int launch_trimul_epilogue(const TriMulArgs& a, hipStream_t s) {
+  if (a.N <= 0 || a.Np < a.N || (a.Np & 7) || !a.pair || !a.t_buf || !a.out || !a.w_gl || !a.w_out ||
+      !a.ln_c_w || !a.ln_c_b)
+    return AF3_ERR_BAD_ARG;
+  if (!aligned16(a.pair) || !aligned16(a.t_buf) || !aligned16(a.out) || !aligned16(a.w_gl) || !aligned16(a.w_out))
+    return AF3_ERR_BAD_ARG;
+  return a.io_f32 ? launch_tiles(trimul_epilogue_kernel<float>, a, a.N, a.N, s)
+                  : launch_tiles(trimul_epilogue_kernel<bf16_t>, a, a.N, a.N, s);
+}
+int launch_attn_proj(const AttnProjArgs& a, hipStream_t s) {
+  if (a.N <= 0 || !a.pair || a.n_chunks < 0 || a.n_chunks > 4 || a.n_bias < 0) return AF3_ERR_BAD_ARG;
+  if (a.n_chunks > 0 && (!a.w_main || !a.out_main || (a.ld_main & 7) || a.ld_main < a.n_chunks * C)) return AF3_ERR_BAD_ARG;
+  if (a.n_bias > 0 && (!a.w_bias || !a.out_bias)) return AF3_ERR_BAD_ARG;
+  if (!aligned16(a.pair) || !aligned16(a.w_main) || !aligned16(a.out_main) || !aligned16(a.w_bias)) return AF3_ERR_BAD_ARG;
+  return a.io_f32 ? launch_tiles(attn_proj_kernel<float>, a, a.N, a.N, s)
+                  : launch_tiles(attn_proj_kernel<bf16_t>, a, a.N, a.N, s);
+}
+int launch_attn_out(const AttnOutArgs& a, hipStream_t s) {
+  if (a.N <= 0 || !a.og || !a.w_out || !a.out || (a.ld_og & 7) || (a.residual && !a.pair)) return AF3_ERR_BAD_ARG;
+  if (!aligned16(a.og) || !aligned16(a.w_out) || !aligned16(a.out) || !aligned16(a.pair)) return AF3_ERR_BAD_ARG;
+  return a.io_f32 ? launch_tiles(attn_out_kernel<float>, a, a.N, a.N, s)
+                  : launch_tiles(attn_out_kernel<bf16_t>, a, a.N, a.N, s);
+}
+int launch_transition(const TransitionArgs& a, hipStream_t s) {
+  // x is [rows][128]; handled as `rows` positions in one long row
+  if (a.N <= 0 || !a.x || !a.out || !a.w1 || !a.w2 || a.hidden <= 0 || (a.hidden & 63)) return AF3_ERR_BAD_ARG;
+  if (!aligned16(a.x) || !aligned16(a.out) || !aligned16(a.w1) || !aligned16(a.w2)) return AF3_ERR_BAD_ARG;
+  return a.io_f32 ? launch_tiles(transition_kernel<float>, a, 1, a.N, s)
+                  : launch_tiles(transition_kernel<bf16_t>, a, 1, a.N, s);
+}

@@ -1,0 +1,30 @@
+"""Drop-in modules for the reference's hot-path `nn` classes
+(src/distributed_xfold/nn/*): same constructor keywords, parameter names and
+`forward` signatures; `forward` runs the HIP kernels."""
+
+from .base import HipModule, enable_hip
+from .triangle_multiplication import TriangleMultiplication
+from .attention import GridSelfAttention
+from .primitives import Transition
+from .diffusion_transformer import (AdaptiveLayerNorm, AdaLNZero, DiffusionTransition, SelfAttention,
+                                    DiffusionTransformer, CrossAttention, DiffusionCrossAttTransformer)
+from .pairformer import PairformerBlock, PairformerStack
+
+# names used by the reference for the same modules
+XSMMTriangleMultiplication = TriangleMultiplication
+DistributeTriangleMultiplication = TriangleMultiplication
+DistributeGridSelfAttention = GridSelfAttention
+DistributeTransition = Transition
+DistributeAdaLNZero = AdaLNZero
+DistributeDiffusionTransition = DiffusionTransition
+DistributeSelfAttention = SelfAttention
+DistributeDiffusionTransformer = DiffusionTransformer
+DistrubuteCrossAttention = CrossAttention
+DistributeDiffusionCrossAttTransformer = DiffusionCrossAttTransformer
+DistributePairformerBlock = PairformerBlock
+
+__all__ = [
+    "HipModule", "enable_hip", "TriangleMultiplication", "GridSelfAttention", "Transition",
+    "AdaptiveLayerNorm", "AdaLNZero", "DiffusionTransition", "SelfAttention", "DiffusionTransformer",
+    "CrossAttention", "DiffusionCrossAttTransformer", "PairformerBlock", "PairformerStack",
+]

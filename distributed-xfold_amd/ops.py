@@ -1,0 +1,319 @@
+"""Operator layer: torch tensors in, C ABI calls out.
+
+These functions stand where the reference's `torch.ops._alpha_attention.*`
+operators and their Python wrappers stand (src/distributed_xfold/xsmm_kernels/
+prototypes/*.py): they check dtype / shape / device / contiguity (ValueError),
+own the output and scratch allocation through torch's caching allocator, pass
+raw device pointers and the current HIP stream to libaf3hip.so, and turn a
+non-zero return code into a RuntimeError.  No arithmetic happens here.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import lib as _L
+
+_workspaces: dict = {}
+
+
+def _ws(nbytes: int, device) -> torch.Tensor:
+    """Per-device scratch buffer, grown on demand and reused between calls
+    (calls on one stream are ordered, so reuse is safe)."""
+    key = (device.type, device.index)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def release_workspaces():
+    _workspaces.clear()
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return _L.AF3_BF16
+    if t.dtype == torch.float32:
+        return _L.AF3_F32
+    raise ValueError(f"activation dtype must be bfloat16 or float32, got {t.dtype}")
+
+
+def _gpu(t: torch.Tensor, name: str, dtype=None, shape=None) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor):
+        raise ValueError(f"{name}: expected a tensor")
+    if not t.is_cuda:
+        raise ValueError(f"{name}: tensor must live on the GPU (got {t.device}); there is no CPU path")
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError(f"{name}: expected dtype {dtype}, got {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: tensor must be contiguous")
+    return t
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _mask_f32(mask: Optional[torch.Tensor], shape, name: str):
+    if mask is None:
+        return None
+    if not mask.is_cuda:
+        raise ValueError(f"{name}: tensor must live on the GPU")
+    if tuple(mask.shape) != tuple(shape):
+        raise ValueError(f"{name}: expected shape {tuple(shape)}, got {tuple(mask.shape)}")
+    return mask.to(torch.float32).contiguous()
+
+
+# --------------------------------------------------------------------------
+def triangle_multiplication(act, mask, equation_flag, left_norm_input_weight, left_norm_input_bias,
+                            w_proj_gate, center_norm_weight, center_norm_bias,
+                            w_output_projection, w_gating_linear, residual=False, out=None):
+    """traingle_multiplication_forward (csrc/Alpha_Attention.cpp:148-169); returns
+    the update, or act + update written in place when residual=True."""
+    lib = _L.load()
+    _gpu(act, "act")
+    if act.dim() != 3 or act.shape[0] != act.shape[1] or act.shape[2] != 128:
+        raise ValueError(f"act: expected [N, N, 128], got {tuple(act.shape)}")
+    n = act.shape[0]
+    io = _dt(act)
+    maskf = _mask_f32(mask, (n, n), "mask")
+    for nm, t in (("left_norm_input_weight", left_norm_input_weight), ("left_norm_input_bias", left_norm_input_bias),
+                  ("center_norm_weight", center_norm_weight), ("center_norm_bias", center_norm_bias)):
+        _gpu(t, nm, torch.float32, (128,))
+    _gpu(w_proj_gate, "w_proj_gate", torch.bfloat16, (4, 128, 128))
+    _gpu(w_output_projection, "w_output_projection", torch.bfloat16, (128, 128))
+    _gpu(w_gating_linear, "w_gating_linear", torch.bfloat16, (128, 128))
+    if out is None:
+        out = act if residual else torch.empty_like(act)
+    else:
+        _gpu(out, "out", act.dtype, act.shape)
+    nbytes = lib.af3_triangle_multiplication_workspace_bytes(n)
+    ws = _ws(nbytes, act.device)
+    rc = lib.af3_triangle_multiplication_forward(
+        _p(act), io, _p(maskf), int(equation_flag), _p(left_norm_input_weight), _p(left_norm_input_bias),
+        _p(w_proj_gate), _p(center_norm_weight), _p(center_norm_bias), _p(w_output_projection),
+        _p(w_gating_linear), _p(out), int(bool(residual)), n, _p(ws), ws.numel(), _stream(act.device))
+    _L.check(rc, "af3_triangle_multiplication_forward")
+    return out
+
+
+def grid_self_attn(pair, mask, transpose, act_norm_weight, act_norm_bias, w_pair_bias, nonbatched_bias,
+                   w_qkvg, w_output, num_head, residual=False, out=None):
+    """grid_self_attn_forward (csrc/Alpha_Attention.cpp:50-70) fused with the steps
+    of DistributeGridSelfAttention.xsmm_forward (nn/d_attention.py:58-85)."""
+    lib = _L.load()
+    _gpu(pair, "pair")
+    if pair.dim() != 3 or pair.shape[0] != pair.shape[1] or pair.shape[2] != 128:
+        raise ValueError(f"pair: expected [N, N, 128], got {tuple(pair.shape)}")
+    n = pair.shape[0]
+    io = _dt(pair)
+    maskf = _mask_f32(mask, (n, n), "mask")
+    if act_norm_weight is not None:
+        _gpu(act_norm_weight, "act_norm_weight", torch.float32, (128,))
+        _gpu(act_norm_bias, "act_norm_bias", torch.float32, (128,))
+    if w_pair_bias is not None:
+        _gpu(w_pair_bias, "w_pair_bias", torch.bfloat16)
+        if w_pair_bias.dim() != 2 or w_pair_bias.shape[1] != 128 or w_pair_bias.shape[0] % 32 \
+                or w_pair_bias.shape[0] < num_head:
+            raise ValueError("w_pair_bias: expected [roundup(num_head, 32), 128]")
+    if nonbatched_bias is not None:
+        _gpu(nonbatched_bias, "nonbatched_bias", torch.float32, (num_head, n, n))
+    _gpu(w_qkvg, "w_qkvg", torch.bfloat16, (4, 128, 128))
+    _gpu(w_output, "w_output", torch.bfloat16, (128, 128))
+    if out is None:
+        out = pair if residual else torch.empty_like(pair)
+    else:
+        _gpu(out, "out", pair.dtype, pair.shape)
+    nbytes = lib.af3_grid_self_attn_workspace_bytes(n, num_head)
+    ws = _ws(nbytes, pair.device)
+    rc = lib.af3_grid_self_attn_forward(
+        _p(pair), io, _p(maskf), int(bool(transpose)), _p(act_norm_weight), _p(act_norm_bias),
+        _p(w_pair_bias), _p(nonbatched_bias), _p(w_qkvg), _p(w_output), int(num_head),
+        _p(out), int(bool(residual)), n, _p(ws), ws.numel(), _stream(pair.device))
+    _L.check(rc, "af3_grid_self_attn_forward")
+    return out
+
+
+def transition128(act, layernorm_weight, layernorm_bias, w1_packed, w2, residual=False, out=None):
+    """transition_forward (csrc/Alpha_Attention.cpp:116-125) for 128-channel rows."""
+    lib = _L.load()
+    _gpu(act, "act")
+    if act.shape[-1] != 128:
+        raise ValueError("act: last dimension must be 128")
+    io = _dt(act)
+    hidden = w2.shape[1]
+    _gpu(layernorm_weight, "layernorm_weight", torch.float32, (128,))
+    _gpu(layernorm_bias, "layernorm_bias", torch.float32, (128,))
+    _gpu(w1_packed, "w1_packed", torch.bfloat16, (hidden // 64, 128, 128))
+    _gpu(w2, "w2", torch.bfloat16, (128, hidden))
+    rows = act.numel() // 128
+    if out is None:
+        out = act if residual else torch.empty_like(act)
+    else:
+        _gpu(out, "out", act.dtype, act.shape)
+    rc = lib.af3_transition_forward(_p(act), io, _p(layernorm_weight), _p(layernorm_bias), _p(w1_packed),
+                                    _p(w2), int(hidden), _p(out), int(bool(residual)), rows,
+                                    _stream(act.device))
+    _L.check(rc, "af3_transition_forward")
+    return out
+
+
+def batch_diffusion_self_attention(q_data, key_mask, nonbatched_bias, w_qkvg, query_b, num_head,
+                                   out_dtype=torch.bfloat16):
+    """batch_diffusion_self_attention_forward (csrc/Alpha_Attention.cpp:72-92).
+    q_data [B, S, C] bf16 (already normalised); returns [B, S, H, C/H]."""
+    lib = _L.load()
+    _gpu(q_data, "q_data", torch.bfloat16)
+    if q_data.dim() != 3:
+        raise ValueError("q_data: expected [B, S, C]")
+    b, s, c = q_data.shape
+    km = _mask_f32(key_mask, (s,), "key_mask")
+    if nonbatched_bias is not None:
+        _gpu(nonbatched_bias, "nonbatched_bias", torch.float32, (num_head, s, s))
+    _gpu(w_qkvg, "w_qkvg", torch.bfloat16, (4 * c, c))
+    if query_b is not None:
+        _gpu(query_b, "query_b", torch.float32, (c,))
+    out = torch.empty((b, s, num_head, c // num_head), dtype=out_dtype, device=q_data.device)
+    nbytes = lib.af3_batch_diffusion_self_attention_workspace_bytes(b, s, c)
+    ws = _ws(nbytes, q_data.device)
+    rc = lib.af3_batch_diffusion_self_attention_forward(
+        _p(q_data), _p(km), _p(nonbatched_bias), _p(w_qkvg), _p(query_b), int(num_head), _p(out),
+        _dt(out), b, s, c, _p(ws), ws.numel(), _stream(q_data.device))
+    _L.check(rc, "af3_batch_diffusion_self_attention_forward")
+    return out
+
+
+def batch_diffusion_cross_attention(q_data, m_data, pair_logits, mask_q, mask_k, w_qg, w_kv, query_b,
+                                    num_head, out_dtype=torch.bfloat16):
+    """batch_diffusion_cross_attention_forward (csrc/Alpha_Attention.cpp:127-146).
+    q_data [B, Sq, C], m_data [B, Sk, C] bf16; pair_logits [Bb, H, Sq, Sk] fp32 and
+    masks [Bb, Sq] / [Bb, Sk] with B a multiple of Bb; returns [B, Sq, H, C/H]."""
+    lib = _L.load()
+    _gpu(q_data, "q_data", torch.bfloat16)
+    _gpu(m_data, "m_data", torch.bfloat16)
+    b, sq, c = q_data.shape
+    sk = m_data.shape[1]
+    if m_data.shape[0] != b or m_data.shape[2] != c:
+        raise ValueError("m_data: batch / channel mismatch with q_data")
+    bias_batches = b
+    if pair_logits is not None:
+        _gpu(pair_logits, "pair_logits", torch.float32)
+        bias_batches = pair_logits.shape[0]
+        if tuple(pair_logits.shape[1:]) != (num_head, sq, sk):
+            raise ValueError("pair_logits: expected [Bb, H, Sq, Sk]")
+    mq = mk = None
+    if mask_q is not None:
+        bias_batches = mask_q.shape[0]
+        mq = _mask_f32(mask_q, (bias_batches, sq), "mask_q")
+        mk = _mask_f32(mask_k, (bias_batches, sk), "mask_k")
+    if pair_logits is not None and pair_logits.shape[0] != bias_batches:
+        raise ValueError("pair_logits and masks must share their batch size")
+    _gpu(w_qg, "w_qg", torch.bfloat16, (2 * c, c))
+    _gpu(w_kv, "w_kv", torch.bfloat16, (2 * c, c))
+    if query_b is not None:
+        _gpu(query_b, "query_b", torch.float32, (c,))
+    out = torch.empty((b, sq, num_head, c // num_head), dtype=out_dtype, device=q_data.device)
+    nbytes = lib.af3_batch_diffusion_cross_attention_workspace_bytes(b, sq, sk, c)
+    ws = _ws(nbytes, q_data.device)
+    rc = lib.af3_batch_diffusion_cross_attention_forward(
+        _p(q_data), _p(m_data), _p(pair_logits), _p(mq), _p(mk), bias_batches, _p(w_qg), _p(w_kv),
+        _p(query_b), int(num_head), _p(out), _dt(out), b, sq, sk, c, _p(ws), ws.numel(),
+        _stream(q_data.device))
+    _L.check(rc, "af3_batch_diffusion_cross_attention_forward")
+    return out
+
+
+def pair_logits(pair, norm_weight, norm_bias, w_padded, n_out):
+    """LayerNorm + projection of the pair tensor to [n_out, N, N] fp32 logits
+    (nn/d_pairformer.py:160-162, nn/d_diffusion_transformer.py:299-305)."""
+    lib = _L.load()
+    _gpu(pair, "pair")
+    if pair.dim() != 3 or pair.shape[0] != pair.shape[1] or pair.shape[2] != 128:
+        raise ValueError(f"pair: expected [N, N, 128], got {tuple(pair.shape)}")
+    n = pair.shape[0]
+    _gpu(norm_weight, "norm_weight", torch.float32, (128,))
+    if norm_bias is not None:
+        _gpu(norm_bias, "norm_bias", torch.float32, (128,))
+    _gpu(w_padded, "w_padded", torch.bfloat16)
+    if w_padded.dim() != 2 or w_padded.shape[1] != 128 or w_padded.shape[0] % 32 or w_padded.shape[0] < n_out:
+        raise ValueError("w_padded: expected [roundup(n_out, 32), 128]")
+    out = torch.empty((n_out, n, n), dtype=torch.float32, device=pair.device)
+    rc = lib.af3_pair_logits_forward(_p(pair), _dt(pair), _p(norm_weight), _p(norm_bias), _p(w_padded),
+                                     int(n_out), _p(out), n, _stream(pair.device))
+    _L.check(rc, "af3_pair_logits_forward")
+    return out
+
+
+def layer_norm(x, weight=None, bias=None, scale=None, shift=None):
+    """Row LayerNorm (+ optional adaptive scale/shift) -> bf16.  scale/shift are
+    fp32 views [cond_rows, C] that may be column slices of one wider tensor."""
+    lib = _L.load()
+    _gpu(x, "x")
+    c = x.shape[-1]
+    rows = x.numel() // c
+    for nm, t in (("weight", weight), ("bias", bias)):
+        if t is not None:
+            _gpu(t, nm, torch.float32, (c,))
+    cond_rows = cond_ld = 0
+    if scale is not None:
+        for nm, t in (("scale", scale), ("shift", shift)):
+            if not t.is_cuda or t.dtype != torch.float32 or t.dim() != 2 or t.shape[1] != c or t.stride(1) != 1:
+                raise ValueError(f"{nm}: expected an fp32 GPU matrix [cond_rows, {c}] with unit column stride")
+        if scale.stride(0) != shift.stride(0) or scale.shape[0] != shift.shape[0]:
+            raise ValueError("scale and shift must share rows and row stride")
+        cond_rows, cond_ld = scale.shape[0], scale.stride(0)
+        if rows % cond_rows:
+            raise ValueError("rows must be a multiple of the conditioning rows")
+    y = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    rc = lib.af3_layer_norm_forward(_p(x), _dt(x), _p(y), rows, c, _p(weight), _p(bias), _p(scale), _p(shift),
+                                    cond_rows, cond_ld, _stream(x.device))
+    _L.check(rc, "af3_layer_norm_forward")
+    return y
+
+
+def linear(x, w, bias=None, out_dtype=torch.bfloat16, mode=_L.LINEAR_PLAIN, alpha=1.0, sigmoid=False,
+           gate=None, residual=None, out=None):
+    """y = epilogue(x @ w.T) on bf16 MFMA (af3_linear_forward)."""
+    lib = _L.load()
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(w, "w", torch.bfloat16)
+    k = x.shape[-1]
+    m = x.numel() // k
+    n = w.shape[0]
+    if w.dim() != 2 or w.shape[1] != k:
+        raise ValueError(f"w: expected [N, {k}], got {tuple(w.shape)}")
+    if bias is not None:
+        _gpu(bias, "bias", torch.float32, (n,))
+    n_out = n // 2 if mode == _L.LINEAR_SWIGLU else n
+    shape = tuple(x.shape[:-1]) + (n_out,)
+    if out is None:
+        out = torch.empty(shape, dtype=out_dtype, device=x.device)
+    else:
+        _gpu(out, "out", None, shape)
+    gate_rows = 0
+    if gate is not None:
+        _gpu(gate, "gate", torch.float32)
+        if gate.shape[-1] != n:
+            raise ValueError("gate: last dimension must equal the output width")
+        gate_rows = gate.numel() // n
+        if m % gate_rows:
+            raise ValueError("rows must be a multiple of the gate rows")
+    res_dt = 0
+    if residual is not None:
+        _gpu(residual, "residual", None, shape)
+        res_dt = _dt(residual)
+    rc = lib.af3_linear_forward(_p(x), _p(w), _p(bias), _p(out), _dt(out), m, n, k, int(mode), float(alpha),
+                                int(bool(sigmoid)), _p(gate), gate_rows, _p(residual), res_dt,
+                                _stream(x.device))
+    _L.check(rc, "af3_linear_forward")
+    return out

@@ -1,0 +1,217 @@
+/* C ABI of libaf3hip.so: the AlphaFold3 Pairformer / diffusion-transformer hot
+ * path of hasaki321/Distributed-xfold as hand-written gfx950 (MI355X) kernels.
+ *
+ * Each entry point stands where one of the reference's fused CPU operators
+ * (namespace `_alpha_attention`, src/distributed_xfold/xsmm_kernels/csrc/
+ * Alpha_Attention.cpp:181-222) or one of the eager PyTorch steps wrapped around
+ * them stands; the reference interface it replaces is cited on each.
+ *
+ * Conventions
+ *  - All pointers are DEVICE pointers, 16-byte aligned, dense row-major unless a
+ *    stride argument says otherwise.  Nothing here allocates, frees or
+ *    synchronises: work is enqueued on `stream` and the caller owns every
+ *    buffer, including the scratch `workspace` whose size the matching
+ *    *_workspace_bytes function returns.
+ *  - Activations of the residual stream are bf16 (AF3_BF16) or fp32 (AF3_F32);
+ *    matrix operands are always rounded to bf16 for the MFMA units and
+ *    accumulated in fp32.  Weights are bf16 in the packed layouts described per
+ *    function (the host packs them once, as the reference's load_xsmm_params
+ *    does); LayerNorm scales/offsets and biases are fp32.
+ *  - Return value: AF3_OK (0) or a negative AF3_ERR_* code; af3_error_string
+ *    names it.  A non-zero return means nothing was enqueued by the failing
+ *    step.
+ */
+#ifndef AF3_HIP_H_
+#define AF3_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AF3_OK 0
+#define AF3_ERR_BAD_ARG (-1)
+#define AF3_ERR_WORKSPACE (-2)
+#define AF3_ERR_LAUNCH (-3)
+#define AF3_ERR_UNSUPPORTED (-4)
+
+#define AF3_BF16 0
+#define AF3_F32 1
+
+typedef void* af3_stream_t; /* a hipStream_t */
+
+int af3_abi_version(void);
+const char* af3_error_string(int code);
+
+/* ---------------------------------------------------------------------------
+ * Triangle multiplication.  Replaces
+ *   torch.ops._alpha_attention.traingle_multiplication_forward
+ *   (csrc/Alpha_Attention.cpp:148-169 schema :206-210; bodies
+ *   csrc/triangle_multiplication{,_bf16}.h) together with the residual add of
+ *   nn/d_pairformer.py:122-123.
+ * act [N,N,128]; mask [N,N] fp32 0/1 or NULL; equation_flag 0 = outgoing
+ * "ikc,jkc->ijc", 1 = incoming "kjc,kic->ijc" (prototypes/
+ * TriangleMultiplication.py:34-38).  out [N,N,128] in io_dtype; with
+ * residual != 0, out = act + update and out may alias act.
+ * Packed weights:
+ *   w_proj_gate [4][128][128]: chunk 0/1 = operand a, channels 0-63 / 64-127,
+ *     chunk 2/3 = operand b; inside a chunk rows 0-63 are `projection` rows and
+ *     rows 64-127 the matching `gate` rows.  Operand a of channel c is row 2c of
+ *     the nn.Linear weight, operand b row 2c+1 (d_triangle_multiplication.py:
+ *     162-165, de-interleave :128-129).
+ *   w_gating_linear, w_output_projection [128][128] as stored by nn.Linear.
+ */
+size_t af3_triangle_multiplication_workspace_bytes(int64_t n_token);
+int af3_triangle_multiplication_forward(
+    const void* act, int io_dtype, const float* mask, int equation_flag,
+    const float* left_norm_input_weight, const float* left_norm_input_bias,
+    const uint16_t* w_proj_gate,
+    const float* center_norm_weight, const float* center_norm_bias,
+    const uint16_t* w_output_projection, const uint16_t* w_gating_linear,
+    void* out, int residual, int64_t n_token,
+    void* workspace, size_t workspace_bytes, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Triangle (grid) self-attention.  Replaces
+ *   torch.ops._alpha_attention.grid_self_attn_forward
+ *   (csrc/Alpha_Attention.cpp:50-70, schema :182-185; bodies
+ *   csrc/grid_self_attention{,_bf16}.h) AND the eager steps
+ *   DistributeGridSelfAttention.xsmm_forward wraps around it
+ *   (nn/d_attention.py:58-85): LayerNorm, the 128->H pair-bias projection, the
+ *   key-mask bias, the transpose for the ending-node operator and its inverse,
+ *   plus the residual add of nn/d_pairformer.py:132,144.
+ * pair [N,N,128]; mask [N,N] fp32 0/1 indexed (row of the possibly transposed
+ * tensor, key) exactly as d_attention.py:63 uses it; masked keys are replaced by
+ * -1e9.  act_norm_* NULL means `pair` is already normalised (operator-level
+ * use).  Pair bias: either w_pair_bias ([roundup(H,32)][128], zero padded;
+ * projected from LayerNorm(pair)) or a precomputed nonbatched_bias [H,N,N]
+ * fp32, or neither.
+ * Packed weights: w_qkvg [4][128][128] = q, k, v, gating_query as stored by
+ * nn.Linear ([out, in]; equal to the reference's query_w[C,H,d] transposed and
+ * flattened); w_output [128][128] likewise.  q is scaled by head_dim^-1/2.
+ */
+size_t af3_grid_self_attn_workspace_bytes(int64_t n_token, int num_head);
+int af3_grid_self_attn_forward(
+    const void* pair, int io_dtype, const float* mask, int transpose,
+    const float* act_norm_weight, const float* act_norm_bias,
+    const uint16_t* w_pair_bias, const float* nonbatched_bias,
+    const uint16_t* w_qkvg, const uint16_t* w_output, int num_head,
+    void* out, int residual, int64_t n_token,
+    void* workspace, size_t workspace_bytes, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Transition (SwiGLU) on 128-channel activations, one fused kernel.  Replaces
+ *   torch.ops._alpha_attention.transition_forward
+ *   (csrc/Alpha_Attention.cpp:116-125, schema :187-189; body csrc/transition.h)
+ *   and DistributeTransition.forward (nn/d_primitives.py:31-35), plus the
+ *   residual add of nn/d_pairformer.py:146.
+ * act [rows,128]; w1 [hidden/64][128][128]: slab s holds transition1 rows
+ * 64s..64s+63 (the silu half) followed by rows hidden+64s..hidden+64s+63 (the
+ * linear half); w2 [128][hidden] as stored by nn.Linear.  hidden = factor*128.
+ */
+int af3_transition_forward(
+    const void* act, int io_dtype,
+    const float* layernorm_weight, const float* layernorm_bias,
+    const uint16_t* w1_packed, const uint16_t* w2, int hidden,
+    void* out, int residual, int64_t rows, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Pair-biased gated self-attention without output projection.  Replaces
+ *   torch.ops._alpha_attention.batch_diffusion_self_attention_forward
+ *   (csrc/Alpha_Attention.cpp:72-92, schema :191-194; bodies
+ *   csrc/batch_diffusion_self_attention{,_bf16}.h), used for the Pairformer
+ *   single attention and the diffusion transformer
+ *   (nn/d_diffusion_transformer.py:197-218).
+ * q_data [B,S,C] bf16, already (adaptive-)LayerNorm-ed; key_mask [S] fp32 0/1
+ * (masked keys replaced by -1e9) or NULL; nonbatched_bias [H,S,S] fp32 shared
+ * by the batch, or NULL.  w_qkvg [4C][C] bf16 = q, k, v, gating_query rows as
+ * stored by nn.Linear; query_b [C] fp32.  head_dim = C/H in {24, 32, 48}.
+ * out [B,S,H,head_dim] (= [B,S,C]) in out_dtype: sigmoid(gate) * softmax(..) v.
+ */
+size_t af3_batch_diffusion_self_attention_workspace_bytes(int64_t batch, int64_t seq, int channels);
+int af3_batch_diffusion_self_attention_forward(
+    const uint16_t* q_data, const float* key_mask, const float* nonbatched_bias,
+    const uint16_t* w_qkvg, const float* query_b, int num_head,
+    void* out, int out_dtype, int64_t batch, int64_t seq, int channels,
+    void* workspace, size_t workspace_bytes, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Windowed (atom) cross-attention without output projection.  Replaces
+ *   torch.ops._alpha_attention.batch_diffusion_cross_attention_forward
+ *   (csrc/Alpha_Attention.cpp:127-146, schema :201-204; bodies
+ *   csrc/batch_diffusion_cross_attention{,_bf16}.h) and the bias construction
+ *   of DistrubuteCrossAttention.xsmm_forward (nn/d_diffusion_transformer.py:
+ *   400-417).
+ * q_data [B,Sq,C], m_data [B,Sk,C] bf16 (already adaptive-LayerNorm-ed), B =
+ * samples * subsets.  Bias = pair_logits[b % bias_batches][H][Sq][Sk] (fp32 or
+ * NULL) + 1e9 where mask_q[b % bias_batches][q] == 0 and
+ * mask_k[b % bias_batches][k] == 0 (masks fp32 0/1 or both NULL).  A fully
+ * batched bias [B,H,Sq,Sk], as the reference operator takes, is the case
+ * bias_batches == B with NULL masks.
+ * w_qg [2C][C] = q_projection, gating_query; w_kv [2C][C] = k_projection,
+ * v_projection (nn.Linear layout); query_b [C] fp32.
+ */
+size_t af3_batch_diffusion_cross_attention_workspace_bytes(int64_t batch, int64_t sq, int64_t sk, int channels);
+int af3_batch_diffusion_cross_attention_forward(
+    const uint16_t* q_data, const uint16_t* m_data,
+    const float* pair_logits, const float* mask_q, const float* mask_k, int64_t bias_batches,
+    const uint16_t* w_qg, const uint16_t* w_kv, const float* query_b, int num_head,
+    void* out, int out_dtype, int64_t batch, int64_t sq, int64_t sk, int channels,
+    void* workspace, size_t workspace_bytes, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Pair-logit projection: out[h][i][j] = (LayerNorm(pair)[i][j] . w[h]).
+ * Replaces the eager `single_pair_logits_projection(single_pair_logits_norm(
+ * pair)).permute(2,0,1)` of nn/d_pairformer.py:160-162 and the
+ * `pair_logits_projection` + rearrange of nn/d_diffusion_transformer.py:299-305.
+ * pair [N,N,128]; norm_bias may be NULL; w [roundup(n_out,32)][128] zero padded.
+ * out [n_out][N][N] fp32.
+ */
+int af3_pair_logits_forward(
+    const void* pair, int io_dtype, const float* norm_weight, const float* norm_bias,
+    const uint16_t* w, int n_out, float* out, int64_t n_token, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Row LayerNorm / adaptive LayerNorm -> bf16.  Replaces fastnn.LayerNorm on
+ * the single / diffusion / atom activations and AdaptiveLayerNorm.forward
+ * (nn/d_diffusion_transformer.py:61-74):
+ *   y = LN(x) [* weight + bias];  if scale: y = sigmoid(scale[r]) * y + shift[r],
+ *   r = row % cond_rows (the conditioning is shared by the sample batch).
+ * x [rows,C] in x_dtype, y [rows,C] bf16, scale/shift fp32 with `cond_rows`
+ * rows of stride `cond_ld` elements (so both can live in one [cond_rows, 2C]
+ * projection output).
+ */
+int af3_layer_norm_forward(
+    const void* x, int x_dtype, uint16_t* y, int64_t rows, int channels,
+    const float* weight, const float* bias,
+    const float* scale, const float* shift, int64_t cond_rows, int64_t cond_ld,
+    af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Dense projection y = epilogue(x W^T) on bf16 MFMA.  Replaces the eager
+ * nn.Linear / fastnn.gated_linear_unit / AdaLNZero steps around the fused
+ * operators (nn/d_diffusion_transformer.py:99-118, 142-145; nn/d_primitives.py:
+ * 33-34).  x [M,K] bf16, w [N,K] bf16 (nn.Linear layout).
+ *  mode AF3_LINEAR_PLAIN : y = (x W^T + bias) * alpha, optional sigmoid; y [M,N]
+ *  mode AF3_LINEAR_SWIGLU: y = silu(a) * b, y [M,N/2] bf16; w rows packed in
+ *        blocks of 64: 32 rows of the silu half, then the 32 matching rows of
+ *        the linear half
+ *  mode AF3_LINEAR_GATE_RES: y = residual + gate[m % gate_rows] * (x W^T + bias)
+ *        (gate fp32 [gate_rows,N] or NULL; residual in res_dtype or NULL)
+ */
+#define AF3_LINEAR_PLAIN 0
+#define AF3_LINEAR_SWIGLU 2
+#define AF3_LINEAR_GATE_RES 3
+int af3_linear_forward(
+    const uint16_t* x, const uint16_t* w, const float* bias,
+    void* y, int y_dtype, int64_t m, int n, int k,
+    int mode, float alpha, int sigmoid,
+    const float* gate, int64_t gate_rows,
+    const void* residual, int res_dtype, af3_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AF3_HIP_H_ */

@@ -65,6 +65,29 @@ LN_EPS = 1e-5
 MASK_FILL = -1e9
 
 
+# bf16 emulation: inside `with bf16_emulation():` every point where the HIP
+# kernels hand a value to the matrix cores or to HBM as bf16 is rounded here
+# too (the reference's own bf16 kernels round at the same kind of points,
+# csrc/triangle_multiplication_bf16.h:160-162,230,273,503 and
+# csrc/grid_self_attention_bf16.h:250).  Outside the context `_r` is the
+# identity and the functions are the exact formulas.
+_EMULATE = False
+
+
+class bf16_emulation:
+    def __enter__(self):
+        global _EMULATE
+        self._old, _EMULATE = _EMULATE, True
+
+    def __exit__(self, *exc):
+        global _EMULATE
+        _EMULATE = self._old
+
+
+def _r(t: torch.Tensor) -> torch.Tensor:
+    return t.to(torch.bfloat16).to(t.dtype) if _EMULATE else t
+
+
 def _sub(p: Params, prefix: str) -> dict:
     """Entries of `p` below `prefix.` with the prefix removed."""
     pre = prefix + "."
@@ -115,20 +138,20 @@ def triangle_multiplication(pair, mask, p: Params, outgoing: bool):
     form operand a, odd ones operand b (the reshape(c, 2, ...) at :162-165).
     """
     c = pair.shape[-1]
-    x = layer_norm(pair, p["left_norm_input.weight"], p["left_norm_input.bias"])
+    x = _r(layer_norm(pair, p["left_norm_input.weight"], p["left_norm_input.bias"]))
     proj = linear(x, p["projection.weight"]).permute(2, 0, 1)       # [2c, N, N]
     if mask is not None:
         proj = proj * mask.to(x.dtype)[None]
     gate = linear(x, p["gate.weight"]).permute(2, 0, 1)
-    proj = proj * torch.sigmoid(gate)
+    proj = _r(proj * torch.sigmoid(gate))
     proj = proj.reshape(c, 2, *proj.shape[1:])
     a, b = proj[:, 0], proj[:, 1]                                    # [c, N, N]
     if outgoing:
         out = torch.einsum("cik,cjk->cij", a, b)
     else:
         out = torch.einsum("ckj,cki->cij", a, b)
-    out = out.permute(1, 2, 0)
-    out = layer_norm(out, p["center_norm.weight"], p["center_norm.bias"])
+    out = _r(out).permute(1, 2, 0)
+    out = _r(layer_norm(out, p["center_norm.weight"], p["center_norm.bias"]))
     out = linear(out, p["output_projection.weight"])
     out = out * torch.sigmoid(linear(x, p["gating_linear.weight"]))
     return out
@@ -145,11 +168,14 @@ def dot_product_attention(q, k, v, mask=None, bias=None):
     mask boolean/0-1, broadcastable to [..., Q, K]; masked logits are
     REPLACED by -1e9 after the bias has been added.
     """
-    logits = (q * (q.shape[-1] ** -0.5)) @ k.transpose(-1, -2)
+    logits = _r(q * (q.shape[-1] ** -0.5)) @ _r(k).transpose(-1, -2)
     if bias is not None:
         logits = logits + bias.to(logits.dtype)
     if mask is not None:
         logits = logits.masked_fill(~mask.to(torch.bool), MASK_FILL)
+    if _EMULATE:   # un-normalised probabilities are rounded before they meet v
+        e = _r(torch.exp(logits - logits.amax(dim=-1, keepdim=True)))
+        return (e @ _r(v)) / e.sum(dim=-1, keepdim=True)
     weights = torch.softmax(logits, dim=-1)
     return weights @ v
 
@@ -209,8 +235,8 @@ def grid_self_attention(pair, mask, p: Params, num_head: int, transpose: bool,
     if full_pair is None:
         full_pair = pair
     w, b = p["act_norm.weight"], p["act_norm.bias"]
-    x = layer_norm(pair, w, b)
-    nb = linear(layer_norm(full_pair, w, b), p["pair_bias_projection.weight"])
+    x = _r(layer_norm(pair, w, b))
+    nb = linear(_r(layer_norm(full_pair, w, b)), p["pair_bias_projection.weight"])
     nb = nb.permute(2, 0, 1)                                         # [H, Q, K]
     if transpose:
         x = x.permute(1, 0, 2)
@@ -226,7 +252,7 @@ def grid_self_attention(pair, mask, p: Params, num_head: int, transpose: bool,
     key_mask = mask.to(torch.bool)[:, None, None, :]
     avg = dot_product_attention(q, k, v, mask=key_mask, bias=nb[None])
     avg = avg.permute(0, 2, 1, 3).reshape(n_row, n_key, c)
-    avg = avg * torch.sigmoid(linear(x, p["gating_query.weight"]))
+    avg = _r(avg * _r(torch.sigmoid(linear(x, p["gating_query.weight"]))))
     out = linear(avg, p["output_projection.weight"])
     if transpose:
         out = out.permute(1, 0, 2)
@@ -241,12 +267,12 @@ def gated_linear_unit(x, weight_t):
     """kernel_test/transition.py:40-42: y = x @ W; silu(first half) * second half."""
     y = x @ weight_t.to(x.dtype)
     a, b = torch.chunk(y, 2, dim=-1)
-    return torch.nn.functional.silu(a) * b
+    return _r(torch.nn.functional.silu(a) * b)
 
 
 def transition(x, p: Params):
     """nn/d_primitives.py:31-35: LN -> GLU(transition1) -> transition2; no biases."""
-    x = layer_norm(x, p["input_layer_norm.weight"], p["input_layer_norm.bias"])
+    x = _r(layer_norm(x, p["input_layer_norm.weight"], p["input_layer_norm.bias"]))
     c = gated_linear_unit(x, p["transition1.weight"].transpose(0, 1))
     return linear(c, p["transition2.weight"])
 
@@ -264,12 +290,12 @@ def adaptive_layer_norm(x, single_cond, p: Params):
     Without: an ordinary affine LayerNorm.
     """
     if single_cond is None:
-        return layer_norm(x, p["layer_norm.weight"], p.get("layer_norm.bias"))
+        return _r(layer_norm(x, p["layer_norm.weight"], p.get("layer_norm.bias")))
     xn = layer_norm(x)
-    s = layer_norm(single_cond.to(x.dtype), p["single_cond_layer_norm.weight"])
+    s = _r(layer_norm(single_cond.to(x.dtype), p["single_cond_layer_norm.weight"]))
     scale = linear(s, p["single_cond_scale.weight"], p["single_cond_scale.bias"])
     shift = linear(s, p["single_cond_bias.weight"])
-    return torch.sigmoid(scale) * xn + shift
+    return _r(torch.sigmoid(scale) * xn + shift)
 
 
 def adaln_zero(x, single_cond, p: Params):
@@ -277,7 +303,7 @@ def adaln_zero(x, single_cond, p: Params):
     sigmoid(adaptive_zero_cond(single_cond)) when conditioned."""
     out = linear(x, p["transition2.weight"])
     if single_cond is not None:
-        cond = linear(single_cond.to(x.dtype), p["adaptive_zero_cond.weight"],
+        cond = linear(_r(single_cond.to(x.dtype)), p["adaptive_zero_cond.weight"],
                       p.get("adaptive_zero_cond.bias"))
         out = torch.sigmoid(cond) * out
     return out
@@ -312,7 +338,7 @@ def self_attention(x, mask, pair_logits, single_cond, p: Params, num_head: int):
     avg = avg.permute(0, 2, 1, 3).reshape(B, N, c)
     if not batched:
         avg = avg[0]
-    avg = avg * torch.sigmoid(linear(xa, p["gating_query.weight"]))
+    avg = _r(avg * _r(torch.sigmoid(linear(xa, p["gating_query.weight"]))))
     return adaln_zero(avg, single_cond, _sub(p, "adaptive_zero_init"))
 
 
@@ -371,11 +397,15 @@ def cross_attention(x_q, x_k, mask_q, mask_k, pair_logits, single_cond_q,
     q = q.reshape(q.shape[:-1] + (num_head, dk))
     k = k.reshape(k.shape[:-1] + (num_head, dk))
     v = v.reshape(v.shape[:-1] + (num_head, dv))
-    logits = torch.einsum("...qhc,...khc->...hqk", q * dk ** -0.5, k) + bias
-    weights = torch.softmax(logits, dim=-1)
-    avg = torch.einsum("...hqk,...khc->...qhc", weights, v)
+    logits = torch.einsum("...qhc,...khc->...hqk", _r(q * dk ** -0.5), _r(k)) + bias
+    if _EMULATE:
+        e = _r(torch.exp(logits - logits.amax(dim=-1, keepdim=True)))
+        weights = e / e.sum(dim=-1, keepdim=True)
+    else:
+        weights = torch.softmax(logits, dim=-1)
+    avg = torch.einsum("...hqk,...khc->...qhc", weights, _r(v))
     avg = avg.reshape(avg.shape[:-2] + (-1,))
-    avg = avg * torch.sigmoid(linear(xq, p["gating_query.weight"]))
+    avg = _r(avg * _r(torch.sigmoid(linear(xq, p["gating_query.weight"]))))
     return adaln_zero(avg, single_cond_q, _sub(p, "adaptive_zero_init"))
 
 

@@ -1,0 +1,145 @@
+"""CPU-side checks of the boundary: the shared library loads and exports every
+symbol include/af3_hip.h declares, the ctypes table matches the header, and the
+host-side weight packing / module plumbing behaves (no GPU compute)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from oracle import af3_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "af3_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(af3_[a-z0-9_]+)\s*\(", text)))
+
+
+def count_params(name):
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    m = re.search(r"\b%s\s*\((.*?)\)\s*;" % re.escape(name), text, flags=re.S)
+    args = m.group(1).strip()
+    return 0 if args in ("", "void") else args.count(",") + 1
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for required in ("af3_triangle_multiplication_forward", "af3_grid_self_attn_forward",
+                     "af3_transition_forward", "af3_batch_diffusion_self_attention_forward",
+                     "af3_batch_diffusion_cross_attention_forward"):
+        assert required in syms
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    if not os.path.exists(pkg.lib.LIB_PATH):
+        pytest.fail("libaf3hip.so is not built: run __graft_entry__.build()")
+    lib = ctypes.CDLL(pkg.lib.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} declared in af3_hip.h but not exported"
+
+
+def test_ctypes_table_matches_header(pkg):
+    assert sorted(pkg.lib.SIGNATURES) == declared_symbols()
+    for name, (_, args) in pkg.lib.SIGNATURES.items():
+        assert len(args) == count_params(name), name
+
+
+def test_error_strings_and_version(pkg):
+    lib = pkg.lib.load()
+    assert lib.af3_abi_version() == 1
+    assert lib.af3_error_string(0) == b"ok"
+    assert b"workspace" in lib.af3_error_string(-2)
+    with pytest.raises(pkg.lib.Af3Error):
+        pkg.lib.check(-1, "x")
+
+
+def test_workspace_queries(pkg):
+    lib = pkg.lib.load()
+    n = 100
+    np_ = 104
+    assert lib.af3_triangle_multiplication_workspace_bytes(n) >= 3 * 128 * n * np_ * 2
+    assert lib.af3_grid_self_attn_workspace_bytes(n, 4) >= n * n * (5 * 128 * 2 + 4 * 4)
+    assert lib.af3_triangle_multiplication_workspace_bytes(0) == 0
+
+
+def test_null_and_bad_arguments_are_rejected_without_a_gpu(pkg):
+    """Argument validation happens before any launch, so it can run here."""
+    lib = pkg.lib.load()
+    assert lib.af3_transition_forward(None, 0, None, None, None, None, 512, None, 0, 10, None) == -1
+    assert lib.af3_linear_forward(None, None, None, None, 0, 1, 8, 8, 0, 1.0, 0, None, 0, None, 0, None) == -1
+    assert lib.af3_triangle_multiplication_forward(None, 0, None, 0, None, None, None, None, None, None, None,
+                                                   None, 0, 8, None, 0, None) == -1
+
+
+def test_cpu_tensors_raise(pkg):
+    with pytest.raises(ValueError):
+        pkg.ops.layer_norm(torch.randn(4, 128))
+    mod = pkg.nn.Transition(c_x=128)
+    with pytest.raises(ValueError):
+        mod(torch.randn(4, 128))
+
+
+def test_pack_swiglu_and_pad_rows(pkg):
+    from distributed_xfold_amd.nn.base import pack_swiglu, pad_rows
+    hidden, c = 128, 8
+    w = torch.arange(2 * hidden * c, dtype=torch.float32).reshape(2 * hidden, c)
+    pk = pack_swiglu(w, 32)
+    for blk in range(hidden // 32):
+        assert torch.equal(pk[64 * blk: 64 * blk + 32], w[32 * blk: 32 * blk + 32])
+        assert torch.equal(pk[64 * blk + 32: 64 * blk + 64], w[hidden + 32 * blk: hidden + 32 * blk + 32])
+    padded = pad_rows(torch.ones(4, 8), 32)
+    assert padded.shape == (32, 8) and padded[4:].abs().sum() == 0 and padded[:4].sum() == 32
+
+
+def test_trimul_packing_matches_the_interleave(pkg):
+    """Packed chunk layout: operand a of channel c is nn.Linear row 2c, operand b
+    row 2c+1 (reference de-interleave, nn/d_triangle_multiplication.py:128-129)."""
+    mod = pkg.nn.TriangleMultiplication()
+    packed = mod.packed()["w_proj_gate"].float()
+    wp = mod.projection.weight.detach().bfloat16().float()
+    wg = mod.gate.weight.detach().bfloat16().float()
+    for chunk in range(4):
+        half, lo = chunk // 2, 64 * (chunk % 2)
+        for r in (0, 17, 63):
+            ch = lo + r
+            assert torch.equal(packed[chunk, r], wp[2 * ch + half])
+            assert torch.equal(packed[chunk, 64 + r], wg[2 * ch + half])
+
+
+def test_modules_share_the_reference_parameter_names(pkg):
+    g = torch.Generator().manual_seed(0)
+    pairs = [
+        (pkg.nn.PairformerBlock(), O.make_pairformer_block_params(g)),
+        (pkg.nn.PairformerBlock(with_single=False), O.make_pairformer_block_params(g, with_single=False)),
+        (pkg.nn.DiffusionTransformer(num_blocks=4), O.make_diffusion_transformer_params(g, num_blocks=4)),
+        (pkg.nn.DiffusionCrossAttTransformer(), O.make_cross_att_transformer_params(g)),
+        (pkg.nn.GridSelfAttention(), O.make_grid_self_attention_params(g)),
+        (pkg.nn.TriangleMultiplication(), O.make_triangle_multiplication_params(g)),
+        (pkg.nn.Transition(c_x=384), O.make_transition_params(g, 384)),
+    ]
+    for mod, params in pairs:
+        assert sorted(mod.state_dict()) == sorted(params)
+        for k, v in mod.state_dict().items():
+            assert v.shape == params[k].shape, k
+
+
+def test_reference_constructor_signatures(pkg):
+    """The reference's distributed classes take a device mesh first
+    (nn/d_attention.py:24, nn/d_primitives.py:23, nn/d_pairformer.py:37-47)."""
+    mesh = object()
+    nn = pkg.nn
+    assert nn.DistributeGridSelfAttention(mesh, c_pair=128, num_head=4, transpose=True).transpose is True
+    assert nn.DistributeTransition(mesh, c_x=384, num_intermediate_factor=4).c_x == 384
+    assert nn.DistributeTransition(mesh, 128, 2).num_intermediate_factor == 2
+    assert nn.XSMMTriangleMultiplication(c_pair=128, _outgoing=False).c_equation == "kjc,kic->ijc"
+    blk = nn.DistributePairformerBlock(mesh, with_single=False)
+    assert not hasattr(blk, "single_attention_")
+    sa = nn.DistributeSelfAttention(mesh, c_x=384, num_head=16, use_single_cond=False, use_batch_infer=False)
+    assert sa.qkv_dim == 24
+    assert hasattr(sa, "load_xsmm_params") and hasattr(sa, "xsmm_forward")

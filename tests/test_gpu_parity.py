@@ -1,0 +1,368 @@
+"""GPU parity tests: the HIP path (through the C ABI) against the CPU oracle on
+the same seeded inputs and bf16-representable weights.
+
+Figures of merit (max |err| / RMS of the expected tensor):
+  * vs the bf16-EMULATING oracle (rounds where the kernels round): <= 1e-2, the
+    tolerance the north star states for bf16;
+  * vs the EXACT float64 oracle: reported, and bounded by 4e-2 (a chain of four
+    bf16 roundings of MFMA operands, each ~0.16% rms, reaches ~2e-2 at the 5-sigma
+    element of a million-element tensor; the bound documents that, it is not the
+    parity claim).
+Outputs are requested in fp32 so that the comparison is not dominated by the
+final rounding of the output dtype; bf16 outputs get one bf16 ulp of slack.
+"""
+
+import os
+import sys
+
+import pytest
+import torch
+
+from oracle import af3_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL_EMU = 1e-2
+TOL_EXACT = 4e-2
+D = torch.float64
+LOG = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out", "parity.log")
+
+
+def note(msg):
+    print(msg, flush=True)
+    try:
+        os.makedirs(os.path.dirname(LOG), exist_ok=True)
+        with open(LOG, "a") as f:
+            f.write(msg + "\n")
+    except OSError:
+        pass
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def rb(t):
+    return O.round_bf16(t)
+
+
+def rparams(p):
+    return {k: rb(v) for k, v in p.items()}
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def check(name, got, exact, emu, tol_emu=TOL_EMU, tol_exact=TOL_EXACT, bf16_out=False):
+    got = got.detach().float().cpu()
+    assert torch.isfinite(got).all(), f"{name}: non-finite output"
+    e_exact = O.rel_err(got, exact)
+    e_emu = O.rel_err(got, emu)
+    note(f"{name}: rel err vs bf16-emulating oracle {e_emu:.3e}, vs exact oracle {e_exact:.3e}")
+    if bf16_out:
+        # allow one bf16 ulp of the expected value on top of the tolerance
+        rms = float(torch.sqrt((emu.double() ** 2).mean()))
+        slack = tol_emu * rms + emu.abs().double() * 2.0 ** -7
+        assert ((got.double() - emu.double()).abs() <= slack).all(), f"{name}: bf16 output beyond 1 ulp + tol"
+    else:
+        assert e_emu <= tol_emu, f"{name}: {e_emu} vs emulating oracle"
+    assert e_exact <= tol_exact, f"{name}: {e_exact} vs exact oracle"
+
+
+def both(fn):
+    """(exact float64 result, bf16-emulating float64 result) of an oracle call."""
+    exact = fn()
+    with O.bf16_emulation():
+        emu = fn()
+    return exact, emu
+
+
+def seq_and_pair_mask(n, live):
+    seq = (torch.arange(n) < live).float()
+    return seq, seq[:, None] * seq[None, :]
+
+
+# ------------------------------------------------------------------ primitives
+@pytest.mark.parametrize("m,n,k", [(1, 8, 8), (100, 72, 40), (257, 130, 128), (384, 384, 768)])
+def test_linear_plain(gpu_pkg, m, n, k):
+    note(f"test_linear_plain m={m} n={n} k={k}")
+    g = gen(m + n + k)
+    x, w = rb(torch.randn(m, k, generator=g)), rb(torch.randn(n, k, generator=g) * 0.1)
+    b = torch.randn(n, generator=g)
+    got = gpu_pkg.ops.linear(x.to(dev()).bfloat16(), w.to(dev()).bfloat16(), bias=b.to(dev()),
+                             out_dtype=torch.float32, alpha=0.5)
+    want = (x.double() @ w.double().T + b.double()) * 0.5
+    assert O.rel_err(got.cpu(), want) < 1e-5
+    got = gpu_pkg.ops.linear(x.to(dev()).bfloat16(), w.to(dev()).bfloat16(), out_dtype=torch.float32, sigmoid=True)
+    assert O.rel_err(got.cpu(), torch.sigmoid(x.double() @ w.double().T)) < 1e-5
+
+
+def test_linear_swiglu_and_gate_res(gpu_pkg):
+    note("test_linear_swiglu_and_gate_res")
+    g = gen(3)
+    m, k, hidden = 70, 48, 96
+    x = rb(torch.randn(m, k, generator=g))
+    w1 = rb(torch.randn(2 * hidden, k, generator=g) * 0.2)
+    from distributed_xfold_amd.nn.base import pack_swiglu
+    h = gpu_pkg.ops.linear(x.to(dev()).bfloat16(), pack_swiglu(w1, 32).to(dev()).bfloat16(),
+                           mode=gpu_pkg.lib.LINEAR_SWIGLU)
+    y = x.double() @ w1.double().T
+    want = torch.nn.functional.silu(y[:, :hidden]) * y[:, hidden:]
+    assert O.rel_err(h.float().cpu(), want) < 1e-2
+    w2 = rb(torch.randn(40, hidden, generator=g) * 0.2)
+    gate = torch.rand(35, 40, generator=g)
+    res = torch.randn(m, 40, generator=g)
+    hb = rb(want.float())
+    out = gpu_pkg.ops.linear(hb.to(dev()).bfloat16(), w2.to(dev()).bfloat16(), out_dtype=torch.float32,
+                             mode=gpu_pkg.lib.LINEAR_GATE_RES, gate=gate.to(dev()), residual=res.to(dev()))
+    want2 = res.double() + gate.double().repeat(2, 1) * (hb.double() @ w2.double().T)
+    assert O.rel_err(out.cpu(), want2) < 1e-5
+
+
+@pytest.mark.parametrize("c", [16, 128, 384, 768])
+def test_layer_norm_and_adaln(gpu_pkg, c):
+    note(f"test_layer_norm_and_adaln c={c}")
+    g = gen(c)
+    x = torch.randn(3, 37, c, generator=g) * 2 + 0.5
+    w, b = torch.randn(c, generator=g), torch.randn(c, generator=g)
+    got = gpu_pkg.ops.layer_norm(x.to(dev()), w.to(dev()), b.to(dev()))
+    want = O.layer_norm(x.double(), w, b)
+    assert O.rel_err(got.float().cpu(), want) < 6e-3          # bf16 output rounding only
+    ss = torch.randn(37, 2 * c, generator=g).to(dev())
+    got = gpu_pkg.ops.layer_norm(x.to(dev()).bfloat16(), scale=ss[:, :c], shift=ss[:, c:])
+    xb = x.bfloat16().double()
+    want = torch.sigmoid(ss[:, :c].cpu().double()) * O.layer_norm(xb) + ss[:, c:].cpu().double()
+    assert O.rel_err(got.float().cpu(), want) < 6e-3
+
+
+# ----------------------------------------------------------------- pair path
+@pytest.mark.parametrize("rows,factor", [(300, 4), (128, 2), (1000, 4)])
+def test_transition128(gpu_pkg, rows, factor):
+    note(f"test_transition128 rows={rows} factor={factor}")
+    g = gen(rows)
+    p = rparams(O.make_transition_params(g, 128, factor))
+    x = rb(torch.randn(rows, 128, generator=g))
+    mod = gpu_pkg.nn.Transition(c_x=128, num_intermediate_factor=factor)
+    mod.load_state_dict(p)
+    mod.to(dev())
+    got = mod(x.to(dev()))
+    exact, emu = both(lambda: O.transition(x.double(), O.cast_params(p, D)))
+    check("transition128", got, exact, emu)
+    gotb = mod(x.to(dev()).bfloat16())
+    check("transition128[bf16 io]", gotb, exact, emu, bf16_out=True)
+
+
+@pytest.mark.parametrize("n,live,outgoing", [(37, 30, True), (37, 30, False), (130, 111, True), (130, 111, False),
+                                             (256, 256, True)])
+def test_triangle_multiplication(gpu_pkg, n, live, outgoing):
+    note(f"test_triangle_multiplication n={n} live={live} outgoing={outgoing}")
+    g = gen(n + int(outgoing))
+    p = rparams(O.make_triangle_multiplication_params(g))
+    pair = rb(torch.randn(n, n, 128, generator=g))
+    _, mask = seq_and_pair_mask(n, live)
+    if n == 37:     # a ragged, non-symmetric mask as the reference's kernel test draws (triangle_multiplication.py:143)
+        mask = (torch.rand(n, n, generator=g) > 0.2).float()
+    mod = gpu_pkg.nn.TriangleMultiplication(c_pair=128, _outgoing=outgoing)
+    mod.load_state_dict(p)
+    mod.to(dev())
+    got = mod(pair.to(dev()), mask.to(dev()))
+    exact, emu = both(lambda: O.triangle_multiplication(pair.double(), mask.double(), O.cast_params(p, D), outgoing))
+    check(f"trimul[{'out' if outgoing else 'in'}] n={n}", got, exact, emu)
+    gotb = mod(pair.to(dev()).bfloat16(), mask.to(dev()))
+    check(f"trimul[{'out' if outgoing else 'in'}] n={n} [bf16 io]", gotb, exact, emu, bf16_out=True)
+
+
+@pytest.mark.parametrize("n,live,transpose", [(37, 30, False), (37, 30, True), (130, 111, False), (130, 111, True),
+                                              (200, 200, False)])
+def test_grid_self_attention(gpu_pkg, n, live, transpose):
+    note(f"test_grid_self_attention n={n} live={live} transpose={transpose}")
+    g = gen(2 * n + int(transpose))
+    p = rparams(O.make_grid_self_attention_params(g, std=0.1))
+    pair = rb(torch.randn(n, n, 128, generator=g))
+    _, mask = seq_and_pair_mask(n, live)
+    if n == 37:
+        mask = (torch.rand(n, n, generator=g) > 0.2).float()
+        mask[:, 0] = 1
+    mod = gpu_pkg.nn.GridSelfAttention(c_pair=128, num_head=4, transpose=transpose)
+    mod.load_state_dict(p)
+    mod.to(dev())
+    got = mod(pair.to(dev()), mask.to(dev()))
+    exact, emu = both(lambda: O.grid_self_attention(pair.double(), mask.double(), O.cast_params(p, D), 4, transpose))
+    check(f"triattn[{'end' if transpose else 'start'}] n={n}", got, exact, emu)
+
+
+def test_grid_self_attention_masked_keys_are_exact(gpu_pkg):
+    """Masked keys must carry exactly zero weight: moving the value of a masked
+    key's pixel arbitrarily far changes no output outside that pixel's own row
+    entry (bit-exact), and a fully masked row is the uniform average."""
+    note("test_grid_self_attention_masked_keys_are_exact")
+    n = 48
+    g = gen(5)
+    p = rparams(O.make_grid_self_attention_params(g, std=0.1))
+    p["pair_bias_projection.weight"] = torch.zeros_like(p["pair_bias_projection.weight"])
+    pair = rb(torch.randn(n, n, 128, generator=g))
+    mask = torch.ones(n, n)
+    mask[:, 40:] = 0          # keys 40.. masked in every row
+    mask[7, :] = 0            # row 7 fully masked
+    mod = gpu_pkg.nn.GridSelfAttention(c_pair=128, num_head=4, transpose=False)
+    mod.load_state_dict(p)
+    mod.to(dev())
+    y1 = mod(pair.to(dev()), mask.to(dev())).cpu()
+    pair2 = pair.clone()
+    pair2[:, 40:] = rb(torch.randn(n, n - 40, 128, generator=g) * 50)
+    y2 = mod(pair2.to(dev()), mask.to(dev())).cpu()
+    rows = [r for r in range(n) if r != 7]
+    assert torch.equal(y1[rows][:, :40], y2[rows][:, :40])
+    exact = O.grid_self_attention(pair.double(), mask.double(), O.cast_params(p, D), 4, False)
+    assert O.rel_err(y1[7], exact[7]) < TOL_EXACT             # uniform over all 48 keys
+
+
+# ------------------------------------------------- single / diffusion attention
+@pytest.mark.parametrize("n,c,h,batch,cond", [(50, 384, 16, 0, False), (130, 768, 16, 3, True), (64, 128, 4, 2, True)])
+def test_self_attention(gpu_pkg, n, c, h, batch, cond):
+    note(f"test_self_attention n={n} c={c} h={h} batch={batch} cond={cond}")
+    g = gen(n + c)
+    cs = 384 if c != 128 else 128
+    p = rparams(O.make_self_attention_params(g, c, cs, cond, std=0.05))
+    x = rb(torch.randn(*((batch, n, c) if batch else (n, c)), generator=g))
+    s = rb(torch.randn(n, cs, generator=g)) if cond else None
+    mask = (torch.arange(n) < n - 5).float()
+    pl = torch.randn(h, n, n, generator=g)
+    mod = gpu_pkg.nn.SelfAttention(c_x=c, c_single_cond=cs, num_head=h, use_single_cond=cond,
+                                   use_batch_infer=bool(batch))
+    mod.load_state_dict(p)
+    mod.to(dev())
+    got = mod(x.to(dev()), mask.to(dev()), pl.to(dev()), None if s is None else s.to(dev()))
+    exact, emu = both(lambda: O.self_attention(x.double(), mask.double(), pl.double(),
+                                               None if s is None else s.double(), O.cast_params(p, D), h))
+    check(f"self_attention c={c}", got, exact, emu)
+
+
+def test_diffusion_transition_and_generic_transition(gpu_pkg):
+    note("test_diffusion_transition_and_generic_transition")
+    g = gen(77)
+    n, c, cs = 70, 768, 384
+    p = rparams(O.make_diffusion_transition_params(g, c, cs, 2, True, std=0.05))
+    x, s = rb(torch.randn(2, n, c, generator=g)), rb(torch.randn(n, cs, generator=g))
+    mod = gpu_pkg.nn.DiffusionTransition(c_x=c, c_single_cond=cs, use_single_cond=True)
+    mod.load_state_dict(p)
+    mod.to(dev())
+    got = mod(x.to(dev()), s.to(dev()))
+    exact, emu = both(lambda: O.diffusion_transition(x.double(), s.double(), O.cast_params(p, D)))
+    check("diffusion_transition", got, exact, emu)
+    p2 = rparams(O.make_transition_params(g, 384, 4, std=0.05))
+    xs = rb(torch.randn(n, 384, generator=g))
+    mod2 = gpu_pkg.nn.Transition(c_x=384)
+    mod2.load_state_dict(p2)
+    mod2.to(dev())
+    exact, emu = both(lambda: O.transition(xs.double(), O.cast_params(p2, D)))
+    check("transition c=384", mod2(xs.to(dev())), exact, emu)
+
+
+def test_cross_attention(gpu_pkg):
+    note("test_cross_attention")
+    g = gen(91)
+    B, S, Q, K, c, H = 2, 7, 32, 128, 128, 4
+    p = rparams(O.make_cross_attention_params(g, c, c, std=0.05))
+    xq, xk = rb(torch.randn(B, S, Q, c, generator=g)), rb(torch.randn(B, S, K, c, generator=g))
+    mq = torch.rand(S, Q, generator=g) > 0.2
+    mk = torch.rand(S, K, generator=g) > 0.2
+    pl = torch.randn(S, H, Q, K, generator=g)
+    cq, ck = rb(torch.randn(S, Q, c, generator=g)), rb(torch.randn(S, K, c, generator=g))
+    mod = gpu_pkg.nn.CrossAttention(num_head=H)
+    mod.load_state_dict(p)
+    mod.to(dev())
+    t = lambda a: a.to(dev())
+    got = mod(t(xq), t(xk), t(mq)[None], t(mk)[None], t(pl)[None], t(cq)[None], t(ck)[None])
+    fn = lambda dt: O.cross_attention(xq.to(dt), xk.to(dt), mq[None], mk[None], pl[None].to(dt),
+                                      cq[None].to(dt), ck[None].to(dt), O.cast_params(p, dt), H)
+    exact, emu = both(lambda: fn(D))
+    live = mq[None, :, :, None].expand(B, S, Q, c)
+    # live queries against the float64 oracle; padded queries follow fp32
+    # absorption of the +1e9 bias (uniform over padded keys), checked vs an fp32 run
+    check("cross_attention[live q]", got.cpu() * live, exact * live, emu * live)
+    ref32 = fn(torch.float32)
+    assert O.rel_err(got.cpu().float() * ~live, ref32 * ~live) < TOL_EXACT
+
+
+# ---------------------------------------------------------------------- blocks
+@pytest.mark.parametrize("n,live,io", [(64, 58, torch.float32), (100, 100, torch.bfloat16)])
+def test_pairformer_block(gpu_pkg, n, live, io):
+    note(f"test_pairformer_block n={n} live={live} io={io}")
+    g = gen(n)
+    p = rparams(O.make_pairformer_block_params(g))
+    pair, single = rb(torch.randn(n, n, 128, generator=g)), rb(torch.randn(n, 384, generator=g))
+    seq_mask, pair_mask = seq_and_pair_mask(n, live)
+    blk = gpu_pkg.nn.PairformerBlock()
+    blk.load_state_dict(p)
+    blk.to(dev())
+    gp, gs = blk(pair.to(dev()).to(io), pair_mask.to(dev()), single.to(dev()).to(io), seq_mask.to(dev()))
+    fn = lambda: O.pairformer_block(pair.double(), pair_mask.double(), single.double(), seq_mask.double(),
+                                    O.cast_params(p, D))
+    (ep, es), (mp, ms) = both(fn)
+    if io == torch.float32:
+        # compare the UPDATE (block output minus input), the harder target
+        check("pairformer_block pair update", gp.cpu() - pair, ep - pair.double(), mp - pair.double(), tol_emu=2e-2)
+        check("pairformer_block single update", gs.cpu() - single, es - single.double(), ms - single.double(),
+              tol_emu=2e-2)
+    else:
+        check("pairformer_block pair [bf16 io]", gp, ep, mp, bf16_out=True)
+        check("pairformer_block single [bf16 io]", gs, es, ms, bf16_out=True)
+
+
+def test_diffusion_transformer(gpu_pkg):
+    note("test_diffusion_transformer")
+    g = gen(123)
+    n, B, nb = 72, 2, 4
+    p = rparams(O.make_diffusion_transformer_params(g, num_blocks=nb, std=0.05))
+    act = rb(torch.randn(B, n, 768, generator=g))
+    s = rb(torch.randn(n, 384, generator=g))
+    pc = rb(torch.randn(n, n, 128, generator=g))
+    mask = (torch.arange(n) < n - 7).float()
+    mod = gpu_pkg.nn.DiffusionTransformer(num_blocks=nb, use_batch_infer=True)
+    mod.load_state_dict(p)
+    mod.to(dev())
+    got = mod(act.to(dev()).clone(), mask.to(dev()), s.to(dev()), pc.to(dev()))
+    exact, emu = both(lambda: O.diffusion_transformer(act.double(), mask.double(), s.double(), pc.double(),
+                                                      O.cast_params(p, D), 16, nb, 4))
+    check("diffusion_transformer update", got.cpu() - act, exact - act.double(), emu - act.double(), tol_emu=2e-2)
+
+
+def test_cross_att_transformer(gpu_pkg):
+    note("test_cross_att_transformer")
+    g = gen(321)
+    B, S, Q, K, c, cp = 2, 9, 32, 128, 128, 16
+    p = rparams(O.make_cross_att_transformer_params(g, std=0.05))
+    act = rb(torch.randn(B, S, Q, c, generator=g))
+    qm = torch.ones(S, Q, dtype=torch.bool)
+    qm[-1, 20:] = False
+    idx = torch.randint(0, (S - 1) * Q + 20, (S, K), generator=g)   # keys come from live atoms only
+    gm = torch.rand(S, K, generator=g) > 0.1
+    km = gm.clone()
+    cq, pc = rb(torch.randn(S, Q, c, generator=g)), rb(torch.randn(S, Q, K, cp, generator=g))
+    ck = rb(torch.randn(S, K, c, generator=g))
+    mod = gpu_pkg.nn.DiffusionCrossAttTransformer()
+    mod.load_state_dict(p)
+    mod.to(dev())
+    t = lambda a: a.to(dev())
+    got = mod(t(act).clone(), t(qm), (t(idx), t(gm)), t(km), t(cq), t(ck), t(pc))
+    exact, emu = both(lambda: O.cross_att_transformer(act.double(), qm, idx, gm, km, cq.double(), ck.double(),
+                                                      pc.double(), O.cast_params(p, D)))
+    live = qm[None, :, :, None].expand(B, S, Q, c)
+    # padded query atoms only ever feed themselves here; compare the live ones
+    check("cross_att_transformer update[live q]", (got.cpu() - act) * live, (exact - act.double()) * live,
+          (emu - act.double()) * live, tol_emu=2e-2)
+
+
+# --------------------------------------------------------------- error handling
+def test_cpu_tensor_is_rejected(gpu_pkg):
+    mod = gpu_pkg.nn.Transition(c_x=128).to(dev())
+    with pytest.raises(ValueError):
+        mod(torch.randn(4, 128))
+
+
+def test_bad_shape_is_rejected(gpu_pkg):
+    mod = gpu_pkg.nn.TriangleMultiplication().to(dev())
+    with pytest.raises(ValueError):
+        mod(torch.randn(8, 9, 128, device=dev()), torch.ones(8, 9, device=dev()))
