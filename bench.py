@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Benchmark of the Pairformer hot path on one MI355X.
+
+One "step" is one full Pairformer block (triangle multiplication out/in,
+triangle attention start/end, pair transition, pair-biased single attention,
+single transition) at N_token = 768, c_pair = 128, c_single = 384, bf16 residual
+stream, synthetic N(0,1) inputs resident in HBM, random-init weights N(0,0.02),
+last 10% of the tokens masked as padding.  Prints ONE JSON line:
+
+  metric / value   Pairformer ms per block (lower is better)
+  roofline         the dominant kernel (by time per block) against the MI355X
+                   dense bf16 MFMA peak, its launch timed live with HIP events
+  cpu_baseline     the CPU oracle (eager PyTorch restatement of the reference
+                   formulas, fp32) timed on this host's cores on a bounded
+                   sample, scaled to the metric's unit
+  per_op_ms / tflops_per_op   informational breakdown
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--n-token N]
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0
+
+
+def flops_trimul(n):      # one direction
+    return 256.0 * n ** 3 + 196608.0 * n ** 2
+
+
+def flops_triattn(n):     # one direction
+    return 512.0 * n ** 3 + 164864.0 * n ** 2
+
+
+def flops_block(n):
+    return (2 * flops_trimul(n) + 2 * flops_triattn(n) + 393216.0 * n ** 2
+            + 5632.0 * n ** 2 + 1474560.0 * n + 3538944.0 * n)
+
+
+def flops_contraction(n):     # the N x N x N contraction of 128 channels alone
+    return 256.0 * n ** 3
+
+
+def flops_attention_core(n):  # QK^T and PV for N rows x 4 heads x d=32
+    return 512.0 * n ** 3
+
+
+def gpu_time_ms(fn, iters, warmup=2):
+    """Average duration of fn() in ms, timed with HIP events on torch's current
+    stream (the stream handed to the C ABI)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def cpu_baseline(n_metric, budget_s=25.0):
+    """The CPU oracle on this host's cores: one Pairformer block, fp32, at the
+    largest of N in {128, 256, 384} that fits the time budget; scaled to the
+    metric's N by algorithmic FLOPs and flagged as such."""
+    import torch
+    from oracle import af3_oracle as O
+    g = torch.Generator().manual_seed(0)
+    p = O.make_pairformer_block_params(g)
+    threads = torch.get_num_threads()
+    measured = None
+    for n in (128, 256, 384):
+        if measured is not None:
+            est = measured[1] * flops_block(n) / flops_block(measured[0]) * 1.5
+            if est > budget_s:
+                break
+        pair, single = torch.randn(n, n, 128, generator=g), torch.randn(n, 384, generator=g)
+        seq = (torch.arange(n) < int(0.9 * n)).float()
+        pm = seq[:, None] * seq[None, :]
+        t0 = time.perf_counter()
+        with torch.no_grad():
+            O.pairformer_block(pair, pm, single, seq, p)
+        measured = (n, time.perf_counter() - t0)
+    n, secs = measured
+    scaled_ms = secs * 1e3 * flops_block(n_metric) / flops_block(n)
+    return {
+        "value": round(scaled_ms, 1), "unit": "ms/block", "cores": threads, "kind": "port",
+        "sample": (f"CPU oracle (eager PyTorch fp32 restatement of the reference formulas), one Pairformer "
+                   f"block at N={n}: {secs * 1e3:.0f} ms measured on {threads} threads; value is that time "
+                   f"scaled by algorithmic FLOPs to N={n_metric} (extrapolated)"),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--n-token", type=int, default=768)
+    ap.add_argument("--io", choices=["bf16", "f32"], default="bf16", help="dtype of the residual stream")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build keeps the whole pair tensor on ONE GPU (no sharding, no collectives); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    pkg.lib.load()                       # raises if the HIP library is missing
+    from oracle import af3_oracle as O   # parameter generator + CPU baseline only
+
+    dev = torch.device("cuda:0")
+    n = args.n_token
+    io = torch.bfloat16 if args.io == "bf16" else torch.float32
+    g = torch.Generator().manual_seed(0)
+    blk = pkg.nn.PairformerBlock()
+    blk.load_state_dict(O.make_pairformer_block_params(g))
+    blk = blk.to(dev)
+    blk.load_hip_params()
+    pair = torch.randn(n, n, 128, generator=g).to(dev).to(io)
+    single = torch.randn(n, 384, generator=g).to(dev).to(io)
+    seq_mask = (torch.arange(n) < int(0.9 * n)).float().to(dev)
+    pair_mask = (seq_mask[:, None] * seq_mask[None, :]).contiguous()
+
+    def step():
+        blk(pair, pair_mask, single, seq_mask)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    if not torch.isfinite(pair.float()).all():
+        raise RuntimeError("non-finite pair activations after the timed steps")
+
+    # ---- per-operator breakdown (untimed with respect to the headline) ----
+    it = max(3, min(args.steps, 10))
+    per_op = {
+        "trimul_out": gpu_time_ms(lambda: blk.triangle_multiplication_outgoing.run(pair, pair_mask, True), it),
+        "trimul_in": gpu_time_ms(lambda: blk.triangle_multiplication_incoming.run(pair, pair_mask, True), it),
+        "triattn_start": gpu_time_ms(lambda: blk.pair_attention1.run(pair, pair_mask, True), it),
+        "triattn_end": gpu_time_ms(lambda: blk.pair_attention2.run(pair, pair_mask, True), it),
+        "pair_transition": gpu_time_ms(lambda: blk.pair_transition.run(pair, True), it),
+    }
+    tflops_per_op = {
+        "trimul_out": flops_trimul(n) / per_op["trimul_out"] / 1e9,
+        "trimul_in": flops_trimul(n) / per_op["trimul_in"] / 1e9,
+        "triattn_start": flops_triattn(n) / per_op["triattn_start"] / 1e9,
+        "triattn_end": flops_triattn(n) / per_op["triattn_end"] / 1e9,
+        "pair_transition": 393216.0 * n * n / per_op["pair_transition"] / 1e9,
+    }
+
+    # ---- roofline of the dominant kernel, one launch timed with HIP events ----
+    npad = (n + 7) // 8 * 8
+    a = (torch.randn(128, n, npad, generator=g) * 0.1).to(dev).bfloat16()
+    b = (torch.randn(128, n, npad, generator=g) * 0.1).to(dev).bfloat16()
+    a[:, :, n:] = 0
+    b[:, :, n:] = 0
+    t_buf = torch.empty_like(a)
+    qkvg = (torch.randn(n * n, 512, generator=g) * 0.5).to(dev).bfloat16()
+    nb = torch.randn(4, n, n, generator=g).to(dev)
+    og = torch.empty((n * n, 128), dtype=torch.bfloat16, device=dev)
+    ms_contract = gpu_time_ms(lambda: pkg.ops.triangle_contraction(a, b, t_buf), it)
+    ms_attn = gpu_time_ms(lambda: pkg.ops.grid_attention_core(qkvg, nb, pair_mask, 4, og), it)
+    kernels = {
+        "gemm_nt_kernel (triangle contraction)": (ms_contract, flops_contraction(n)),
+        "flash_kernel (triangle attention core)": (ms_attn, flops_attention_core(n)),
+    }
+    dom = max(kernels, key=lambda k: kernels[k][0])      # each runs twice per block
+    dom_ms, dom_flops = kernels[dom]
+    achieved = dom_flops / dom_ms / 1e9
+    roofline = {
+        "kernel": dom, "bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+        "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+        "launch_ms": round(dom_ms, 4),
+        "others": {k: {"launch_ms": round(v[0], 4), "tflops": round(v[1] / v[0] / 1e9, 2)}
+                   for k, v in kernels.items() if k != dom},
+    }
+
+    out = {
+        "metric": "Pairformer ms/block at N=%d bf16" % n,
+        "value": round(ms_per_step, 4), "unit": "ms/block", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"one Pairformer block, N_token={n}, c_pair=128, c_single=384, "
+                               f"{args.io} residual stream, bf16 MFMA operands / fp32 accumulate, "
+                               "10% trailing tokens masked, random-init weights N(0,0.02)"},
+        "block_tflops": round(flops_block(n) / ms_per_step / 1e9, 2),
+        "per_op_ms": {k: round(v, 4) for k, v in per_op.items()},
+        "tflops_per_op": {k: round(v, 2) for k, v in tflops_per_op.items()},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(n)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

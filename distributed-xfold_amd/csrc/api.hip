@@ -315,4 +315,34 @@ int af3_linear_forward(
   return launch_gemm_nt(g, static_cast<hipStream_t>(stream));
 }
 
+// ------------------------------------------------------- kernel-level entry points
+int af3_triangle_contraction_forward(
+    const uint16_t* a, const uint16_t* b, uint16_t* t, int64_t n, af3_stream_t stream) {
+  if (!a || !b || !t || n <= 0 || n > 8192) return AF3_ERR_BAD_ARG;
+  const int64_t np = pad8(n);
+  GemmArgs g;
+  g.A = a; g.B = b; g.C = t;
+  g.M = g.N = (int)n; g.K = (int)np; g.batch = C_PAIR;
+  g.lda = g.ldb = g.ldc = np;
+  g.sA = g.sB = g.sC = n * np;
+  return launch_gemm_nt(g, static_cast<hipStream_t>(stream));
+}
+
+int af3_grid_attention_core_forward(
+    const uint16_t* qkvg, const float* pair_bias, const float* mask, uint16_t* og,
+    int64_t n, int num_head, af3_stream_t stream) {
+  if (!qkvg || !og || n <= 0 || n > 8192 || num_head <= 0 || C_PAIR % num_head) return AF3_ERR_BAD_ARG;
+  const int d = C_PAIR / num_head;
+  if (d != 32) return AF3_ERR_UNSUPPORTED;
+  FlashArgs f;
+  f.q = qkvg; f.k = qkvg + C_PAIR; f.v = qkvg + 2 * C_PAIR; f.g = qkvg + 3 * C_PAIR;
+  f.q_ss = f.k_ss = f.v_ss = f.g_ss = 4 * C_PAIR;
+  f.q_sb = f.k_sb = f.v_sb = f.g_sb = n * 4 * C_PAIR;
+  f.out = og; f.out_f32 = 0; f.o_ss = C_PAIR; f.o_sb = n * C_PAIR;
+  f.B = (int)n; f.H = num_head; f.Sq = f.Sk = (int)n; f.d = d;
+  f.bias = pair_bias; f.bias_sb = 0; f.bias_sh = n * n; f.bias_sq = n;
+  f.key_mask = mask; f.km_sb = n;
+  return launch_flash_attention(f, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

@@ -317,3 +317,42 @@ def linear(x, w, bias=None, out_dtype=torch.bfloat16, mode=_L.LINEAR_PLAIN, alph
                                 _stream(x.device))
     _L.check(rc, "af3_linear_forward")
     return out
+
+
+# ---------------------------------------------------------- kernel-level entries
+def triangle_contraction(a, b, out=None):
+    """t[c] = a[c] @ b[c].T for channel-major bf16 operands [128, N, ld], ld = N
+    rounded up to 8 with zero padding (the contraction stage alone)."""
+    lib = _L.load()
+    _gpu(a, "a", torch.bfloat16)
+    _gpu(b, "b", torch.bfloat16, a.shape)
+    if a.dim() != 3 or a.shape[0] != 128 or a.shape[2] != (a.shape[1] + 7) // 8 * 8:
+        raise ValueError("a: expected [128, N, roundup(N, 8)]")
+    if out is None:
+        out = torch.empty_like(a)
+    else:
+        _gpu(out, "out", torch.bfloat16, a.shape)
+    rc = lib.af3_triangle_contraction_forward(_p(a), _p(b), _p(out), a.shape[1], _stream(a.device))
+    _L.check(rc, "af3_triangle_contraction_forward")
+    return out
+
+
+def grid_attention_core(qkvg, pair_bias, mask, num_head, out=None):
+    """The flash-attention stage of the triangle attention on projected operands
+    qkvg [N*N, 512] bf16 -> gated output [N*N, 128] bf16."""
+    lib = _L.load()
+    _gpu(qkvg, "qkvg", torch.bfloat16)
+    if qkvg.dim() != 2 or qkvg.shape[1] != 512:
+        raise ValueError("qkvg: expected [N*N, 512]")
+    n = int(round(qkvg.shape[0] ** 0.5))
+    if n * n != qkvg.shape[0]:
+        raise ValueError("qkvg: row count must be a square")
+    if pair_bias is not None:
+        _gpu(pair_bias, "pair_bias", torch.float32, (num_head, n, n))
+    maskf = _mask_f32(mask, (n, n), "mask")
+    if out is None:
+        out = torch.empty((n * n, 128), dtype=torch.bfloat16, device=qkvg.device)
+    rc = lib.af3_grid_attention_core_forward(_p(qkvg), _p(pair_bias), _p(maskf), _p(out), n, int(num_head),
+                                             _stream(qkvg.device))
+    _L.check(rc, "af3_grid_attention_core_forward")
+    return out

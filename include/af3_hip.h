@@ -211,6 +211,28 @@ int af3_linear_forward(
     const float* gate, int64_t gate_rows,
     const void* residual, int res_dtype, af3_stream_t stream);
 
+/* ---------------------------------------------------------------------------
+ * Kernel-level entry points: the two MFMA-bound inner kernels on their own,
+ * so that a caller (the benchmark's roofline leg, a profiler) can time exactly
+ * one launch.  They are the inner stages of the operators above.
+ *
+ * af3_triangle_contraction_forward: t[c][i][j] = sum_k a[c][i][k] * b[c][j][k]
+ *   for 128 channels, the contraction stage of the triangle multiplication
+ *   (csrc/triangle_multiplication_bf16.h:257-401).  a, b, t are channel-major
+ *   bf16 [128][n_token][ld] with ld = n_token rounded up to 8; columns
+ *   n_token..ld-1 of a and b must be zero.
+ * af3_grid_attention_core_forward: the flash attention stage of the triangle
+ *   attention (csrc/grid_self_attention_bf16.h:226-481) on already projected
+ *   operands: qkvg [(b*N + s)][4*128] bf16 (q scaled | k | v | sigmoid gate),
+ *   pair bias [H][N][N] fp32 or NULL, key mask [N][N] fp32 0/1 or NULL,
+ *   og [(b*N + s)][128] bf16 = gate * softmax(q k^T + bias) v.
+ */
+int af3_triangle_contraction_forward(
+    const uint16_t* a, const uint16_t* b, uint16_t* t, int64_t n_token, af3_stream_t stream);
+int af3_grid_attention_core_forward(
+    const uint16_t* qkvg, const float* pair_bias, const float* mask, uint16_t* og,
+    int64_t n_token, int num_head, af3_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -143,3 +143,13 @@ def test_reference_constructor_signatures(pkg):
     sa = nn.DistributeSelfAttention(mesh, c_x=384, num_head=16, use_single_cond=False, use_batch_infer=False)
     assert sa.qkv_dim == 24
     assert hasattr(sa, "load_xsmm_params") and hasattr(sa, "xsmm_forward")
+
+
+def test_library_is_not_older_than_its_sources(pkg):
+    """A stale libaf3hip.so (sources edited, library not rebuilt) would make the
+    ctypes table and the binary disagree about argument lists."""
+    csrc = os.path.join(os.path.dirname(pkg.lib.LIB_PATH), "csrc")
+    so_time = os.path.getmtime(pkg.lib.LIB_PATH)
+    srcs = [os.path.join(csrc, f) for f in os.listdir(csrc) if f.endswith((".hip", ".h"))] + [HEADER]
+    stale = [os.path.basename(f) for f in srcs if os.path.getmtime(f) > so_time + 1]
+    assert not stale, f"rebuild libaf3hip.so (make -C {csrc}): newer sources {stale}"
