@@ -174,14 +174,17 @@ def main():
     a[:, :, n:] = 0
     b[:, :, n:] = 0
     t_buf = torch.empty_like(a)
-    qkvg = (torch.randn(n * n, 512, generator=g) * 0.5).to(dev).bfloat16()
-    nb = torch.randn(4, n, n, generator=g).to(dev)
+    q_, k_, g_ = ((torch.randn(n, 4, n, 32, generator=g) * 0.5).to(dev).bfloat16() for _ in range(3))
+    vt_ = (torch.randn(n, 4, 32, npad, generator=g) * 0.5).to(dev).bfloat16()
+    nb = torch.randn(4, n, npad, generator=g).to(dev).bfloat16()
+    vt_[..., n:] = 0
+    nb[..., n:] = 0
     og = torch.empty((n * n, 128), dtype=torch.bfloat16, device=dev)
     ms_contract = gpu_time_ms(lambda: pkg.ops.triangle_contraction(a, b, t_buf), it)
-    ms_attn = gpu_time_ms(lambda: pkg.ops.grid_attention_core(qkvg, nb, pair_mask, 4, og), it)
+    ms_attn = gpu_time_ms(lambda: pkg.ops.grid_attention_core(q_, k_, vt_, g_, nb, pair_mask, og), it)
     kernels = {
         "gemm_nt_kernel (triangle contraction)": (ms_contract, flops_contraction(n)),
-        "flash_kernel (triangle attention core)": (ms_attn, flops_attention_core(n)),
+        "triattn_flash_kernel (triangle attention core)": (ms_attn, flops_attention_core(n)),
     }
     dom = max(kernels, key=lambda k: kernels[k][0])      # each runs twice per block
     dom_ms, dom_flops = kernels[dom]

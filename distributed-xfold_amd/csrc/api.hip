@@ -95,9 +95,10 @@ int af3_triangle_multiplication_forward(
 // ------------------------------------------------------------ triangle attention
 size_t af3_grid_self_attn_workspace_bytes(int64_t n, int num_head) {
   if (n <= 0 || num_head <= 0) return 0;
+  // general path: qkvg + og + fp32 bias; fast path: q, k, g, vt planes + og + bf16 bias (smaller)
   return align_up((size_t)n * n * 4 * C_PAIR * sizeof(bf16_t), 256) +
          align_up((size_t)n * n * C_PAIR * sizeof(bf16_t), 256) +
-         align_up((size_t)num_head * n * n * sizeof(float), 256);
+         align_up((size_t)num_head * n * pad8(n) * sizeof(float), 256) + 4 * 256;
 }
 
 int af3_grid_self_attn_forward(
@@ -111,41 +112,66 @@ int af3_grid_self_attn_forward(
   if (w_pair_bias && nonbatched_bias) return AF3_ERR_BAD_ARG;
   if (misaligned(pair) || misaligned(out) || misaligned(mask) || misaligned(nonbatched_bias)) return AF3_ERR_BAD_ARG;
   const int d = C_PAIR / num_head;
-  if (d != 32) return AF3_ERR_UNSUPPORTED;
-  Carver ws(workspace, workspace_bytes);
-  bf16_t* qkvg = ws.take<bf16_t>((size_t)n * n * 4 * C_PAIR);
-  bf16_t* og = ws.take<bf16_t>((size_t)n * n * C_PAIR);
-  float* nb = ws.take<float>((size_t)num_head * n * n);
-  if (!ws.ok) return AF3_ERR_WORKSPACE;
+  if (d != 32 || num_head != 4) return AF3_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-
-  AttnProjArgs p;
-  p.pair = pair; p.io_f32 = io_dtype == AF3_F32; p.N = (int)n; p.transpose = transpose != 0;
-  p.ln_w = ln_w; p.ln_b = ln_b;
-  p.w_main = w_qkvg; p.n_chunks = 4;
-  p.chunk_ops = SEG_BIAS_SCALE | (SEG_PLAIN << 4) | (SEG_PLAIN << 8) | (SEG_SIGMOID << 12);
-  p.q_scale = 1.0f / sqrtf((float)d);
-  p.out_main = qkvg; p.ld_main = 4 * C_PAIR;
-  p.w_bias = w_pair_bias; p.n_bias = w_pair_bias ? num_head : 0; p.out_bias = nb;
-  p.skip_ln = ln_w == nullptr;
-  int rc = launch_attn_proj(p, s);
-  if (rc) return rc;
-
-  FlashArgs f;
-  f.q = qkvg; f.k = qkvg + C_PAIR; f.v = qkvg + 2 * C_PAIR; f.g = qkvg + 3 * C_PAIR;
-  f.q_ss = f.k_ss = f.v_ss = f.g_ss = 4 * C_PAIR;
-  f.q_sb = f.k_sb = f.v_sb = f.g_sb = n * 4 * C_PAIR;
-  f.out = og; f.out_f32 = 0; f.o_ss = C_PAIR; f.o_sb = n * C_PAIR;
-  f.B = (int)n; f.H = num_head; f.Sq = f.Sk = (int)n; f.d = d;
-  f.bias = w_pair_bias ? nb : nonbatched_bias;
-  f.bias_sb = 0; f.bias_sh = n * n; f.bias_sq = n;
-  f.key_mask = mask; f.km_sb = n;
-  rc = launch_flash_attention(f, s);
-  if (rc) return rc;
+  Carver ws(workspace, workspace_bytes);
+  bf16_t* og = nullptr;
+  int rc;
+  if (nonbatched_bias == nullptr) {
+    // Fast path: the pair bias (if any) is projected here, so everything the
+    // attention core needs is produced in its preferred form: base-2 logits,
+    // bf16 bias, head-major planes, V transposed.
+    const float LOG2E = 1.4426950408889634f;
+    const int64_t ldn = pad8(n);
+    bf16_t* q = ws.take<bf16_t>((size_t)n * n * C_PAIR);
+    bf16_t* k = ws.take<bf16_t>((size_t)n * n * C_PAIR);
+    bf16_t* g = ws.take<bf16_t>((size_t)n * n * C_PAIR);
+    bf16_t* vt = ws.take<bf16_t>((size_t)n * C_PAIR * ldn);
+    og = ws.take<bf16_t>((size_t)n * n * C_PAIR);
+    bf16_t* bias = ws.take<bf16_t>((size_t)num_head * n * ldn);
+    if (!ws.ok) return AF3_ERR_WORKSPACE;
+    TriAttnProjArgs p;
+    p.pair = pair; p.io_f32 = io_dtype == AF3_F32; p.N = (int)n; p.transpose = transpose != 0;
+    p.skip_ln = ln_w == nullptr; p.ln_w = ln_w; p.ln_b = ln_b;
+    p.w_qkvg = w_qkvg; p.w_bias = w_pair_bias; p.n_bias = w_pair_bias ? num_head : 0;
+    p.q_scale = LOG2E / sqrtf((float)d); p.bias_scale = LOG2E;
+    p.q = q; p.k = k; p.vt = vt; p.g = g; p.bias = bias; p.ldn = ldn;
+    rc = launch_triattn_proj(p, s);
+    if (rc) return rc;
+    TriAttnArgs t;
+    t.q = q; t.k = k; t.vt = vt; t.g = g; t.bias = w_pair_bias ? bias : nullptr;
+    t.mask = mask; t.og = og; t.N = (int)n; t.ldn = ldn;
+    rc = launch_triattn_flash(t, s);
+    if (rc) return rc;
+  } else {
+    // General path: an external fp32 bias [H][N][N] (operator-level contract).
+    bf16_t* qkvg = ws.take<bf16_t>((size_t)n * n * 4 * C_PAIR);
+    og = ws.take<bf16_t>((size_t)n * n * C_PAIR);
+    if (!ws.ok) return AF3_ERR_WORKSPACE;
+    AttnProjArgs p;
+    p.pair = pair; p.io_f32 = io_dtype == AF3_F32; p.N = (int)n; p.transpose = transpose != 0;
+    p.ln_w = ln_w; p.ln_b = ln_b; p.skip_ln = ln_w == nullptr;
+    p.w_main = w_qkvg; p.n_chunks = 4;
+    p.chunk_ops = SEG_BIAS_SCALE | (SEG_PLAIN << 4) | (SEG_PLAIN << 8) | (SEG_SIGMOID << 12);
+    p.q_scale = 1.0f / sqrtf((float)d);
+    p.out_main = qkvg; p.ld_main = 4 * C_PAIR;
+    rc = launch_attn_proj(p, s);
+    if (rc) return rc;
+    FlashArgs f;
+    f.q = qkvg; f.k = qkvg + C_PAIR; f.v = qkvg + 2 * C_PAIR; f.g = qkvg + 3 * C_PAIR;
+    f.q_ss = f.k_ss = f.v_ss = f.g_ss = 4 * C_PAIR;
+    f.q_sb = f.k_sb = f.v_sb = f.g_sb = n * 4 * C_PAIR;
+    f.out = og; f.out_f32 = 0; f.o_ss = C_PAIR; f.o_sb = n * C_PAIR;
+    f.B = (int)n; f.H = num_head; f.Sq = f.Sk = (int)n; f.d = d;
+    f.bias = nonbatched_bias; f.bias_sb = 0; f.bias_sh = n * n; f.bias_sq = n;
+    f.key_mask = mask; f.km_sb = n;
+    rc = launch_flash_attention(f, s);
+    if (rc) return rc;
+  }
 
   AttnOutArgs o;
   o.og = og; o.ld_og = C_PAIR; o.w_out = w_output; o.pair = pair; o.out = out;
-  o.io_f32 = p.io_f32; o.N = (int)n; o.transpose = p.transpose; o.residual = residual != 0;
+  o.io_f32 = io_dtype == AF3_F32; o.N = (int)n; o.transpose = transpose != 0; o.residual = residual != 0;
   return launch_attn_out(o, s);
 }
 
@@ -329,20 +355,13 @@ int af3_triangle_contraction_forward(
 }
 
 int af3_grid_attention_core_forward(
-    const uint16_t* qkvg, const float* pair_bias, const float* mask, uint16_t* og,
-    int64_t n, int num_head, af3_stream_t stream) {
-  if (!qkvg || !og || n <= 0 || n > 8192 || num_head <= 0 || C_PAIR % num_head) return AF3_ERR_BAD_ARG;
-  const int d = C_PAIR / num_head;
-  if (d != 32) return AF3_ERR_UNSUPPORTED;
-  FlashArgs f;
-  f.q = qkvg; f.k = qkvg + C_PAIR; f.v = qkvg + 2 * C_PAIR; f.g = qkvg + 3 * C_PAIR;
-  f.q_ss = f.k_ss = f.v_ss = f.g_ss = 4 * C_PAIR;
-  f.q_sb = f.k_sb = f.v_sb = f.g_sb = n * 4 * C_PAIR;
-  f.out = og; f.out_f32 = 0; f.o_ss = C_PAIR; f.o_sb = n * C_PAIR;
-  f.B = (int)n; f.H = num_head; f.Sq = f.Sk = (int)n; f.d = d;
-  f.bias = pair_bias; f.bias_sb = 0; f.bias_sh = n * n; f.bias_sq = n;
-  f.key_mask = mask; f.km_sb = n;
-  return launch_flash_attention(f, static_cast<hipStream_t>(stream));
+    const uint16_t* q, const uint16_t* k, const uint16_t* vt, const uint16_t* g,
+    const uint16_t* pair_bias, const float* mask, uint16_t* og, int64_t n, af3_stream_t stream) {
+  if (n <= 0 || n > 8192) return AF3_ERR_BAD_ARG;
+  TriAttnArgs t;
+  t.q = q; t.k = k; t.vt = vt; t.g = g; t.bias = pair_bias; t.mask = mask; t.og = og;
+  t.N = (int)n; t.ldn = pad8(n);
+  return launch_triattn_flash(t, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

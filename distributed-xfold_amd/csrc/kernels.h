@@ -74,7 +74,10 @@ struct AttnProjArgs {
   int64_t ld_main = 0;
   const bf16_t* w_bias = nullptr;  // [roundup(n_bias, 32)][128]
   int n_bias = 0;
-  float* out_bias = nullptr;       // [n_bias][N][N]
+  float* out_bias = nullptr;       // [n_bias][N][N] fp32, or
+  bf16_t* out_bias_bf16 = nullptr; // [n_bias][N][ld_bias] bf16 (values times bias_scale)
+  int64_t ld_bias = 0;
+  float bias_scale = 1.f;
 };
 int launch_attn_proj(const AttnProjArgs& a, hipStream_t s);
 
@@ -116,3 +119,29 @@ struct FlashArgs {
   int bias_mod = 0;  // > 0: bias, qpad and kpad are indexed by batch % bias_mod
 };
 int launch_flash_attention(const FlashArgs& a, hipStream_t stream);
+
+// ---------------------------------------------------------------- triattn.hip
+// Head-major scratch of the triangle-attention fast path (all bf16):
+//   q, k, g [b][h][s][32];  vt [b][h][32][ldn];  bias [h][q][ldn] (times log2 e, pad columns zero)
+struct TriAttnProjArgs {
+  const void* pair = nullptr;  // [N][N][128]
+  int io_f32 = 0, N = 0, transpose = 0, skip_ln = 0;
+  const float *ln_w = nullptr, *ln_b = nullptr;
+  const bf16_t* w_qkvg = nullptr;  // [4][128][128]
+  const bf16_t* w_bias = nullptr;  // [32][128], rows >= 4 zero
+  int n_bias = 0;                  // 0 or 4
+  float q_scale = 1.f, bias_scale = 1.f;
+  bf16_t *q = nullptr, *k = nullptr, *vt = nullptr, *g = nullptr, *bias = nullptr;
+  int64_t ldn = 0;
+};
+int launch_triattn_proj(const TriAttnProjArgs& a, hipStream_t stream);
+
+struct TriAttnArgs {
+  const bf16_t *q = nullptr, *k = nullptr, *vt = nullptr, *g = nullptr;
+  const bf16_t* bias = nullptr;  // or null
+  const float* mask = nullptr;   // [N][N] 0/1 or null
+  bf16_t* og = nullptr;          // [(b*N + s)][128]
+  int N = 0;
+  int64_t ldn = 0;
+};
+int launch_triattn_flash(const TriAttnArgs& a, hipStream_t stream);

@@ -21,181 +21,9 @@
 // pixel-major stores; the fragments are the same registers in both.
 #include "common.h"
 #include "kernels.h"
+#include "tile_common.h"
 
 namespace {
-
-constexpr int C = 128;    // pair channels
-constexpr int TM = 128;   // positions per tile
-constexpr int LDX = 136;  // LDS row stride (bf16) for [row][128] tiles: 272 B
-constexpr int LDS_F = 132;  // LDS row stride (fp32) for staged output tiles
-
-struct Tile {
-  int o, r0, N;
-  int64_t so, sr;  // pixel index = o * so + r * sr
-  __device__ __forceinline__ int64_t pix(int p) const { return (int64_t)o * so + (int64_t)(r0 + p) * sr; }
-  __device__ __forceinline__ bool valid(int p) const { return r0 + p < N; }
-};
-
-__device__ __forceinline__ Tile make_tile(int N, bool column_mode) {
-  const int tiles_r = (N + TM - 1) / TM;
-  Tile t;
-  t.N = N;
-  t.o = blockIdx.x / tiles_r;
-  t.r0 = (blockIdx.x % tiles_r) * TM;
-  t.so = column_mode ? 1 : N;
-  t.sr = column_mode ? N : 1;
-  return t;
-}
-
-// LayerNorm of a tile of pixels from global memory into sX[p][c] (bf16).
-// Thread (prow = tid / 16, chunk = tid % 16) handles channels 8*chunk..+7 of
-// pixels prow, prow + 16, ...; 16 lanes cooperate on one pixel's statistics.
-// Out-of-range pixels become zero rows.
-template <typename TIO>
-__device__ __forceinline__ void load_ln_tile(const TIO* x, const Tile& t, const float* lnw,
-                                             const float* lnb, bf16_t* sX, int tid, bool skip_ln = false) {
-  const int chunk = tid & 15, prow = tid >> 4;
-  float w[8], b[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    w[e] = lnw ? lnw[chunk * 8 + e] : 1.f;
-    b[e] = lnb ? lnb[chunk * 8 + e] : 0.f;
-  }
-  float v[8][8];
-#pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int p = it * 16 + prow;
-    if (t.valid(p)) {
-      Elem<TIO>::load8(x + t.pix(p) * C + chunk * 8, v[it]);
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[it][e] = 0.f;
-    }
-  }
-#pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int p = it * 16 + prow;
-    float s = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) s += v[it][e];
-    const float mean = group16_sum(s) * (1.f / C);
-    float q = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) { const float d = v[it][e] - mean; q += d * d; }
-    const float rstd = rsqrtf(group16_sum(q) * (1.f / C) + LN_EPS);
-    float o[8];
-    const bool ok = t.valid(p);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) o[e] = ok ? (skip_ln ? v[it][e] : (v[it][e] - mean) * rstd * w[e] + b[e]) : 0.f;
-    *reinterpret_cast<u32x4*>(sX + p * LDX + chunk * 8) = pack8(o);
-  }
-}
-
-// In-place LayerNorm of the rows of sX (bf16 in LDS), same thread mapping.
-__device__ __forceinline__ void ln_inplace_tile(bf16_t* sX, const float* lnw, const float* lnb, int tid) {
-  const int chunk = tid & 15, prow = tid >> 4;
-#pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int p = it * 16 + prow;
-    float v[8];
-    unpack8(*reinterpret_cast<const u32x4*>(sX + p * LDX + chunk * 8), v);
-    float s = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) s += v[e];
-    const float mean = group16_sum(s) * (1.f / C);
-    float q = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) { const float d = v[e] - mean; q += d * d; }
-    const float rstd = rsqrtf(group16_sum(q) * (1.f / C) + LN_EPS);
-    float o[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) o[e] = (v[e] - mean) * rstd * lnw[chunk * 8 + e] + lnb[chunk * 8 + e];
-    *reinterpret_cast<u32x4*>(sX + p * LDX + chunk * 8) = pack8(o);
-  }
-}
-
-// Copy `rows` x 128 bf16 weights (row-major, contiguous) into sW[row][LDX].
-__device__ __forceinline__ void load_w_rows(const bf16_t* gW, bf16_t* sW, int rows, int tid) {
-  for (int idx = tid; idx < rows * 16; idx += 256) {
-    const int row = idx >> 4, ch = idx & 15;
-    *reinterpret_cast<u32x4*>(sW + row * LDX + ch * 8) =
-        *reinterpret_cast<const u32x4*>(gW + row * C + ch * 8);
-  }
-}
-
-// The wave's 32 pixels as 8 k-step fragments (k = 128 channels).
-__device__ __forceinline__ void load_x_frags(const bf16_t* sX, int wave, int lane, bf16x8* xf) {
-#pragma unroll
-  for (int ks = 0; ks < 8; ++ks) xf[ks] = lds_frag(sX, LDX, wave * 32, ks * 16, lane);
-}
-
-// acc[nt] = tile nt (32 weight rows) of  X * W^T  (D form) or  W * X^T  (T form)
-template <bool TFORM, int NT>
-__device__ __forceinline__ void mfma_chunk(const bf16x8* xf, const bf16_t* sW, int lane, f32x16* acc) {
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[nt][r] = 0.f;
-#pragma unroll
-  for (int ks = 0; ks < 8; ++ks)
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const bf16x8 wf = lds_frag(sW, LDX, nt * 32, ks * 16, lane);
-      acc[nt] = TFORM ? mfma32(wf, xf[ks], acc[nt]) : mfma32(xf[ks], wf, acc[nt]);
-    }
-}
-
-// T-form accumulators (lane = pixel, 4 consecutive channels per register
-// quad) -> fp32 staging tile sS[px][LDS_F].
-__device__ __forceinline__ void stage_t_f32(const f32x16* acc, float* sS, int wave, int lane) {
-  const int px = wave * 32 + (lane & 31);
-#pragma unroll
-  for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int ch = nt * 32 + 8 * g + 4 * (lane >> 5);
-      f32x4 v = {acc[nt][4 * g], acc[nt][4 * g + 1], acc[nt][4 * g + 2], acc[nt][4 * g + 3]};
-      *reinterpret_cast<f32x4*>(sS + px * LDS_F + ch) = v;
-    }
-}
-
-// T-form accumulators -> bf16 staging tile sS[px][LDX]
-__device__ __forceinline__ void stage_t_bf16(const f32x16* acc, bf16_t* sS, int wave, int lane) {
-  const int px = wave * 32 + (lane & 31);
-#pragma unroll
-  for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int ch = nt * 32 + 8 * g + 4 * (lane >> 5);
-      u32x2 v;
-      v.x = pack2bf(acc[nt][4 * g], acc[nt][4 * g + 1]);
-      v.y = pack2bf(acc[nt][4 * g + 2], acc[nt][4 * g + 3]);
-      *reinterpret_cast<u32x2*>(sS + px * LDX + ch) = v;
-    }
-}
-
-// Staged fp32 tile -> residual stream: out[pix] = (res ? res[pix] : 0) + tile
-template <typename TIO>
-__device__ __forceinline__ void store_tile_f32(const float* sS, const Tile& t, TIO* out, const TIO* res, int tid) {
-  const int chunk = tid & 15, prow = tid >> 4;
-#pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int p = it * 16 + prow;
-    if (!t.valid(p)) continue;
-    float v[8];
-    const f32x4 a = *reinterpret_cast<const f32x4*>(sS + p * LDS_F + chunk * 8);
-    const f32x4 b = *reinterpret_cast<const f32x4*>(sS + p * LDS_F + chunk * 8 + 4);
-    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-    const int64_t off = t.pix(p) * C + chunk * 8;
-    if (res) {
-      float rr[8];
-      Elem<TIO>::load8(res + off, rr);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] += rr[e];
-    }
-    Elem<TIO>::store8(out + off, v);
-  }
-}
 
 // ============================================================================
 // triangle multiplication, prologue
@@ -374,10 +202,16 @@ __global__ __launch_bounds__(256) void attn_proj_kernel(AttnProjArgs a) {
     const int p = wave * 32 + (lane & 31);
     if (t.valid(p)) {
       const int64_t pixel = t.pix(p);  // = q * N + k
+      const int q = (int)(pixel / a.N), k = (int)(pixel % a.N);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int h = h0 + acc_row(r, lane);
-        if (h < a.n_bias) a.out_bias[(int64_t)h * a.N * a.N + pixel] = acc[0][r];
+        if (h < a.n_bias) {
+          if (a.out_bias_bf16)
+            a.out_bias_bf16[((int64_t)h * a.N + q) * a.ld_bias + k] = f2bf(acc[0][r] * a.bias_scale);
+          else
+            a.out_bias[(int64_t)h * a.N * a.N + pixel] = acc[0][r];
+        }
       }
     }
     __syncthreads();
@@ -523,7 +357,8 @@ int launch_trimul_epilogue(const TriMulArgs& a, hipStream_t s) {
 int launch_attn_proj(const AttnProjArgs& a, hipStream_t s) {
   if (a.N <= 0 || !a.pair || a.n_chunks < 0 || a.n_chunks > 4 || a.n_bias < 0) return AF3_ERR_BAD_ARG;
   if (a.n_chunks > 0 && (!a.w_main || !a.out_main || (a.ld_main & 7) || a.ld_main < a.n_chunks * C)) return AF3_ERR_BAD_ARG;
-  if (a.n_bias > 0 && (!a.w_bias || !a.out_bias)) return AF3_ERR_BAD_ARG;
+  if (a.n_bias > 0 && (!a.w_bias || (!a.out_bias && !a.out_bias_bf16))) return AF3_ERR_BAD_ARG;
+  if (a.out_bias_bf16 && a.ld_bias < a.N) return AF3_ERR_BAD_ARG;
   if (!aligned16(a.pair) || !aligned16(a.w_main) || !aligned16(a.out_main) || !aligned16(a.w_bias)) return AF3_ERR_BAD_ARG;
   return a.io_f32 ? launch_tiles(attn_proj_kernel<float>, a, a.N, a.N, s)
                   : launch_tiles(attn_proj_kernel<bf16_t>, a, a.N, a.N, s);

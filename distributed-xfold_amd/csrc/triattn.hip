@@ -1,0 +1,348 @@
+// Triangle attention, the fast path: projection kernel + flash kernel that
+// share a head-major scratch layout.
+//
+// Scratch layout (bf16), for rows b of the (possibly transposed) operator:
+//   Q, K, G : [b][h][s][32]          one 4 KB-contiguous slab per 64 positions
+//   Vt      : [b][h][32][ldn]        V transposed (keys contiguous), ldn = N up to 8
+//   bias    : [h][q][ldn]            pair bias * log2(e); columns N..ldn-1 are zero
+// so every tile the flash kernel stages is a run of full 16-byte chunks with no
+// transposition and no boundary code.
+//
+// Flash kernel: same wave-level scheme as attention.hip (S^T = K Q^T so a lane
+// owns one query; bf16 probabilities feed O^T += V^T P^T directly), plus
+//   * exponentials in base 2 (log2(e) folded into q and the bias upstream);
+//   * the pair bias is the INITIAL VALUE of the MFMA accumulator;
+//   * the key mask rides in the matrix product: K gets a 33rd column holding 0,
+//     -1e9 (masked key) or -inf (tile padding) and Q a matching 1.0.  A masked
+//     logit is bias + q.k - 1e9, which fp32 rounds to -1e9 for every key alike:
+//     masked keys get weight exactly 0 and a fully masked row is uniform, as
+//     with the reference's additive 1e9 * (mask - 1);
+//   * workgroup ids are remapped so that each XCD (ids are dealt round-robin to
+//     the 8 XCDs) walks a contiguous range of (head, row, query-tile): the six
+//     query tiles that share one row's K/V, and the head's bias, stay in that
+//     XCD's L2.
+#include "common.h"
+#include "kernels.h"
+#include "tile_common.h"
+
+namespace {
+
+constexpr int H = 4, D = 32;
+
+// ============================================================================
+// projections: LN -> q (scaled), k, sigmoid gate (position-major) and v
+// (channel-major), + pair-bias heads
+// ============================================================================
+template <typename TIO>
+__global__ __launch_bounds__(256, 2) void triattn_proj_kernel(TriAttnProjArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t sX[TM * LDX];  // LN tile, then staging
+  __shared__ __attribute__((aligned(16))) bf16_t sW[TM * LDX];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // (b, s) = (o, r): for the transposed operator a tile is a column segment
+  const Tile t = make_tile(a.N, a.transpose != 0);
+  const TIO* x = reinterpret_cast<const TIO*>(a.pair);
+  load_w_rows(a.w_qkvg, sW, TM, tid);
+  load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0);
+  __syncthreads();
+  bf16x8 xf[8];
+  load_x_frags(sX, wave, lane, xf);
+  __syncthreads();  // sX is free from here on: it becomes the staging tile
+
+  const int64_t bh0 = (int64_t)t.o * H;  // (b * H + h) for h = 0
+  // chunk order q, k, v, g as packed in w_qkvg; v takes the channel-major route.
+  // Two 32-row weight tiles at a time keep the live accumulators at 32 registers.
+#pragma unroll 1
+  for (int chunk = 0; chunk < 4; ++chunk) {
+#pragma unroll
+    for (int pairt = 0; pairt < 2; ++pairt) {
+      f32x16 acc[2];
+      if (chunk == 2) {
+        // v: D form, lane owns channel (lane & 31) of a tile, registers walk pixels
+        mfma_chunk<false, 2>(xf, sW + pairt * 64 * LDX, lane, acc);
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+          const int ch = (pairt * 2 + nt) * 32 + (lane & 31);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int p0 = wave * 32 + 8 * g + 4 * (lane >> 5);
+            u32x2 pk;
+            pk.x = pack2bf(acc[nt][4 * g], acc[nt][4 * g + 1]);
+            pk.y = pack2bf(acc[nt][4 * g + 2], acc[nt][4 * g + 3]);
+            *reinterpret_cast<u32x2*>(sX + ch * LDX + p0) = pk;
+          }
+        }
+      } else {
+        mfma_chunk<true, 2>(xf, sW + pairt * 64 * LDX, lane, acc);
+        const int px = wave * 32 + (lane & 31);
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float y = acc[nt][4 * g + e];
+              v[e] = chunk == 0 ? y * a.q_scale : (chunk == 3 ? sigmoidf_(y) : y);
+            }
+            const int ch = (pairt * 2 + nt) * 32 + 8 * g + 4 * (lane >> 5);
+            u32x2 pk;
+            pk.x = pack2bf(v[0], v[1]);
+            pk.y = pack2bf(v[2], v[3]);
+            *reinterpret_cast<u32x2*>(sX + px * LDX + ch) = pk;
+          }
+      }
+    }
+    __syncthreads();  // staging visible; every wave is done with sW
+    if (chunk == 2) {
+      // Vt[(b*H + h)*32 + d][s]: per channel 128 consecutive positions
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int idx = tid + 256 * i, ch = idx >> 4, pc = idx & 15;
+        const int r = t.r0 + pc * 8;
+        if (r < a.ldn)
+          *reinterpret_cast<u32x4*>(a.vt + (bh0 * D + ch) * a.ldn + r) =
+              *reinterpret_cast<const u32x4*>(sX + ch * LDX + pc * 8);
+      }
+    } else {
+      bf16_t* plane = chunk == 0 ? a.q : (chunk == 1 ? a.k : a.g);
+      const int ck = tid & 15, prow = tid >> 4;
+      const int h = ck >> 2, part = ck & 3;
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const int p = it * 16 + prow;
+        if (t.valid(p))
+          *reinterpret_cast<u32x4*>(plane + ((bh0 + h) * a.N + t.r0 + p) * D + part * 8) =
+              *reinterpret_cast<const u32x4*>(sX + p * LDX + ck * 8);
+      }
+    }
+    // next weights straight into sW (every wave passed the barrier above, so sW is free)
+    if (chunk < 3) load_w_rows(a.w_qkvg + (int64_t)(chunk + 1) * TM * C, sW, TM, tid);
+    else if (a.n_bias > 0) load_w_rows(a.w_bias, sW, 32, tid);
+    __syncthreads();
+  }
+
+  // pair-bias heads (T form: lane = pixel, rows = heads): bias[h][q][k] with
+  // (q, k) the pixel's own (row, col) in the un-transposed pair tensor
+  if (a.n_bias > 0) {
+    f32x16 acc[1];
+    mfma_chunk<true, 1>(xf, sW, lane, acc);
+    if ((lane >> 5) == 0) {  // heads 0..3 are accumulator rows 0..3: registers 0..3 of the low half
+      const int p = wave * 32 + lane;
+      const int r = t.r0 + p;
+      if (!a.transpose) {
+        // q = o, k = r: consecutive lanes write consecutive keys; pad columns get zeros
+        if (r < a.ldn) {
+#pragma unroll
+          for (int h = 0; h < H; ++h)
+            a.bias[((int64_t)h * a.N + t.o) * a.ldn + r] = f2bf(t.valid(p) ? acc[0][h] * a.bias_scale : 0.f);
+        }
+      } else if (t.valid(p)) {
+        // q = r, k = o
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+          bf16_t* row = a.bias + ((int64_t)h * a.N + r) * a.ldn;
+          row[t.o] = f2bf(acc[0][h] * a.bias_scale);
+          if (t.o == a.N - 1)
+            for (int k = a.N; k < a.ldn; ++k) row[k] = 0;
+        }
+      }
+    }
+  }
+}
+
+// ============================================================================
+// flash attention core
+// ============================================================================
+constexpr int KT = 64;       // keys per LDS tile
+constexpr int LDK = 56;      // sK row: 32 head-dim + 16 mask k-step + 8 pad (bf16); 112 B
+constexpr int LDV = KT + 4;  // sVt / sB row: 136 B = 34 dwords, so 32 lanes' 8-byte reads hit 32 bank pairs
+constexpr int QW = 128;      // queries per workgroup
+constexpr uint32_t BF16_ONE = 0x3F80u, BF16_NEG_INF = 0xFF80u, BF16_NEG_1E9 = 0xCE6Eu;
+
+__global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t sK[2][KT * LDK];
+  __shared__ __attribute__((aligned(16))) bf16_t sVt[2][D * LDV];
+  __shared__ __attribute__((aligned(16))) bf16_t sB[2][QW * LDV];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int hh = lane >> 5, j = lane & 31;
+  const int N = a.N;
+  const int QT = (N + QW - 1) / QW;
+  // XCD-aware remap: physical id -> (xcd, slot) -> logical id; logical order is
+  // (head, row, query tile) with the query tile fastest.
+  const int total = H * N * QT;
+  const int per_xcd = (total + 7) / 8;
+  const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (logical >= total) return;
+  const int qt = logical % QT;
+  const int b = (logical / QT) % N;
+  const int h = logical / (QT * N);
+  const int q0 = qt * QW;
+  const int qw = q0 + wave * 32 + j;
+  const int qi = min(qw, N - 1);
+  const int64_t bh = (int64_t)b * H + h;
+
+  bf16x8 qf[3];
+  {
+    const bf16_t* qp = a.q + (bh * N + qi) * D + 8 * hh;
+    qf[0] = as_frag(*reinterpret_cast<const u32x4*>(qp));
+    qf[1] = as_frag(*reinterpret_cast<const u32x4*>(qp + 16));
+    u32x4 one = {hh == 0 ? BF16_ONE : 0u, 0u, 0u, 0u};
+    qf[2] = as_frag(one);
+  }
+
+  // loaders, one 16-byte chunk each per tile:
+  //   K   thread (key = tid / 4, c = tid % 4)            + the mask k-step by c < 2
+  //   Vt  thread (d = tid / 8, kc = tid % 8)
+  //   bias: four chunks, idx = tid + 256 i -> (q = idx / 8, kc = idx % 8)
+  const int k_key = tid >> 2, k_c = tid & 3;
+  const int v_d = tid >> 3, v_kc = (tid & 7) * 8;
+  const bf16_t* kbase = a.k + bh * N * D;
+  const bf16_t* vbase = a.vt + (bh * D + v_d) * a.ldn + v_kc;
+  const float* mrow = a.mask ? a.mask + (int64_t)b * N : nullptr;
+  const bf16_t* bias_h = a.bias ? a.bias + (int64_t)h * N * a.ldn : nullptr;
+  u32x4 rk, rv, rb[4];
+  uint32_t rmask;
+  auto gload = [&](int k0) {
+    const u32x4 z = {0, 0, 0, 0};
+    const int key = k0 + k_key;
+    rk = z;
+    rmask = BF16_NEG_INF;
+    if (key < N) {
+      rk = *reinterpret_cast<const u32x4*>(kbase + (int64_t)key * D + k_c * 8);
+      rmask = (mrow && mrow[key] == 0.f) ? BF16_NEG_1E9 : 0u;
+    }
+    rv = (k0 + v_kc < a.ldn) ? *reinterpret_cast<const u32x4*>(vbase + k0) : z;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + 256 * i, q = q0 + (idx >> 3), kc = k0 + (idx & 7) * 8;
+      rb[i] = (bias_h && q < N && kc < a.ldn) ? *reinterpret_cast<const u32x4*>(bias_h + (int64_t)q * a.ldn + kc) : z;
+    }
+  };
+  auto sstore = [&](int buf) {
+    *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + k_c * 8]) = rk;
+    if (k_c < 2) {
+      u32x4 m = {k_c == 0 ? rmask : 0u, 0u, 0u, 0u};
+      *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + 32 + k_c * 8]) = m;
+    }
+    // rows of sVt / sB are 8-byte aligned only: two 8-byte stores per chunk
+    u32x2* pv = reinterpret_cast<u32x2*>(&sVt[buf][v_d * LDV + v_kc]);
+    pv[0] = u32x2{rv.x, rv.y};
+    pv[1] = u32x2{rv.z, rv.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + 256 * i;
+      u32x2* pb = reinterpret_cast<u32x2*>(&sB[buf][(idx >> 3) * LDV + (idx & 7) * 8]);
+      pb[0] = u32x2{rb[i].x, rb[i].y};
+      pb[1] = u32x2{rb[i].z, rb[i].w};
+    }
+  };
+
+  f32x16 o;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) o[r] = 0.f;
+  float m_run = -__builtin_huge_valf(), l_run = 0.f;
+
+  const int nkt = (N + KT - 1) / KT;
+  gload(0);
+  sstore(0);
+  __syncthreads();
+
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nkt) gload((kt + 1) * KT);
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      if (kt * KT + sub * 32 >= N) break;  // uniform across the workgroup
+      // accumulator starts as the pair bias: s[4g + e] <-> key 8g + 4hh + e of this sub-tile
+      f32x16 s;
+      const bf16_t* bp = &sB[buf][(wave * 32 + j) * LDV + sub * 32 + 4 * hh];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const u32x2 w = *reinterpret_cast<const u32x2*>(bp + 8 * g);
+        s[4 * g] = bflo(w.x); s[4 * g + 1] = bfhi(w.x); s[4 * g + 2] = bflo(w.y); s[4 * g + 3] = bfhi(w.y);
+      }
+#pragma unroll
+      for (int ks = 0; ks < 3; ++ks)
+        s = mfma32(lds_frag(sK[buf], LDK, sub * 32, ks * 16, lane), qf[ks], s);
+
+      float mx = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+#pragma unroll
+      for (int g = 1; g < 4; ++g) mx = fmaxf(mx, fmaxf(fmaxf(s[4 * g], s[4 * g + 1]), fmaxf(s[4 * g + 2], s[4 * g + 3])));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      m_run = m_new;
+      float psum = 0.f;
+      bf16x8 pf[2];
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        float pv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          pv[e] = __builtin_amdgcn_exp2f(s[8 * half + e] - m_new);
+          psum += pv[e];
+        }
+        pf[half] = as_frag(pack8(pv));
+      }
+      l_run = l_run * alpha + psum;
+      if (__any(alpha != 1.f)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[r] *= alpha;
+      }
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const bf16_t* vp = &sVt[buf][j * LDV + sub * 32 + 16 * half + 4 * hh];
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(vp);
+        const u32x2 hi = *reinterpret_cast<const u32x2*>(vp + 8);
+        u32x4 vv;
+        vv.x = lo.x; vv.y = lo.y; vv.z = hi.x; vv.w = hi.y;
+        o = mfma32(as_frag(vv), pf[half], o);
+      }
+    }
+    if (kt + 1 < nkt) sstore(buf ^ 1);
+    __syncthreads();
+  }
+
+  const float inv = 1.f / (l_run + __shfl_xor(l_run, 32));
+  if (qw >= N) return;
+  const bf16_t* gp = a.g + (bh * N + qw) * D + 4 * hh;
+  bf16_t* op = a.og + ((int64_t)b * N + qw) * 128 + h * D + 4 * hh;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const u32x2 gw = *reinterpret_cast<const u32x2*>(gp + 8 * g);
+    u32x2 w;
+    w.x = pack2bf(o[4 * g] * inv * bflo(gw.x), o[4 * g + 1] * inv * bfhi(gw.x));
+    w.y = pack2bf(o[4 * g + 2] * inv * bflo(gw.y), o[4 * g + 3] * inv * bfhi(gw.y));
+    *reinterpret_cast<u32x2*>(op + 8 * g) = w;
+  }
+}
+
+bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+}  // namespace
+
+int launch_triattn_proj(const TriAttnProjArgs& a, hipStream_t stream) {
+  if (a.N <= 0 || !a.pair || !a.w_qkvg || !a.q || !a.k || !a.vt || !a.g) return AF3_ERR_BAD_ARG;
+  if (a.ldn < a.N || (a.ldn & 7)) return AF3_ERR_BAD_ARG;
+  if (a.n_bias != 0 && (a.n_bias != H || !a.w_bias || !a.bias)) return AF3_ERR_BAD_ARG;
+  if (!al16(a.pair) || !al16(a.w_qkvg) || !al16(a.w_bias) || !al16(a.q) || !al16(a.k) || !al16(a.vt) ||
+      !al16(a.g) || !al16(a.bias))
+    return AF3_ERR_BAD_ARG;
+  const int64_t tiles = (int64_t)a.N * ((a.N + TM - 1) / TM);
+  if (tiles > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  if (a.io_f32) hipLaunchKernelGGL(triattn_proj_kernel<float>, dim3((unsigned)tiles), dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL(triattn_proj_kernel<bf16_t>, dim3((unsigned)tiles), dim3(256), 0, stream, a);
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+int launch_triattn_flash(const TriAttnArgs& a, hipStream_t stream) {
+  if (!a.q || !a.k || !a.vt || !a.g || !a.og || a.N <= 0) return AF3_ERR_BAD_ARG;
+  if (a.ldn < a.N || (a.ldn & 7)) return AF3_ERR_BAD_ARG;
+  if (!al16(a.q) || !al16(a.k) || !al16(a.vt) || !al16(a.g) || !al16(a.og) || !al16(a.bias)) return AF3_ERR_BAD_ARG;
+  const int64_t total = (int64_t)((a.N + QW - 1) / QW) * H * a.N;
+  const int64_t blocks = (total + 7) / 8 * 8;
+  if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  hipLaunchKernelGGL(triattn_flash_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}

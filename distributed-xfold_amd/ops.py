@@ -337,22 +337,27 @@ def triangle_contraction(a, b, out=None):
     return out
 
 
-def grid_attention_core(qkvg, pair_bias, mask, num_head, out=None):
-    """The flash-attention stage of the triangle attention on projected operands
-    qkvg [N*N, 512] bf16 -> gated output [N*N, 128] bf16."""
+def grid_attention_core(q, k, vt, g, pair_bias, mask, out=None):
+    """The flash-attention stage of the triangle attention on projected, head-major
+    bf16 operands in base-2 form: q, k, g [N, 4, N, 32] (q and the bias
+    pre-multiplied by log2(e); g = sigmoid gate), vt [N, 4, 32, ld], pair_bias
+    [4, N, ld] or None, ld = N rounded up to 8 with zero padding.  Returns the
+    gated output [N*N, 128] bf16."""
     lib = _L.load()
-    _gpu(qkvg, "qkvg", torch.bfloat16)
-    if qkvg.dim() != 2 or qkvg.shape[1] != 512:
-        raise ValueError("qkvg: expected [N*N, 512]")
-    n = int(round(qkvg.shape[0] ** 0.5))
-    if n * n != qkvg.shape[0]:
-        raise ValueError("qkvg: row count must be a square")
+    _gpu(q, "q", torch.bfloat16)
+    if q.dim() != 4 or q.shape[1] != 4 or q.shape[3] != 32 or q.shape[0] != q.shape[2]:
+        raise ValueError("q: expected [N, 4, N, 32]")
+    n = q.shape[0]
+    ld = (n + 7) // 8 * 8
+    _gpu(k, "k", torch.bfloat16, q.shape)
+    _gpu(g, "g", torch.bfloat16, q.shape)
+    _gpu(vt, "vt", torch.bfloat16, (n, 4, 32, ld))
     if pair_bias is not None:
-        _gpu(pair_bias, "pair_bias", torch.float32, (num_head, n, n))
+        _gpu(pair_bias, "pair_bias", torch.bfloat16, (4, n, ld))
     maskf = _mask_f32(mask, (n, n), "mask")
     if out is None:
-        out = torch.empty((n * n, 128), dtype=torch.bfloat16, device=qkvg.device)
-    rc = lib.af3_grid_attention_core_forward(_p(qkvg), _p(pair_bias), _p(maskf), _p(out), n, int(num_head),
-                                             _stream(qkvg.device))
+        out = torch.empty((n * n, 128), dtype=torch.bfloat16, device=q.device)
+    rc = lib.af3_grid_attention_core_forward(_p(q), _p(k), _p(vt), _p(g), _p(pair_bias), _p(maskf), _p(out), n,
+                                             _stream(q.device))
     _L.check(rc, "af3_grid_attention_core_forward")
     return out

@@ -223,15 +223,19 @@ int af3_linear_forward(
  *   n_token..ld-1 of a and b must be zero.
  * af3_grid_attention_core_forward: the flash attention stage of the triangle
  *   attention (csrc/grid_self_attention_bf16.h:226-481) on already projected
- *   operands: qkvg [(b*N + s)][4*128] bf16 (q scaled | k | v | sigmoid gate),
- *   pair bias [H][N][N] fp32 or NULL, key mask [N][N] fp32 0/1 or NULL,
- *   og [(b*N + s)][128] bf16 = gate * softmax(q k^T + bias) v.
+ *   operands, bf16, head-major, in base-2 form (4 heads of 32, ld = n_token
+ *   rounded up to 8):
+ *     q  [b][h][s][32] = query * log2(e)/sqrt(32);  k, g [b][h][s][32] (g = sigmoid gate);
+ *     vt [b][h][32][ld] = value transposed, columns n_token..ld-1 zero;
+ *     pair_bias [h][q][ld] = bias * log2(e), pad columns zero, or NULL;
+ *   key mask [N][N] fp32 0/1 or NULL;
+ *   og [(b*N + s)][128] = gate * softmax(q k^T + bias) v.
  */
 int af3_triangle_contraction_forward(
     const uint16_t* a, const uint16_t* b, uint16_t* t, int64_t n_token, af3_stream_t stream);
 int af3_grid_attention_core_forward(
-    const uint16_t* qkvg, const float* pair_bias, const float* mask, uint16_t* og,
-    int64_t n_token, int num_head, af3_stream_t stream);
+    const uint16_t* q, const uint16_t* k, const uint16_t* vt, const uint16_t* g,
+    const uint16_t* pair_bias, const float* mask, uint16_t* og, int64_t n_token, af3_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -236,7 +236,7 @@ def grid_self_attention(pair, mask, p: Params, num_head: int, transpose: bool,
         full_pair = pair
     w, b = p["act_norm.weight"], p["act_norm.bias"]
     x = _r(layer_norm(pair, w, b))
-    nb = linear(_r(layer_norm(full_pair, w, b)), p["pair_bias_projection.weight"])
+    nb = _r(linear(_r(layer_norm(full_pair, w, b)), p["pair_bias_projection.weight"]))
     nb = nb.permute(2, 0, 1)                                         # [H, Q, K]
     if transpose:
         x = x.permute(1, 0, 2)

@@ -401,3 +401,47 @@ def test_bad_shape_is_rejected(gpu_pkg):
     mod = gpu_pkg.nn.TriangleMultiplication().to(dev())
     with pytest.raises(ValueError):
         mod(torch.randn(8, 9, 128, device=dev()), torch.ones(8, 9, device=dev()))
+
+
+# ---------------------------------------------------------- kernel-level entries
+@pytest.mark.parametrize("n", [70, 256])
+def test_kernel_level_contraction(gpu_pkg, n):
+    note(f"test_kernel_level_contraction n={n}")
+    g = gen(n)
+    npad = (n + 7) // 8 * 8
+    a = torch.zeros(128, n, npad)
+    b = torch.zeros(128, n, npad)
+    a[:, :, :n] = rb(torch.randn(128, n, n, generator=g))
+    b[:, :, :n] = rb(torch.randn(128, n, n, generator=g))
+    t = gpu_pkg.ops.triangle_contraction(a.to(dev()).bfloat16(), b.to(dev()).bfloat16())
+    want = torch.bmm(a.double(), b.double().transpose(1, 2))
+    assert_within_bf16_ulp("contraction", t[:, :, :n], want, ulps=1.01, atol=1e-3)
+
+
+@pytest.mark.parametrize("n", [40, 200])
+def test_kernel_level_attention_core(gpu_pkg, n):
+    """Base-2 operands in, gate * softmax(q k^T + bias, masked) v out."""
+    note(f"test_kernel_level_attention_core n={n}")
+    g = gen(n)
+    log2e = 1.4426950408889634
+    npad = (n + 7) // 8 * 8
+    qkvg = rb(torch.randn(n, n, 4, 4, 32, generator=g) * 0.7)       # [b, s, (q k v g), h, d]
+    qkvg[:, :, 3] = torch.sigmoid(qkvg[:, :, 3]).bfloat16().float()
+    bias = torch.zeros(4, n, npad)
+    bias[:, :, :n] = rb(torch.randn(4, n, n, generator=g))
+    mask = (torch.rand(n, n, generator=g) > 0.2).float()
+    mask[:, 0] = 1
+    mask[3, :] = 0                                                  # one fully masked row
+    hm = lambda i: qkvg[:, :, i].permute(0, 2, 1, 3).contiguous()       # [b, h, s, d]
+    vt = torch.zeros(n, 4, 32, npad)
+    vt[..., :n] = hm(2).transpose(-1, -2)
+    t = lambda x: x.to(dev()).bfloat16()
+    og = gpu_pkg.ops.grid_attention_core(t(hm(0)), t(hm(1)), t(vt), t(hm(3)), t(bias), mask.to(dev()))
+    q, k, v, gt = (qkvg[:, :, i].permute(0, 2, 1, 3).double() for i in range(4))   # [b, h, s, d]
+    logits = (q @ k.transpose(-1, -2) + bias[None, :, :, :n].double()) / log2e
+    logits = logits.masked_fill(mask[:, None, None, :] == 0, -1e9)
+    want = (torch.softmax(logits, -1) @ v) * gt
+    want = want.permute(0, 2, 1, 3).reshape(n * n, 128)
+    e_max, e_rms = _errs(og.float().cpu(), want)
+    note(f"attention core n={n}: max {e_max:.3e} rms {e_rms:.3e}")
+    assert e_rms < 5e-3 and e_max < 4e-2                            # bf16 probabilities and output
