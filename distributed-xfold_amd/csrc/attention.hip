@@ -96,7 +96,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
   };
   // V^T rows that no chunk covers (head dim padding) must read as zero
   for (int idx = tid; idx < 2 * DVT * 32 * LDV; idx += NT) (&sVt[0][0])[idx] = 0;
-  __syncthreads();
+  lds_barrier();
 
   f32x16 o[DVT];
 #pragma unroll
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
   const int nkt = (a.Sk + KT - 1) / KT;
   gload(0);
   sstore(0);
-  __syncthreads();
+  lds_barrier();
 
   for (int kt = 0; kt < nkt; ++kt) {
     const int buf = kt & 1;
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
         }
     }
     if (kt + 1 < nkt) sstore(buf ^ 1);
-    __syncthreads();
+    lds_barrier();
   }
 
   const float l_tot = l_run + __shfl_xor(l_run, 32);

@@ -125,4 +125,13 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits
+// for every outstanding global load and STORE of the wave (vmcnt(0)), which
+// exposes the full HBM write latency at each barrier of a kernel that streams
+// results out while it keeps computing.  None of the kernels here passes data
+// between threads through global memory, so waiting for LDS alone is enough.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 #define LN_EPS 1e-5f

@@ -70,7 +70,7 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(GemmArgs g) {
   const int nk = (g.K + BK - 1) / BK;
   gload(0);
   sstore(0);
-  __syncthreads();
+  lds_barrier();
 
   for (int kt = 0; kt < nk; ++kt) {
     const int buf = kt & 1;
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(GemmArgs g) {
         for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(fa[i], fb[j], acc[i][j]);
     }
     if (kt + 1 < nk) sstore(buf ^ 1);
-    __syncthreads();
+    lds_barrier();
   }
 
   // ---------------------------------------------------------------- epilogue

@@ -29,8 +29,8 @@ namespace {
 // triangle multiplication, prologue
 // ============================================================================
 template <typename TIO>
-__global__ __launch_bounds__(256) void trimul_prologue_kernel(TriMulArgs a) {
-  __shared__ __attribute__((aligned(16))) bf16_t sX[TM * LDX];
+__global__ __launch_bounds__(256, 2) void trimul_prologue_kernel(TriMulArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t sX[TM * LDX];  // LN tile, then the [64 ch][px] staging tile
   __shared__ __attribute__((aligned(16))) bf16_t sW[TM * LDX];
   __shared__ float sMask[TM];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -39,19 +39,24 @@ __global__ __launch_bounds__(256) void trimul_prologue_kernel(TriMulArgs a) {
   const Tile t = make_tile(a.N, !a.outgoing);
   const TIO* x = reinterpret_cast<const TIO*>(a.pair);
 
+  WChunkRegs wr;
+  wr.load(a.w_pg, tid);
   if (tid < TM) sMask[tid] = (t.valid(tid) ? (a.mask ? a.mask[t.pix(tid)] : 1.f) : 0.f);
   load_ln_tile<TIO>(x, t, a.ln_in_w, a.ln_in_b, sX, tid);
-  __syncthreads();
+  wr.store(sW, tid);
+  lds_barrier();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
+  lds_barrier();  // sX is free from here on
 
   // weight chunks: [P(64 ch) | G(64 ch)] for a ch 0-63, a ch 64-127, b ch 0-63, b ch 64-127
+#pragma unroll 1
   for (int chunk = 0; chunk < 4; ++chunk) {
-    load_w_rows(a.w_pg + (int64_t)chunk * TM * C, sW, TM, tid);
-    __syncthreads();
+    // request the next weights before this chunk's stores go out (vector
+    // memory operations retire in order)
+    if (chunk < 3) wr.load(a.w_pg + (int64_t)(chunk + 1) * TM * C, tid);
     f32x16 acc[4];
     mfma_chunk<false, 4>(xf, sW, lane, acc);
-    __syncthreads();  // sW is free: reuse it as the [64 ch][LDX px] staging tile
     // D form: lane owns channel (lane & 31) of tiles 0/1 (P) and 2/3 (G)
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
@@ -66,19 +71,21 @@ __global__ __launch_bounds__(256) void trimul_prologue_kernel(TriMulArgs a) {
         u32x2 pk;
         pk.x = pack2bf(v[0], v[1]);
         pk.y = pack2bf(v[2], v[3]);
-        *reinterpret_cast<u32x2*>(sW + ch * LDX + p0) = pk;
+        *reinterpret_cast<u32x2*>(sX + ch * LDX + p0) = pk;
       }
     }
-    __syncthreads();
+    lds_barrier();  // staging visible; every wave is done with sW
+    if (chunk < 3) wr.store(sW, tid);
     bf16_t* dst = (chunk < 2 ? a.a_buf : a.b_buf) + ((int64_t)(chunk & 1) * 64 * a.N + t.o) * a.Np;
-    for (int idx = tid; idx < 64 * 16; idx += 256) {
-      const int ch = idx >> 4, pc = idx & 15;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + 256 * i, ch = idx >> 4, pc = idx & 15;
       const int r = t.r0 + pc * 8;
       if (r < a.Np)
         *reinterpret_cast<u32x4*>(dst + (int64_t)ch * a.N * a.Np + r) =
-            *reinterpret_cast<const u32x4*>(sW + ch * LDX + pc * 8);
+            *reinterpret_cast<const u32x4*>(sX + ch * LDX + pc * 8);
     }
-    __syncthreads();
+    lds_barrier();
   }
 }
 
@@ -86,7 +93,7 @@ __global__ __launch_bounds__(256) void trimul_prologue_kernel(TriMulArgs a) {
 // triangle multiplication, epilogue
 // ============================================================================
 template <typename TIO>
-__global__ __launch_bounds__(256) void trimul_epilogue_kernel(TriMulArgs a) {
+__global__ __launch_bounds__(256, 2) void trimul_epilogue_kernel(TriMulArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t smem[2 * TM * LDX];
   bf16_t* sX = smem;
   bf16_t* sW = smem + TM * LDX;
@@ -96,10 +103,24 @@ __global__ __launch_bounds__(256) void trimul_epilogue_kernel(TriMulArgs a) {
   const Tile t = make_tile(a.N, false);
   const TIO* x = reinterpret_cast<const TIO*>(a.pair);
 
+  // everything this tile needs from memory is requested up front
+  WChunkRegs wr;
+  wr.load(a.w_gl, tid);
+  u32x4 rt[8];  // contraction result t[c][i][j0 + 8 pc ..], c = 16 it + tid / 16
+  const int pc = tid & 15, crow = tid >> 4;
+  const int nvalid = min(max(a.N - (t.r0 + pc * 8), 0), 8);
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int c = it * 16 + crow;
+    const u32x4 z = {0, 0, 0, 0};
+    rt[it] = nvalid > 0 ? *reinterpret_cast<const u32x4*>(a.t_buf + ((int64_t)c * a.N + t.o) * a.Np + t.r0 + pc * 8) : z;
+  }
+
   // 1. output gate from the LayerNorm-ed input: sigmoid(LN(x) Wgl^T), T form, kept in registers
   load_ln_tile<TIO>(x, t, a.ln_in_w, a.ln_in_b, sX, tid);
-  load_w_rows(a.w_gl, sW, TM, tid);
-  __syncthreads();
+  wr.store(sW, tid);
+  wr.load(a.w_out, tid);
+  lds_barrier();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
   f32x16 gate[4];
@@ -108,31 +129,24 @@ __global__ __launch_bounds__(256) void trimul_epilogue_kernel(TriMulArgs a) {
   for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) gate[nt][r] = sigmoidf_(gate[nt][r]);
-  __syncthreads();
+  lds_barrier();
 
-  // 2. contraction result t[c][i][j0..] -> sX[j][c], then center LayerNorm
-  {
-    const int pc = tid & 15, crow = tid >> 4;
-    const int nvalid = min(max(a.N - (t.r0 + pc * 8), 0), 8);
+  // 2. contraction result -> sX[j][c] (transposed), then center LayerNorm
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      const int c = it * 16 + crow;
-      u32x4 raw = {0, 0, 0, 0};
-      if (nvalid > 0)
-        raw = *reinterpret_cast<const u32x4*>(a.t_buf + ((int64_t)c * a.N + t.o) * a.Np + t.r0 + pc * 8);
-      const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
+  for (int it = 0; it < 8; ++it) {
+    const int c = it * 16 + crow;
+    const uint32_t w4[4] = {rt[it].x, rt[it].y, rt[it].z, rt[it].w};
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        bf16_t h = (bf16_t)((e & 1) ? (w4[e >> 1] >> 16) : (w4[e >> 1] & 0xffffu));
-        if (e >= nvalid) h = 0;
-        sX[(pc * 8 + e) * LDX + c] = h;
-      }
+    for (int e = 0; e < 8; ++e) {
+      bf16_t h = (bf16_t)((e & 1) ? (w4[e >> 1] >> 16) : (w4[e >> 1] & 0xffffu));
+      if (e >= nvalid) h = 0;
+      sX[(pc * 8 + e) * LDX + c] = h;
     }
   }
-  load_w_rows(a.w_out, sW, TM, tid);
-  __syncthreads();
+  wr.store(sW, tid);
+  lds_barrier();
   ln_inplace_tile(sX, a.ln_c_w, a.ln_c_b, tid);
-  __syncthreads();
+  lds_barrier();
   load_x_frags(sX, wave, lane, xf);
   f32x16 acc[4];
   mfma_chunk<true, 4>(xf, sW, lane, acc);
@@ -140,9 +154,9 @@ __global__ __launch_bounds__(256) void trimul_epilogue_kernel(TriMulArgs a) {
   for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[nt][r] *= gate[nt][r];
-  __syncthreads();
+  lds_barrier();
   stage_t_f32(acc, sS, wave, lane);
-  __syncthreads();
+  lds_barrier();
   store_tile_f32<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), a.residual ? x : nullptr, tid);
 }
 
@@ -150,7 +164,7 @@ __global__ __launch_bounds__(256) void trimul_epilogue_kernel(TriMulArgs a) {
 // triangle attention: projections
 // ============================================================================
 template <typename TIO>
-__global__ __launch_bounds__(256) void attn_proj_kernel(AttnProjArgs a) {
+__global__ __launch_bounds__(256, 2) void attn_proj_kernel(AttnProjArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t sX[TM * LDX];
   __shared__ __attribute__((aligned(16))) bf16_t sW[TM * LDX];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -158,13 +172,13 @@ __global__ __launch_bounds__(256) void attn_proj_kernel(AttnProjArgs a) {
   const Tile t = make_tile(a.N, a.transpose != 0);
   const TIO* x = reinterpret_cast<const TIO*>(a.pair);
   load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0);
-  __syncthreads();
+  lds_barrier();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
 
   for (int chunk = 0; chunk < a.n_chunks; ++chunk) {
     load_w_rows(a.w_main + (int64_t)chunk * TM * C, sW, TM, tid);
-    __syncthreads();
+    lds_barrier();
     f32x16 acc[4];
     mfma_chunk<true, 4>(xf, sW, lane, acc);
     const int op = (a.chunk_ops >> (4 * chunk)) & 15;
@@ -179,9 +193,9 @@ __global__ __launch_bounds__(256) void attn_proj_kernel(AttnProjArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[nt][r] = sigmoidf_(acc[nt][r]);
     }
-    __syncthreads();
+    lds_barrier();
     stage_t_bf16(acc, sW, wave, lane);
-    __syncthreads();
+    lds_barrier();
     const int ck = tid & 15, prow = tid >> 4;
 #pragma unroll
     for (int it = 0; it < 8; ++it) {
@@ -190,13 +204,13 @@ __global__ __launch_bounds__(256) void attn_proj_kernel(AttnProjArgs a) {
         *reinterpret_cast<u32x4*>(a.out_main + ((int64_t)t.o * a.N + t.r0 + p) * a.ld_main + chunk * C + ck * 8) =
             *reinterpret_cast<const u32x4*>(sW + p * LDX + ck * 8);
     }
-    __syncthreads();
+    lds_barrier();
   }
 
   // pair-bias heads: out_bias[h][q][k] with (q, k) the pixel's own (row, col)
   for (int h0 = 0; h0 < a.n_bias; h0 += 32) {
     load_w_rows(a.w_bias + (int64_t)h0 * C, sW, 32, tid);  // host pads w_bias to a multiple of 32 rows
-    __syncthreads();
+    lds_barrier();
     f32x16 acc[1];
     mfma_chunk<true, 1>(xf, sW, lane, acc);
     const int p = wave * 32 + (lane & 31);
@@ -214,7 +228,7 @@ __global__ __launch_bounds__(256) void attn_proj_kernel(AttnProjArgs a) {
         }
       }
     }
-    __syncthreads();
+    lds_barrier();
   }
 }
 
@@ -241,14 +255,14 @@ __global__ __launch_bounds__(256) void attn_out_kernel(AttnOutArgs a) {
     }
   }
   load_w_rows(a.w_out, sW, TM, tid);
-  __syncthreads();
+  lds_barrier();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
   f32x16 acc[4];
   mfma_chunk<true, 4>(xf, sW, lane, acc);
-  __syncthreads();
+  lds_barrier();
   stage_t_f32(acc, sS, wave, lane);
-  __syncthreads();
+  lds_barrier();
   store_tile_f32<TIO>(sS, t, reinterpret_cast<TIO*>(a.out),
                       a.residual ? reinterpret_cast<const TIO*>(a.pair) : nullptr, tid);
 }
@@ -259,7 +273,7 @@ __global__ __launch_bounds__(256) void attn_out_kernel(AttnOutArgs a) {
 constexpr int LDW2 = 72;  // LDS row stride (bf16) of a [128 out][64 hidden] W2 slab
 
 template <typename TIO>
-__global__ __launch_bounds__(256) void transition_kernel(TransitionArgs a) {
+__global__ __launch_bounds__(256, 2) void transition_kernel(TransitionArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t smem[2 * TM * LDX];
   bf16_t* sX = smem;              // phase 0: LN tile;   later: W1 slab [128][LDX]
   bf16_t* sW1 = smem;
@@ -269,10 +283,10 @@ __global__ __launch_bounds__(256) void transition_kernel(TransitionArgs a) {
   const Tile t = make_tile(a.N, false);
   const TIO* x = reinterpret_cast<const TIO*>(a.x);
   load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid);
-  __syncthreads();
+  lds_barrier();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
-  __syncthreads();
+  lds_barrier();
 
   f32x16 out[4];
 #pragma unroll
@@ -281,16 +295,33 @@ __global__ __launch_bounds__(256) void transition_kernel(TransitionArgs a) {
     for (int r = 0; r < 16; ++r) out[nt][r] = 0.f;
 
   const int n_slabs = a.hidden / 64;
-  for (int hs = 0; hs < n_slabs; ++hs) {
-    // W1 slab: 64 "a" rows then the 64 matching "b" rows (host-packed), K = 128
-    load_w_rows(a.w1 + (int64_t)hs * 128 * C, sW1, 128, tid);
-    // W2 slab: all 128 output rows, hidden columns 64*hs .. +63
-    for (int idx = tid; idx < 128 * 8; idx += 256) {
-      const int row = idx >> 3, ck = idx & 7;
-      *reinterpret_cast<u32x4*>(sW2 + row * LDW2 + ck * 8) =
-          *reinterpret_cast<const u32x4*>(a.w2 + (int64_t)row * a.hidden + hs * 64 + ck * 8);
+  // Slab hs of W1 (64 "a" rows then the 64 matching "b" rows, host-packed, K = 128)
+  // and of W2 (all 128 output rows, hidden columns 64 hs .. +63) are fetched
+  // into registers one slab ahead, so their latency hides behind the MFMAs.
+  WChunkRegs w1r;
+  u32x4 w2r[4];
+  auto fetch = [&](int hs) {
+    w1r.load(a.w1 + (int64_t)hs * 128 * C, tid);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + 256 * i;
+      w2r[i] = *reinterpret_cast<const u32x4*>(a.w2 + (int64_t)(idx >> 3) * a.hidden + hs * 64 + (idx & 7) * 8);
     }
-    __syncthreads();
+  };
+  auto commit = [&]() {
+    w1r.store(sW1, tid);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + 256 * i;
+      *reinterpret_cast<u32x4*>(sW2 + (idx >> 3) * LDW2 + (idx & 7) * 8) = w2r[i];
+    }
+  };
+  fetch(0);
+  commit();
+  lds_barrier();
+#pragma unroll 1
+  for (int hs = 0; hs < n_slabs; ++hs) {
+    if (hs + 1 < n_slabs) fetch(hs + 1);
     // GEMM1, T form: acc[0..1] = a^T (64 hidden x 32 px), acc[2..3] = b^T
     f32x16 acc[4];
     mfma_chunk<true, 4>(xf, sW1, lane, acc);
@@ -320,10 +351,14 @@ __global__ __launch_bounds__(256) void transition_kernel(TransitionArgs a) {
         }
       }
     }
-    __syncthreads();
+    lds_barrier();  // every wave is done with this slab
+    if (hs + 1 < n_slabs) {
+      commit();
+      lds_barrier();
+    }
   }
   stage_t_f32(out, sS, wave, lane);
-  __syncthreads();
+  lds_barrier();
   store_tile_f32<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), a.residual ? x : nullptr, tid);
 }
 

@@ -41,18 +41,31 @@ __global__ __launch_bounds__(256, 2) void triattn_proj_kernel(TriAttnProjArgs a)
   // (b, s) = (o, r): for the transposed operator a tile is a column segment
   const Tile t = make_tile(a.N, a.transpose != 0);
   const TIO* x = reinterpret_cast<const TIO*>(a.pair);
-  load_w_rows(a.w_qkvg, sW, TM, tid);
+  WChunkRegs wr;
+  wr.load(a.w_qkvg, tid);
   load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0);
-  __syncthreads();
+  wr.store(sW, tid);
+  lds_barrier();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
-  __syncthreads();  // sX is free from here on: it becomes the staging tile
+  lds_barrier();  // sX is free from here on: it becomes the staging tile
 
   const int64_t bh0 = (int64_t)t.o * H;  // (b * H + h) for h = 0
   // chunk order q, k, v, g as packed in w_qkvg; v takes the channel-major route.
   // Two 32-row weight tiles at a time keep the live accumulators at 32 registers.
 #pragma unroll 1
   for (int chunk = 0; chunk < 4; ++chunk) {
+    // The next weights are requested BEFORE this chunk's results are stored:
+    // vector memory operations retire in order, so a load issued behind the
+    // stores would make its consumer wait for the stores' round trip to HBM.
+    if (chunk < 3) wr.load(a.w_qkvg + (int64_t)(chunk + 1) * TM * C, tid);
+    else if (a.n_bias > 0) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int idx = tid + 256 * i;
+        wr.r[i] = *reinterpret_cast<const u32x4*>(a.w_bias + (idx >> 4) * C + (idx & 15) * 8);
+      }
+    }
 #pragma unroll
     for (int pairt = 0; pairt < 2; ++pairt) {
       f32x16 acc[2];
@@ -92,7 +105,15 @@ __global__ __launch_bounds__(256, 2) void triattn_proj_kernel(TriAttnProjArgs a)
           }
       }
     }
-    __syncthreads();  // staging visible; every wave is done with sW
+    lds_barrier();  // staging visible; every wave is done with sW
+    if (chunk < 3) wr.store(sW, tid);
+    else if (a.n_bias > 0) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int idx = tid + 256 * i;
+        *reinterpret_cast<u32x4*>(sW + (idx >> 4) * LDX + (idx & 15) * 8) = wr.r[i];
+      }
+    }
     if (chunk == 2) {
       // Vt[(b*H + h)*32 + d][s]: per channel 128 consecutive positions
 #pragma unroll
@@ -115,10 +136,7 @@ __global__ __launch_bounds__(256, 2) void triattn_proj_kernel(TriAttnProjArgs a)
               *reinterpret_cast<const u32x4*>(sX + p * LDX + ck * 8);
       }
     }
-    // next weights straight into sW (every wave passed the barrier above, so sW is free)
-    if (chunk < 3) load_w_rows(a.w_qkvg + (int64_t)(chunk + 1) * TM * C, sW, TM, tid);
-    else if (a.n_bias > 0) load_w_rows(a.w_bias, sW, 32, tid);
-    __syncthreads();
+    lds_barrier();
   }
 
   // pair-bias heads (T form: lane = pixel, rows = heads): bias[h][q][k] with
@@ -246,7 +264,7 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
   const int nkt = (N + KT - 1) / KT;
   gload(0);
   sstore(0);
-  __syncthreads();
+  lds_barrier();
 
   for (int kt = 0; kt < nkt; ++kt) {
     const int buf = kt & 1;
@@ -301,7 +319,7 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
       }
     }
     if (kt + 1 < nkt) sstore(buf ^ 1);
-    __syncthreads();
+    lds_barrier();
   }
 
   const float inv = 1.f / (l_run + __shfl_xor(l_run, 32));
