@@ -36,6 +36,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hh = lane >> 5, j = lane & 31;
+  const int xaddr = half_swap_addr();
   // blockIdx.x = (q_tile * H + head) * B + batch: workgroups in flight together
   // share one (head, q-tile) slab of the pair bias across many batch rows.
   const int b = blockIdx.x % a.B;
@@ -162,7 +163,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
       float mx = s[0];
 #pragma unroll
       for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      mx = fmaxf(mx, half_swap(xaddr, mx));
       const float m_new = fmaxf(m_run, mx);
       const float alpha = __expf(m_run - m_new);  // 0 on the first tile (m_run = -inf, m_new finite)
       m_run = m_new;
@@ -207,7 +208,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
     lds_barrier();
   }
 
-  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float l_tot = l_run + half_swap(xaddr, l_run);
   const float inv = 1.f / l_tot;
   if (!q_ok) return;
   // o[t][4g + e] = out(query j, head-dim 32t + 8g + 4hh + e)

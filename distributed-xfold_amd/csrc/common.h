@@ -81,7 +81,12 @@ template <> struct Elem<float> {
   static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
 };
 
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// sigmoid through the hardware exp2 / reciprocal (about 1 ulp each): four
+// instructions instead of the ~15 of an IEEE division.  exp2 overflows to +inf
+// for very negative x and rcp(inf) = 0, as it should.
+__device__ __forceinline__ float sigmoidf_(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
 
 // ----------------------------------------------------------------------------
 // MFMA 32x32x16 bf16 (D = A[32xK16] * B[K16x32] + C), wave64.
@@ -110,10 +115,24 @@ __device__ __forceinline__ bf16x8 lds_frag(const bf16_t* tile, int ld, int row0,
 // ----------------------------------------------------------------------------
 // reductions over groups of 16 / 64 lanes
 // ----------------------------------------------------------------------------
+// DPP lane permutations inside a row of 16 lanes (no LDS crossbar traffic)
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// sum over each aligned group of 16 lanes, result in every lane of the group:
+// quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_ror:4, row_ror:8
 __device__ __forceinline__ float group16_sum(float v) {
-  v += __shfl_xor(v, 1); v += __shfl_xor(v, 2);
-  v += __shfl_xor(v, 4); v += __shfl_xor(v, 8);
+  v += dpp_mov<0xB1>(v); v += dpp_mov<0x4E>(v);
+  v += dpp_mov<0x124>(v); v += dpp_mov<0x128>(v);
   return v;
+}
+// Exchange with the other half of the wave (lane l <-> lane l ^ 32) through
+// ds_bpermute with the byte address computed once per kernel:
+//   const int xaddr = half_swap_addr();  ...  other = half_swap(xaddr, mine);
+__device__ __forceinline__ int half_swap_addr() { return ((int)(threadIdx.x & 63) ^ 32) << 2; }
+__device__ __forceinline__ float half_swap(int xaddr, float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(xaddr, __builtin_bit_cast(int, v)));
 }
 __device__ __forceinline__ float wave_sum(float v) {
   v = group16_sum(v);

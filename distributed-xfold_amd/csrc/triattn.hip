@@ -184,6 +184,7 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hh = lane >> 5, j = lane & 31;
+  const int xaddr = half_swap_addr();
   const int N = a.N;
   const int QT = (N + QW - 1) / QW;
   // XCD-aware remap: physical id -> (xcd, slot) -> logical id; logical order is
@@ -287,7 +288,7 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
       float mx = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
 #pragma unroll
       for (int g = 1; g < 4; ++g) mx = fmaxf(mx, fmaxf(fmaxf(s[4 * g], s[4 * g + 1]), fmaxf(s[4 * g + 2], s[4 * g + 3])));
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      mx = fmaxf(mx, half_swap(xaddr, mx));
       const float m_new = fmaxf(m_run, mx);
       const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
       m_run = m_new;
@@ -322,7 +323,7 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
     lds_barrier();
   }
 
-  const float inv = 1.f / (l_run + __shfl_xor(l_run, 32));
+  const float inv = 1.f / (l_run + half_swap(xaddr, l_run));
   if (qw >= N) return;
   const bf16_t* gp = a.g + (bh * N + qw) * D + 4 * hh;
   bf16_t* op = a.og + ((int64_t)b * N + qw) * 128 + h * D + 4 * hh;
