@@ -95,10 +95,13 @@ int af3_triangle_multiplication_forward(
 // ------------------------------------------------------------ triangle attention
 size_t af3_grid_self_attn_workspace_bytes(int64_t n, int num_head) {
   if (n <= 0 || num_head <= 0) return 0;
-  // general path: qkvg + og + fp32 bias; fast path: q, k, g, vt planes + og + bf16 bias (smaller)
-  return align_up((size_t)n * n * 4 * C_PAIR * sizeof(bf16_t), 256) +
-         align_up((size_t)n * n * C_PAIR * sizeof(bf16_t), 256) +
-         align_up((size_t)num_head * n * pad8(n) * sizeof(float), 256) + 4 * 256;
+  const size_t e = sizeof(bf16_t), ldn = (size_t)pad8(n);
+  // fast path: q, k, g planes, vt, og, bf16 bias
+  const size_t fast = 3 * align_up((size_t)n * n * C_PAIR * e, 256) + align_up((size_t)n * C_PAIR * ldn * e, 256) +
+                      align_up((size_t)n * n * C_PAIR * e, 256) + align_up((size_t)num_head * n * ldn * e, 256);
+  // general path (external fp32 bias): qkvg + og
+  const size_t general = align_up((size_t)n * n * 4 * C_PAIR * e, 256) + align_up((size_t)n * n * C_PAIR * e, 256);
+  return fast > general ? fast : general;
 }
 
 int af3_grid_self_attn_forward(

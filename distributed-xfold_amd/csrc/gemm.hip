@@ -17,19 +17,30 @@ namespace {
 constexpr int BM = 128, BN = 128, BK = 64;
 constexpr int LDT = BK + 8;  // padded LDS row (bf16 elements): 144 B keeps 16-B reads conflict-free
 
+constexpr int LDC_S = BN + 4;  // fp32 staging row stride of the C tile
+
 template <bool OUT_F32>
-__global__ __launch_bounds__(256) void gemm_nt_kernel(GemmArgs g) {
-  __shared__ __attribute__((aligned(16))) bf16_t sA[2][BM * LDT];
-  __shared__ __attribute__((aligned(16))) bf16_t sB[2][BN * LDT];
+__global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
+  // A/B slabs, double buffered; after the k loop the same memory stages the C tile
+  __shared__ __attribute__((aligned(16))) bf16_t smem[2 * (BM + BN) * LDT];
+  static_assert(BM * LDC_S * 4 <= 2 * (BM + BN) * LDT * 2, "C staging must fit");
+  constexpr int STAGE = (BM + BN) * LDT;  // buffer `buf`: A slab at smem + buf * STAGE, B slab BM rows later
+  float* sC = reinterpret_cast<float*>(smem);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
 
-  // blockIdx.x walks m-tiles fastest: workgroups in flight together work on
-  // the same batch (channel) and few B panels, which keeps them in L2/MALL.
-  const int tiles_m = (g.M + BM - 1) / BM;
-  const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
-  const int bz = blockIdx.y;
+  // XCD-aware mapping: workgroup ids are dealt round-robin to the 8 XCDs, so
+  // id -> (xcd, slot) -> logical id makes each XCD walk a contiguous range of
+  // (batch, n-tile, m-tile), m-tile fastest: the tiles that share a batch's A
+  // and B panels run on one XCD and find them in its L2.
+  const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n * g.batch;
+  const int per_xcd = (total + 7) / 8;
+  const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (logical >= total) return;
+  const int tm = logical % tiles_m, tn = (logical / tiles_m) % tiles_n;
+  const int bz = logical / (tiles_m * tiles_n);
   const int m0 = tm * BM, n0 = tn * BN;
 
   const bf16_t* A = g.A + (int64_t)bz * g.sA;
@@ -38,24 +49,29 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(GemmArgs g) {
   // each thread moves 4 16-byte chunks of A and 4 of B per k slab
   const int ld_row = tid >> 3, ld_kc = (tid & 7) * 8;  // + 32 rows per step
   u32x4 ra[4], rb[4];
-
+  const bf16_t* pa[4];
+  const bf16_t* pb[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = ld_row + 32 * i;
+    pa[i] = A + (int64_t)min(m0 + row, g.M - 1) * g.lda + ld_kc;
+    pb[i] = B + (int64_t)min(n0 + row, g.N - 1) * g.ldb + ld_kc;
+  }
   auto gload = [&](int k0) {
+    const bool ok = k0 + ld_kc < g.K;
+    const u32x4 z = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int row = ld_row + 32 * i;
-      const int k = k0 + ld_kc;
-      const int am = min(m0 + row, g.M - 1), bn = min(n0 + row, g.N - 1);
-      const u32x4 z = {0, 0, 0, 0};
-      ra[i] = (k < g.K) ? *reinterpret_cast<const u32x4*>(A + (int64_t)am * g.lda + k) : z;
-      rb[i] = (k < g.K) ? *reinterpret_cast<const u32x4*>(B + (int64_t)bn * g.ldb + k) : z;
+      ra[i] = ok ? *reinterpret_cast<const u32x4*>(pa[i] + k0) : z;
+      rb[i] = ok ? *reinterpret_cast<const u32x4*>(pb[i] + k0) : z;
     }
   };
   auto sstore = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = ld_row + 32 * i;
-      *reinterpret_cast<u32x4*>(&sA[buf][row * LDT + ld_kc]) = ra[i];
-      *reinterpret_cast<u32x4*>(&sB[buf][row * LDT + ld_kc]) = rb[i];
+      *reinterpret_cast<u32x4*>(smem + buf * STAGE + row * LDT + ld_kc) = ra[i];
+      *reinterpret_cast<u32x4*>(smem + buf * STAGE + (BM + row) * LDT + ld_kc) = rb[i];
     }
   };
 
@@ -79,9 +95,9 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(GemmArgs g) {
     for (int ks = 0; ks < BK / 16; ++ks) {
       bf16x8 fa[2], fb[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) fa[i] = lds_frag(sA[buf], LDT, wm + 32 * i, ks * 16, lane);
+      for (int i = 0; i < 2; ++i) fa[i] = lds_frag(smem + buf * STAGE, LDT, wm + 32 * i, ks * 16, lane);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) fb[j] = lds_frag(sB[buf], LDT, wn + 32 * j, ks * 16, lane);
+      for (int j = 0; j < 2; ++j) fb[j] = lds_frag(smem + buf * STAGE + BM * LDT, LDT, wn + 32 * j, ks * 16, lane);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -91,79 +107,141 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(GemmArgs g) {
     lds_barrier();
   }
 
-  // ---------------------------------------------------------------- epilogue
-  const int col_l = lane & 31;
+  // ------------------------------------------------------------- epilogue
+  // accumulators (lane = column, registers = rows) -> fp32 tile in LDS, then
+  // each thread finishes 8 consecutive columns of a row with 16/32-byte stores
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        sC[(wm + 32 * i + acc_row(r, lane)) * LDC_S + wn + 32 * j + (lane & 31)] = acc[i][j][r];
+  lds_barrier();
+
+  const int cc = (tid & 15) * 8, r0 = tid >> 4;
   if (g.epi == EPI_SWIGLU) {
     // weight rows are packed in blocks of 64: 32 "a" rows then the 32 matching
-    // "b" rows, so MFMA tile j=0 holds a and j=1 holds b for the same hidden
-    // units; output has N/2 columns.
+    // "b" rows; output has N/2 columns.  Threads with cc < 64 produce 8 outputs each.
+    if (cc >= 64) return;
+    const int blk = cc >> 5, off = cc & 31;         // which 64-column block, offset inside its a half
+    const int oc = n0 / 2 + cc;                     // first output column
+    if (n0 + blk * 64 >= g.N) return;               // N % 64 == 0
     bf16_t* C = reinterpret_cast<bf16_t*>(g.C) + (int64_t)bz * g.sC;
-    const int oc = (n0 + wn) / 2 + col_l;
-    if (n0 + wn < g.N) {  // N % 64 == 0: a 64-column wave span is all in or all out
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+    for (int it = 0; it < 8; ++it) {
+      const int row = it * 16 + r0, m = m0 + row;
+      if (m >= g.M) continue;
+      const float* sa = sC + row * LDC_S + blk * 64 + off;
+      float o[8];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm + 32 * i + acc_row(r, lane);
-          if (m < g.M) {
-            const float a = acc[i][0][r], b = acc[i][1][r];
-            C[(int64_t)m * g.ldc + oc] = f2bf(a * sigmoidf_(a) * b);
-          }
-        }
+      for (int e = 0; e < 8; ++e) { const float a = sa[e], b = sa[32 + e]; o[e] = a * sigmoidf_(a) * b; }
+      bf16_t* dst = C + (int64_t)m * g.ldc + oc;
+      if (g.vec_ok) *reinterpret_cast<u32x4*>(dst) = pack8(o);
+      else
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dst[e] = f2bf(o[e]);
     }
     return;
   }
 
+  const int n = n0 + cc;
+  if (n >= g.N) return;
+  const int nv = min(8, g.N - n);  // valid columns of this chunk
+  float bias[8];
+  int op = SEG_PLAIN;
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int n = n0 + wn + 32 * j + col_l;
-    if (n >= g.N) continue;
-    float bias = 0.f;
-    int op = SEG_PLAIN;
+  for (int e = 0; e < 8; ++e) bias[e] = 0.f;
+  if (g.epi == EPI_SEGMENTED) {
+    op = (g.seg_ops >> (4 * (n / g.seg_len))) & 15;  // seg_len % 8 == 0: a chunk never straddles segments
+    if (op == SEG_BIAS_SCALE && g.bias)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) if (e < nv) bias[e] = g.bias[n + e];
+  } else if (g.bias) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) if (e < nv) bias[e] = g.bias[n + e];
+  }
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int row = it * 16 + r0, m = m0 + row;
+    if (m >= g.M) continue;
+    float v[8];
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(sC + row * LDC_S + cc);
+    const f32x4 hi = *reinterpret_cast<const f32x4*>(sC + row * LDC_S + cc + 4);
+    v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+    const bool full = g.vec_ok && nv == 8;
     if (g.epi == EPI_SEGMENTED) {
-      const int seg = n / g.seg_len;
-      op = (g.seg_ops >> (4 * seg)) & 15;
-      if (op == SEG_BIAS_SCALE && g.bias) bias = g.bias[n];
-    } else if (g.bias) {
-      bias = g.bias[n];
-    }
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm + 32 * i + acc_row(r, lane);
-        if (m >= g.M) continue;
-        float v = acc[i][j][r];
-        if (g.epi == EPI_SEGMENTED) {
-          if (op == SEG_BIAS_SCALE) v = (v + bias) * g.alpha;
-          else if (op == SEG_SIGMOID) v = sigmoidf_(v);
-        } else if (g.epi == EPI_GATE_RES) {
-          v += bias;
-          if (g.gate) v *= g.gate[(int64_t)(m % g.gate_rows) * g.ld_gate + n];
-          if (g.res_f32) v += g.res_f32[(int64_t)bz * g.sRes + (int64_t)m * g.ld_res + n];
-          if (g.res_bf16) v += bf2f(g.res_bf16[(int64_t)bz * g.sRes + (int64_t)m * g.ld_res + n]);
-        } else {  // EPI_PLAIN
-          v = (v + bias) * g.alpha;
-          if (g.act_sigmoid) v = sigmoidf_(v);
-        }
-        const int64_t off = (int64_t)bz * g.sC + (int64_t)m * g.ldc + n;
-        if (OUT_F32) reinterpret_cast<float*>(g.C)[off] = v;
-        else reinterpret_cast<bf16_t*>(g.C)[off] = f2bf(v);
+      for (int e = 0; e < 8; ++e) {
+        if (op == SEG_BIAS_SCALE) v[e] = (v[e] + bias[e]) * g.alpha;
+        else if (op == SEG_SIGMOID) v[e] = sigmoidf_(v[e]);
       }
+    } else if (g.epi == EPI_GATE_RES) {
+      const int64_t roff = (int64_t)bz * g.sRes + (int64_t)m * g.ld_res + n;
+      float gt[8], rs[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { gt[e] = 1.f; rs[e] = 0.f; }
+      if (g.gate) {
+        const float* gp = g.gate + (int64_t)(m % g.gate_rows) * g.ld_gate + n;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) if (e < nv) gt[e] = gp[e];
+      }
+      if (g.res_f32) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) if (e < nv) rs[e] = g.res_f32[roff + e];
+      } else if (g.res_bf16) {
+        if (full && g.res_vec_ok) unpack8(*reinterpret_cast<const u32x4*>(g.res_bf16 + roff), rs);
+        else
+#pragma unroll
+          for (int e = 0; e < 8; ++e) if (e < nv) rs[e] = bf2f(g.res_bf16[roff + e]);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = (v[e] + bias[e]) * gt[e] + rs[e];
+    } else {  // EPI_PLAIN
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        v[e] = (v[e] + bias[e]) * g.alpha;
+        if (g.act_sigmoid) v[e] = sigmoidf_(v[e]);
+      }
+    }
+    const int64_t off = (int64_t)bz * g.sC + (int64_t)m * g.ldc + n;
+    if (OUT_F32) {
+      float* dst = reinterpret_cast<float*>(g.C) + off;
+      if (full) {
+        *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<f32x4*>(dst + 4) = f32x4{v[4], v[5], v[6], v[7]};
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) if (e < nv) dst[e] = v[e];
+      }
+    } else {
+      bf16_t* dst = reinterpret_cast<bf16_t*>(g.C) + off;
+      if (full) *reinterpret_cast<u32x4*>(dst) = pack8(v);
+      else
+#pragma unroll
+        for (int e = 0; e < 8; ++e) if (e < nv) dst[e] = f2bf(v[e]);
+    }
   }
 }
 
 }  // namespace
 
-int launch_gemm_nt(const GemmArgs& g, hipStream_t stream) {
+int launch_gemm_nt(const GemmArgs& g_in, hipStream_t stream) {
+  GemmArgs g = g_in;
   if (g.M <= 0 || g.N <= 0 || g.K <= 0 || g.batch <= 0) return AF3_ERR_BAD_ARG;
   if ((g.K & 7) || (g.lda & 7) || (g.ldb & 7) || (g.sA & 7) || (g.sB & 7)) return AF3_ERR_BAD_ARG;
   if (((uintptr_t)g.A & 15) || ((uintptr_t)g.B & 15)) return AF3_ERR_BAD_ARG;
   if (g.epi == EPI_SWIGLU && ((g.N & 63) || g.out_f32)) return AF3_ERR_BAD_ARG;
-  if (g.epi == EPI_SEGMENTED && g.seg_len <= 0) return AF3_ERR_BAD_ARG;
+  if (g.epi == EPI_SEGMENTED && (g.seg_len <= 0 || (g.seg_len & 7))) return AF3_ERR_BAD_ARG;
   if (g.gate && g.gate_rows <= 0) return AF3_ERR_BAD_ARG;
-  const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
-  dim3 grid(tiles, g.batch);
+  // 16/32-byte stores need aligned rows; otherwise the epilogue stores element-wise
+  const int esz = g.out_f32 ? 4 : 2;
+  g.vec_ok = ((uintptr_t)g.C % 16 == 0) && ((g.ldc * esz) % 16 == 0) && ((g.sC * esz) % 16 == 0);
+  g.res_vec_ok = g.res_bf16 && ((uintptr_t)g.res_bf16 % 16 == 0) && (g.ld_res % 8 == 0) && (g.sRes % 8 == 0);
+  const int64_t total = (int64_t)((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN) * g.batch;
+  const int64_t blocks = (total + 7) / 8 * 8;
+  if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  dim3 grid((unsigned)blocks);
   if (g.out_f32) hipLaunchKernelGGL(gemm_nt_kernel<true>, grid, dim3(256), 0, stream, g);
   else hipLaunchKernelGGL(gemm_nt_kernel<false>, grid, dim3(256), 0, stream, g);
   return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;

@@ -25,6 +25,7 @@ struct GemmArgs {
   const float* res_f32 = nullptr;   // GATE_RES: residual added last (either dtype)
   const bf16_t* res_bf16 = nullptr;
   int64_t ld_res = 0, sRes = 0;
+  int vec_ok = 0, res_vec_ok = 0;  // set by launch_gemm_nt: rows aligned for 16-byte stores / loads
 };
 int launch_gemm_nt(const GemmArgs& g, hipStream_t stream);
 
