@@ -8,6 +8,6 @@ library, or with tensors that are not on the GPU, every operator raises.
 """
 
 from . import lib, ops  # noqa: F401
-from . import nn  # noqa: F401
+from . import check, nn  # noqa: F401
 
-__all__ = ["lib", "ops", "nn"]
+__all__ = ["lib", "ops", "nn", "check"]

@@ -367,4 +367,50 @@ int af3_grid_attention_core_forward(
   return launch_triattn_flash(t, static_cast<hipStream_t>(stream));
 }
 
+// ------------------------------------------------------------- fp32 check mode
+int af3_check_gemm_f32(
+    const float* a, const float* b, float* c, int64_t m, int64_t n, int64_t k, int64_t batch,
+    int64_t lda, int64_t ka, int64_t ldb, int64_t kb, int64_t ldc, int64_t sa, int64_t sb, int64_t sc,
+    const float* bias, float alpha, int sigmoid, const float* mul, int64_t mul_rows, int64_t ld_mul,
+    const float* add, int64_t ld_add, int64_t s_add, af3_stream_t stream) {
+  if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff || batch > 65535) return AF3_ERR_BAD_ARG;
+  CkGemmArgs g;
+  g.A = a; g.B = b; g.C = c; g.M = (int)m; g.N = (int)n; g.K = (int)k; g.batch = (int)batch;
+  g.lda = lda; g.ka = ka; g.ldb = ldb; g.kb = kb; g.ldc = ldc; g.sA = sa; g.sB = sb; g.sC = sc;
+  g.bias = bias; g.alpha = alpha; g.sigmoid = sigmoid;
+  g.mul = mul; g.mul_rows = mul_rows; g.ld_mul = ld_mul; g.add = add; g.ld_add = ld_add; g.s_add = s_add;
+  return launch_ck_gemm(g, static_cast<hipStream_t>(stream));
+}
+
+int af3_check_layer_norm_f32(
+    const float* x, float* y, int64_t rows, int channels, const float* weight, const float* bias,
+    const float* scale, const float* shift, int64_t cond_rows, int64_t cond_ld, af3_stream_t stream) {
+  CkNormArgs a;
+  a.x = x; a.y = y; a.rows = rows; a.C = channels; a.weight = weight; a.bias = bias;
+  a.scale = scale; a.shift = shift; a.cond_rows = cond_rows; a.ld_cond = cond_ld;
+  return launch_ck_norm(a, static_cast<hipStream_t>(stream));
+}
+
+int af3_check_elementwise_f32(
+    int op, const float* x0, const float* x1, const float* x2, float* y0, float* y1,
+    int64_t n0, int64_t n1, int flag, af3_stream_t stream) {
+  return launch_ck_elementwise(op, x0, x1, x2, y0, y1, n0, n1, flag, static_cast<hipStream_t>(stream));
+}
+
+int af3_check_attention_f32(
+    const float* q, const float* k, const float* v, float* out,
+    int64_t q_sb, int64_t q_ss, int64_t k_sb, int64_t k_ss, int64_t v_sb, int64_t v_ss, int64_t o_sb, int64_t o_ss,
+    int64_t batch, int num_head, int64_t sq, int64_t sk, int head_dim,
+    const float* bias, int64_t bias_sb, int64_t bias_sh, int64_t bias_sq, int64_t bias_sk, int64_t bias_mod,
+    const float* key_mask, int64_t km_sb, const float* qpad, const float* kpad, af3_stream_t stream) {
+  if (batch > 0x7fffffff || sq > 0x7fffffff || sk > 0x7fffffff || bias_mod > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  CkAttnArgs a;
+  a.q = q; a.k = k; a.v = v; a.out = out;
+  a.q_sb = q_sb; a.q_ss = q_ss; a.k_sb = k_sb; a.k_ss = k_ss; a.v_sb = v_sb; a.v_ss = v_ss; a.o_sb = o_sb; a.o_ss = o_ss;
+  a.B = (int)batch; a.H = num_head; a.Sq = (int)sq; a.Sk = (int)sk; a.d = head_dim;
+  a.bias = bias; a.bias_sb = bias_sb; a.bias_sh = bias_sh; a.bias_sq = bias_sq; a.bias_sk = bias_sk;
+  a.bias_mod = (int)bias_mod; a.key_mask = key_mask; a.km_sb = km_sb; a.qpad = qpad; a.kpad = kpad;
+  return launch_ck_attention(a, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

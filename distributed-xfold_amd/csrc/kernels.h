@@ -146,3 +146,48 @@ struct TriAttnArgs {
   int64_t ldn = 0;
 };
 int launch_triattn_flash(const TriAttnArgs& a, hipStream_t stream);
+
+// --------------------------------------------------------------- check_f32.hip
+struct CkGemmArgs {
+  const float* A = nullptr;  // element (b, m, k) at A[b*sA + m*lda + k*ka]
+  const float* B = nullptr;  // element (b, n, k) at B[b*sB + n*ldb + k*kb]
+  float* C = nullptr;        // element (b, m, n) at C[b*sC + m*ldc + n]
+  int M = 0, N = 0, K = 0, batch = 1;
+  int64_t lda = 0, ka = 1, ldb = 0, kb = 1, ldc = 0, sA = 0, sB = 0, sC = 0;
+  const float* bias = nullptr;  // y = sigmoid?((acc + bias) * alpha) * mul + add
+  float alpha = 1.f;
+  int sigmoid = 0;
+  const float* mul = nullptr;   // [mul_rows][ld_mul], row m % mul_rows
+  int64_t mul_rows = 0, ld_mul = 0;
+  const float* add = nullptr;   // [b*s_add + m*ld_add + n]
+  int64_t ld_add = 0, s_add = 0;
+};
+int launch_ck_gemm(const CkGemmArgs& g, hipStream_t s);
+
+struct CkNormArgs {
+  const float* x = nullptr;
+  float* y = nullptr;
+  int64_t rows = 0;
+  int C = 0;
+  const float *weight = nullptr, *bias = nullptr, *scale = nullptr, *shift = nullptr;
+  int64_t cond_rows = 0, ld_cond = 0;
+};
+int launch_ck_norm(const CkNormArgs& a, hipStream_t s);
+
+enum { CK_TRIMUL_SPLIT = 0, CK_CHAN_TO_PIX = 1, CK_TRANSPOSE_PIX = 2, CK_SWIGLU = 3, CK_BINARY = 4 };
+int launch_ck_elementwise(int op, const float* x0, const float* x1, const float* x2, float* y0, float* y1,
+                          int64_t n0, int64_t n1, int flag, hipStream_t s);
+
+struct CkAttnArgs {
+  const float *q = nullptr, *k = nullptr, *v = nullptr;  // base + batch*sb + pos*ss + head*d
+  float* out = nullptr;
+  int64_t q_sb = 0, q_ss = 0, k_sb = 0, k_ss = 0, v_sb = 0, v_ss = 0, o_sb = 0, o_ss = 0;
+  int B = 0, H = 0, Sq = 0, Sk = 0, d = 0;
+  const float* bias = nullptr;  // bias[bb*bias_sb + h*bias_sh + q*bias_sq + k*bias_sk]
+  int64_t bias_sb = 0, bias_sh = 0, bias_sq = 0, bias_sk = 1;
+  int bias_mod = 0;             // bb = b % bias_mod when > 0 (also indexes qpad / kpad)
+  const float* key_mask = nullptr;  // [.][Sk], batch stride km_sb: 0 -> logit replaced by -1e9
+  int64_t km_sb = 0;
+  const float *qpad = nullptr, *kpad = nullptr;  // [.][Sq], [.][Sk]: +1e9 where both are 0
+};
+int launch_ck_attention(const CkAttnArgs& a, hipStream_t s);

@@ -2,7 +2,7 @@
 (src/distributed_xfold/nn/*): same constructor keywords, parameter names and
 `forward` signatures; `forward` runs the HIP kernels."""
 
-from .base import HipModule, enable_hip
+from .base import HipModule, check_mode, enable_hip, in_check_mode
 from .triangle_multiplication import TriangleMultiplication
 from .attention import GridSelfAttention
 from .primitives import Transition
@@ -24,7 +24,7 @@ DistributeDiffusionCrossAttTransformer = DiffusionCrossAttTransformer
 DistributePairformerBlock = PairformerBlock
 
 __all__ = [
-    "HipModule", "enable_hip", "TriangleMultiplication", "GridSelfAttention", "Transition",
+    "HipModule", "enable_hip", "check_mode", "in_check_mode", "TriangleMultiplication", "GridSelfAttention", "Transition",
     "AdaptiveLayerNorm", "AdaLNZero", "DiffusionTransition", "SelfAttention", "DiffusionTransformer",
     "CrossAttention", "DiffusionCrossAttTransformer", "PairformerBlock", "PairformerStack",
 ]

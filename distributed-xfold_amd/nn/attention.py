@@ -5,8 +5,8 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from .. import ops
-from .base import HipModule, bf16, drop_mesh, f32, pad_rows
+from .. import check, ops
+from .base import HipModule, bf16, drop_mesh, f32, in_check_mode, pad_rows
 
 
 class GridSelfAttention(HipModule):
@@ -53,4 +53,6 @@ class GridSelfAttention(HipModule):
         if full_pair is not None and full_pair is not pair:
             if full_pair.shape != pair.shape or full_pair.data_ptr() != pair.data_ptr():
                 raise ValueError("single-GPU build: full_pair must be the same tensor as pair")
+        if in_check_mode():
+            return check.grid_self_attention(self, pair, mask)
         return self.run(pair.contiguous(), mask, residual=False)

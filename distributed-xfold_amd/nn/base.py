@@ -6,6 +6,31 @@ import torch
 import torch.nn as nn
 
 
+_CHECK_MODE = False
+
+
+class check_mode:
+    """Context manager / switch for the fp32 check mode: inside it every module's
+    `forward` runs the plain fp32 kernels of `check.py` (fp32 tensors in and out,
+    results returned as new tensors) instead of the bf16 MFMA path."""
+
+    def __init__(self, enabled: bool = True):
+        self.enabled = enabled
+
+    def __enter__(self):
+        global _CHECK_MODE
+        self._old, _CHECK_MODE = _CHECK_MODE, self.enabled
+        return self
+
+    def __exit__(self, *exc):
+        global _CHECK_MODE
+        _CHECK_MODE = self._old
+
+
+def in_check_mode() -> bool:
+    return _CHECK_MODE
+
+
 def drop_mesh(args):
     """The reference's distributed classes take a device mesh as their first
     positional argument (e.g. nn/d_attention.py:24); on one GPU it carries no

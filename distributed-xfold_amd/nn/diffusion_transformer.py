@@ -9,9 +9,10 @@ from typing import Optional
 import torch
 import torch.nn as nn
 
+from .. import check
 from .. import lib as L
 from .. import ops
-from .base import HipModule, bf16, drop_mesh, f32, pack_swiglu, pad_rows
+from .base import HipModule, bf16, drop_mesh, f32, in_check_mode, pack_swiglu, pad_rows
 
 
 class AdaptiveLayerNorm(HipModule):
@@ -38,6 +39,8 @@ class AdaptiveLayerNorm(HipModule):
 
     def forward(self, x: torch.Tensor, single_cond: Optional[torch.Tensor] = None) -> torch.Tensor:
         assert (single_cond is None) == (self.use_single_cond is False)
+        if in_check_mode():
+            return check.adaptive_layer_norm(self, x, single_cond)
         p = self.packed()
         x = x.contiguous()
         if not self.use_single_cond:
@@ -84,6 +87,8 @@ class AdaLNZero(HipModule):
 
     def forward(self, x: torch.Tensor, single_cond: Optional[torch.Tensor] = None) -> torch.Tensor:
         assert (single_cond is None) == (self.use_single_cond is False)
+        if in_check_mode():
+            return check.adaln_zero(self, x, single_cond)
         return self.run(x.to(torch.bfloat16).contiguous(), single_cond, x.dtype)
 
 
@@ -112,6 +117,8 @@ class DiffusionTransition(HipModule):
         return self.adaptive_zero_init.run(h, single_cond, x.dtype, residual=x if residual else None)
 
     def forward(self, x: torch.Tensor, single_cond: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if in_check_mode():
+            return check.diffusion_transition(self, x, single_cond)
         return self.run(x.contiguous(), single_cond, residual=False)
 
 
@@ -160,6 +167,9 @@ class SelfAttention(HipModule):
                 single_cond: Optional[torch.Tensor] = None) -> torch.Tensor:
         """x [N, c] or [B, N, c]; mask [N]; pair_logits [H, N, N]."""
         assert (single_cond is None) == (self.use_single_cond is False)
+        if in_check_mode():
+            pl = None if pair_logits is None else pair_logits.to(torch.float32).contiguous()
+            return check.self_attention(self, x, mask, pl, single_cond)
         return self.run(x.contiguous(), mask, pair_logits, single_cond, residual=False)
 
 
@@ -198,6 +208,8 @@ class DiffusionTransformer(HipModule):
                 pair_cond: torch.Tensor) -> torch.Tensor:
         """act [B, N, c_act] (updated in place, as the reference's `act +=`),
         mask [N], single_cond [N, c_single_cond], pair_cond [N, N, c_pair_cond]."""
+        if in_check_mode():
+            return check.diffusion_transformer(self, act, mask, single_cond, pair_cond)
         p = self.packed()
         pair_cond = pair_cond.contiguous()
         if not act.is_contiguous():
@@ -264,6 +276,9 @@ class CrossAttention(HipModule):
     def forward(self, x_q, x_k, mask_q, mask_k, pair_logits=None, single_cond_q=None, single_cond_k=None):
         """x_q [(B,) S, Q, c], x_k [(B,) S, K, c], masks [(1,) S, Q] / [(1,) S, K],
         pair_logits [(1,) S, H, Q, K], conditioning [(1,) S, Q|K, c]."""
+        if in_check_mode():
+            return check.cross_attention(self, x_q.contiguous(), x_k.contiguous(), mask_q, mask_k, pair_logits,
+                                         single_cond_q, single_cond_k)
         return self.run(x_q.contiguous(), x_k.contiguous(), mask_q, mask_k, pair_logits, single_cond_q,
                         single_cond_k, residual=False)
 
@@ -309,6 +324,9 @@ class DiffusionCrossAttTransformer(HipModule):
 
     def forward(self, queries_act, queries_mask, queries_to_keys, keys_mask, queries_single_cond,
                 keys_single_cond, pair_cond):
+        if in_check_mode():
+            return check.cross_att_transformer(self, queries_act, queries_mask, queries_to_keys, keys_mask,
+                                               queries_single_cond, keys_single_cond, pair_cond)
         p = self.packed()
         if not queries_act.is_contiguous():
             raise ValueError("queries_act must be contiguous (it is updated in place)")

@@ -7,9 +7,9 @@ from typing import Optional
 import torch
 import torch.nn as nn
 
-from .. import ops
+from .. import check, ops
 from .attention import GridSelfAttention
-from .base import HipModule, bf16, drop_mesh, f32, pad_rows
+from .base import HipModule, bf16, drop_mesh, f32, in_check_mode, pad_rows
 from .diffusion_transformer import SelfAttention
 from .primitives import Transition
 from .triangle_multiplication import TriangleMultiplication
@@ -54,6 +54,8 @@ class PairformerBlock(HipModule):
     def forward(self, pair: torch.Tensor, pair_mask: torch.Tensor, single: Optional[torch.Tensor] = None,
                 seq_mask: Optional[torch.Tensor] = None, head: int = 0):
         """pair [N, N, c_pair], pair_mask [N, N], single [N, c_single], seq_mask [N]."""
+        if in_check_mode():
+            return check.pairformer_block(self, pair, pair_mask, single, seq_mask)
         if not pair.is_contiguous():
             raise ValueError("pair must be contiguous (it is updated in place)")
         self.triangle_multiplication_outgoing.run(pair, pair_mask, residual=True)

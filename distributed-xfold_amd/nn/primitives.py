@@ -5,9 +5,10 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
+from .. import check
 from .. import lib as L
 from .. import ops
-from .base import HipModule, bf16, drop_mesh, f32, pack_swiglu
+from .base import HipModule, bf16, drop_mesh, f32, in_check_mode, pack_swiglu
 
 
 class Transition(HipModule):
@@ -51,4 +52,6 @@ class Transition(HipModule):
                           residual=x if residual else None, out=x if residual else None)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if in_check_mode():
+            return check.transition(self, x)
         return self.run(x.contiguous(), residual=False)

@@ -5,8 +5,8 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from .. import ops
-from .base import HipModule, bf16, drop_mesh, f32
+from .. import check, ops
+from .base import HipModule, bf16, drop_mesh, f32, in_check_mode
 
 
 class TriangleMultiplication(HipModule):
@@ -61,4 +61,6 @@ class TriangleMultiplication(HipModule):
 
     def forward(self, pair: torch.Tensor, mask: torch.Tensor, head: int = 0) -> torch.Tensor:
         """pair [N, N, c_pair], mask [N, N] -> update [N, N, c_pair] (same dtype)."""
+        if in_check_mode():
+            return check.triangle_multiplication(self, pair, mask)
         return self.run(pair.contiguous(), mask, residual=False)

@@ -361,3 +361,92 @@ def grid_attention_core(q, k, vt, g, pair_bias, mask, out=None):
                                              _stream(q.device))
     _L.check(rc, "af3_grid_attention_core_forward")
     return out
+
+
+# --------------------------------------------------------------- fp32 check mode
+def _f32(t, name):
+    _gpu(t, name, torch.float32)
+    return t
+
+
+def ck_gemm(a, b, *, m, n, k, batch=1, lda, ldb, ka=1, kb=1, sa=0, sb=0, out=None, bias=None, alpha=1.0,
+            sigmoid=False, mul=None, add=None):
+    """fp32 C[b][m][n] = epi(sum_k A(b,m,k) B(b,n,k)) with explicit element strides
+    (af3_check_gemm_f32); C is dense [batch, m, n]."""
+    lib = _L.load()
+    if not (a.is_cuda and b.is_cuda and a.dtype == torch.float32 and b.dtype == torch.float32):
+        raise ValueError("ck_gemm: operands must be fp32 GPU tensors")
+    if out is None:
+        out = torch.empty((batch, m, n) if batch > 1 else (m, n), dtype=torch.float32, device=a.device)
+    mul_rows = ld_mul = 0
+    if mul is not None:
+        _f32(mul, "mul")
+        mul_rows, ld_mul = mul.numel() // n, n
+    ld_add = s_add = 0
+    if add is not None:
+        _f32(add, "add")
+        ld_add, s_add = n, m * n
+    if bias is not None:
+        _f32(bias, "bias")
+    rc = lib.af3_check_gemm_f32(_p(a), _p(b), _p(out), m, n, k, batch, lda, ka, ldb, kb, n, sa, sb, m * n,
+                                _p(bias), float(alpha), int(bool(sigmoid)), _p(mul), mul_rows, ld_mul,
+                                _p(add), ld_add, s_add, _stream(a.device))
+    _L.check(rc, "af3_check_gemm_f32")
+    return out
+
+
+def ck_linear(x, w, bias=None, alpha=1.0, sigmoid=False, mul=None, add=None):
+    """fp32 y = epi(x @ w.T) for contiguous x [..., K], w [N, K]."""
+    _f32(x, "x")
+    _f32(w, "w")
+    k = x.shape[-1]
+    m = x.numel() // k
+    n = w.shape[0]
+    y = ck_gemm(x, w, m=m, n=n, k=k, lda=k, ldb=k, bias=bias, alpha=alpha, sigmoid=sigmoid, mul=mul, add=add)
+    return y.reshape(tuple(x.shape[:-1]) + (n,))
+
+
+def ck_layer_norm(x, weight=None, bias=None, scale=None, shift=None):
+    lib = _L.load()
+    _f32(x, "x")
+    c = x.shape[-1]
+    rows = x.numel() // c
+    cond_rows = cond_ld = 0
+    if scale is not None:
+        cond_rows, cond_ld = scale.shape[0], scale.stride(0)
+    y = torch.empty_like(x)
+    rc = lib.af3_check_layer_norm_f32(_p(x), _p(y), rows, c, _p(weight), _p(bias), _p(scale), _p(shift),
+                                      cond_rows, cond_ld, _stream(x.device))
+    _L.check(rc, "af3_check_layer_norm_f32")
+    return y
+
+
+def ck_elementwise(op, x0, x1, x2, y0, y1, n0, n1, flag):
+    lib = _L.load()
+    rc = lib.af3_check_elementwise_f32(int(op), _p(x0), _p(x1), _p(x2), _p(y0), _p(y1), int(n0), int(n1), int(flag),
+                                       _stream(x0.device))
+    _L.check(rc, "af3_check_elementwise_f32")
+
+
+def ck_attention(q, k, v, num_head, bias=None, bias_strides=(0, 0, 0, 1), bias_mod=0, key_mask=None, km_sb=0,
+                 qpad=None, kpad=None):
+    """fp32 attention; q [B, Sq, H*d], k / v [B, Sk, H*d] (any batch / position
+    strides, unit channel stride); bias addressed with explicit element strides
+    (batch, head, query, key)."""
+    lib = _L.load()
+    for nm, t in (("q", q), ("k", k), ("v", v)):
+        if not (t.is_cuda and t.dtype == torch.float32 and t.dim() == 3 and t.stride(2) == 1):
+            raise ValueError(f"{nm}: expected an fp32 GPU tensor [B, S, C] with unit channel stride")
+    b, sq, c = q.shape
+    sk = k.shape[1]
+    d = c // num_head
+    out = torch.empty((b, sq, c), dtype=torch.float32, device=q.device)
+    km = None if key_mask is None else key_mask.to(torch.float32).contiguous()
+    qp = None if qpad is None else qpad.to(torch.float32).contiguous()
+    kp = None if kpad is None else kpad.to(torch.float32).contiguous()
+    rc = lib.af3_check_attention_f32(
+        _p(q), _p(k), _p(v), _p(out), q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
+        out.stride(0), out.stride(1), b, int(num_head), sq, sk, d, _p(bias), *[int(s) for s in bias_strides],
+        int(bias_mod), _p(km), int(km_sb), _p(qp), _p(kp), _stream(q.device))
+    _L.check(rc, "af3_check_attention_f32")
+    return out

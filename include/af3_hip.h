@@ -237,6 +237,47 @@ int af3_grid_attention_core_forward(
     const uint16_t* q, const uint16_t* k, const uint16_t* vt, const uint16_t* g,
     const uint16_t* pair_bias, const float* mask, uint16_t* og, int64_t n_token, af3_stream_t stream);
 
+/* ---------------------------------------------------------------------------
+ * fp32 check mode.  Plain fp32 kernels (fp32 storage, fp32 FMA arithmetic, no
+ * MFMA, no fusion) from which the host composes every operator above a second
+ * time; they share no code with the bf16 kernels.  They have no counterpart in
+ * the reference's operator set: they exist so that the bf16 path can be checked
+ * on the GPU, at sizes the CPU oracle cannot reach, against an independent
+ * implementation that itself matches the oracle to 1e-4.
+ *
+ * af3_check_gemm_f32: C[b][m][n] = (sigmoid?)((sum_k A(b,m,k) B(b,n,k) + bias[n]) * alpha)
+ *   * mul[m % mul_rows][n] + add(b,m,n), with A(b,m,k) = a[b*sa + m*lda + k*ka] and
+ *   B(b,n,k) = b[b*sb + n*ldb + k*kb] (so either operand may be read transposed).
+ * af3_check_layer_norm_f32: the fp32 twin of af3_layer_norm_forward.
+ * af3_check_elementwise_f32: op 0 triangle-multiplication gating and a/b split
+ *   (x0 proj [N*N,256], x1 gate, x2 mask or NULL -> y0 a, y1 b channel-major
+ *   [128][N][N]; flag 1 = incoming, stored transposed), op 1 channel-major
+ *   [n1][N][N] -> [N][N][n1], op 2 out[j][i][:] = in[i][j][:] with n1 channels,
+ *   op 3 SwiGLU y0[m][f] = silu(x0[m][f]) * x0[m][n1 + f] for n0 rows,
+ *   op 4 y0 = x0 * x1 (flag 0) or x0 + x1 (flag 1) over n0 elements.
+ * af3_check_attention_f32: softmax(q.k + bias, masks) v per (batch, head, query),
+ *   operands addressed base + batch*sb + position*ss + head*head_dim, bias at
+ *   bias[(b % bias_mod)*bias_sb + h*bias_sh + q*bias_sq + k*bias_sk]; key_mask /
+ *   qpad / kpad as in the bf16 entry points.
+ */
+int af3_check_gemm_f32(
+    const float* a, const float* b, float* c, int64_t m, int64_t n, int64_t k, int64_t batch,
+    int64_t lda, int64_t ka, int64_t ldb, int64_t kb, int64_t ldc, int64_t sa, int64_t sb, int64_t sc,
+    const float* bias, float alpha, int sigmoid, const float* mul, int64_t mul_rows, int64_t ld_mul,
+    const float* add, int64_t ld_add, int64_t s_add, af3_stream_t stream);
+int af3_check_layer_norm_f32(
+    const float* x, float* y, int64_t rows, int channels, const float* weight, const float* bias,
+    const float* scale, const float* shift, int64_t cond_rows, int64_t cond_ld, af3_stream_t stream);
+int af3_check_elementwise_f32(
+    int op, const float* x0, const float* x1, const float* x2, float* y0, float* y1,
+    int64_t n0, int64_t n1, int flag, af3_stream_t stream);
+int af3_check_attention_f32(
+    const float* q, const float* k, const float* v, float* out,
+    int64_t q_sb, int64_t q_ss, int64_t k_sb, int64_t k_ss, int64_t v_sb, int64_t v_ss, int64_t o_sb, int64_t o_ss,
+    int64_t batch, int num_head, int64_t sq, int64_t sk, int head_dim,
+    const float* bias, int64_t bias_sb, int64_t bias_sh, int64_t bias_sq, int64_t bias_sk, int64_t bias_mod,
+    const float* key_mask, int64_t km_sb, const float* qpad, const float* kpad, af3_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
