@@ -173,14 +173,15 @@ __global__ __launch_bounds__(256, 2) void triattn_proj_kernel(TriAttnProjArgs a)
 // ============================================================================
 constexpr int KT = 64;       // keys per LDS tile
 constexpr int LDK = 56;      // sK row: 32 head-dim + 16 mask k-step + 8 pad (bf16); 112 B
-constexpr int LDV = KT + 4;  // sVt / sB row: 136 B = 34 dwords, so 32 lanes' 8-byte reads hit 32 bank pairs
+constexpr int LDV = KT + 4;  // sVt row: 136 B = 34 dwords, so 32 lanes' 8-byte reads hit 32 bank pairs
+constexpr int LDB = KT + 8;  // sB row: 144 B, 16-byte aligned for the 16-byte fragment reads
 constexpr int QW = 128;      // queries per workgroup
 constexpr uint32_t BF16_ONE = 0x3F80u, BF16_NEG_INF = 0xFF80u, BF16_NEG_1E9 = 0xCE6Eu;
 
 __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t sK[2][KT * LDK];
   __shared__ __attribute__((aligned(16))) bf16_t sVt[2][D * LDV];
-  __shared__ __attribute__((aligned(16))) bf16_t sB[2][QW * LDV];
+  __shared__ __attribute__((aligned(16))) bf16_t sB[2][QW * LDB];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hh = lane >> 5, j = lane & 31;
@@ -209,34 +210,51 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
     u32x4 one = {hh == 0 ? BF16_ONE : 0u, 0u, 0u, 0u};
     qf[2] = as_frag(one);
   }
+  // Identity fragments: S^T += I * bias^T adds the pair bias inside the matrix
+  // unit.  A-fragment of k-step `st`: lane (row i = j, half hh) holds
+  // I[i][16 st + 8 hh + e], e = 0..7, i.e. a single 1.0 where 16 st + 8 hh + e == i.
+  bf16x8 idf[2];
+#pragma unroll
+  for (int st = 0; st < 2; ++st) {
+    const int e1 = j - 16 * st - 8 * hh;  // position of the 1.0 inside this lane's 8 elements, if any
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+    if (e1 >= 0 && e1 < 8) w[e1 >> 1] = (e1 & 1) ? (BF16_ONE << 16) : BF16_ONE;
+    idf[st] = as_frag(u32x4{w[0], w[1], w[2], w[3]});
+  }
 
   // loaders, one 16-byte chunk each per tile:
   //   K   thread (key = tid / 4, c = tid % 4)            + the mask k-step by c < 2
   //   Vt  thread (d = tid / 8, kc = tid % 8)
   //   bias: four chunks, idx = tid + 256 i -> (q = idx / 8, kc = idx % 8)
+  // Pointers are set up once and advance by one tile per iteration.
   const int k_key = tid >> 2, k_c = tid & 3;
-  const int v_d = tid >> 3, v_kc = (tid & 7) * 8;
-  const bf16_t* kbase = a.k + bh * N * D;
-  const bf16_t* vbase = a.vt + (bh * D + v_d) * a.ldn + v_kc;
-  const float* mrow = a.mask ? a.mask + (int64_t)b * N : nullptr;
-  const bf16_t* bias_h = a.bias ? a.bias + (int64_t)h * N * a.ldn : nullptr;
+  const int v_d = tid >> 3, c8 = (tid & 7) * 8;
+  const bf16_t* pk = a.k + (bh * N + k_key) * D + k_c * 8;
+  const bf16_t* pv = a.vt + (bh * D + v_d) * a.ldn + c8;
+  const float* pm = (a.mask && k_c == 0) ? a.mask + (int64_t)b * N + k_key : nullptr;
+  const bf16_t* pb = a.bias ? a.bias + ((int64_t)h * N + q0 + (tid >> 3)) * a.ldn + c8 : nullptr;
+  const int64_t brow = (int64_t)32 * a.ldn;  // bias chunks i and i + 1 are 32 query rows apart
+  bool bq_ok[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) bq_ok[i] = pb != nullptr && q0 + (tid >> 3) + 32 * i < N;
+  const int ldn = (int)a.ldn;
+
   u32x4 rk, rv, rb[4];
   uint32_t rmask;
   auto gload = [&](int k0) {
     const u32x4 z = {0, 0, 0, 0};
-    const int key = k0 + k_key;
-    rk = z;
-    rmask = BF16_NEG_INF;
-    if (key < N) {
-      rk = *reinterpret_cast<const u32x4*>(kbase + (int64_t)key * D + k_c * 8);
-      rmask = (mrow && mrow[key] == 0.f) ? BF16_NEG_1E9 : 0u;
-    }
-    rv = (k0 + v_kc < a.ldn) ? *reinterpret_cast<const u32x4*>(vbase + k0) : z;
+    const bool key_ok = k0 + k_key < N;
+    rk = key_ok ? *reinterpret_cast<const u32x4*>(pk) : z;
+    rmask = key_ok ? 0u : BF16_NEG_INF;
+    if (pm && key_ok && *pm == 0.f) rmask = BF16_NEG_1E9;
+    const bool col_ok = k0 + c8 < ldn;
+    rv = col_ok ? *reinterpret_cast<const u32x4*>(pv) : z;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int idx = tid + 256 * i, q = q0 + (idx >> 3), kc = k0 + (idx & 7) * 8;
-      rb[i] = (bias_h && q < N && kc < a.ldn) ? *reinterpret_cast<const u32x4*>(bias_h + (int64_t)q * a.ldn + kc) : z;
-    }
+    for (int i = 0; i < 4; ++i) rb[i] = (bq_ok[i] && col_ok) ? *reinterpret_cast<const u32x4*>(pb + i * brow) : z;
+    pk += KT * D;
+    pv += KT;
+    if (pm) pm += KT;
+    if (pb) pb += KT;
   };
   auto sstore = [&](int buf) {
     *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + k_c * 8]) = rk;
@@ -244,17 +262,13 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
       u32x4 m = {k_c == 0 ? rmask : 0u, 0u, 0u, 0u};
       *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + 32 + k_c * 8]) = m;
     }
-    // rows of sVt / sB are 8-byte aligned only: two 8-byte stores per chunk
-    u32x2* pv = reinterpret_cast<u32x2*>(&sVt[buf][v_d * LDV + v_kc]);
-    pv[0] = u32x2{rv.x, rv.y};
-    pv[1] = u32x2{rv.z, rv.w};
+    // rows of sVt are 8-byte aligned only: two 8-byte stores
+    u32x2* pvs = reinterpret_cast<u32x2*>(&sVt[buf][v_d * LDV + c8]);
+    pvs[0] = u32x2{rv.x, rv.y};
+    pvs[1] = u32x2{rv.z, rv.w};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int idx = tid + 256 * i;
-      u32x2* pb = reinterpret_cast<u32x2*>(&sB[buf][(idx >> 3) * LDV + (idx & 7) * 8]);
-      pb[0] = u32x2{rb[i].x, rb[i].y};
-      pb[1] = u32x2{rb[i].z, rb[i].w};
-    }
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<u32x4*>(&sB[buf][((tid >> 3) + 32 * i) * LDB + c8]) = rb[i];
   };
 
   f32x16 o;
@@ -273,14 +287,15 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       if (kt * KT + sub * 32 >= N) break;  // uniform across the workgroup
-      // accumulator starts as the pair bias: s[4g + e] <-> key 8g + 4hh + e of this sub-tile
+      // logits, transposed: s[4g + e] <-> key 8g + 4hh + e of this sub-tile, query j.
+      // bias via the identity product, then K Q^T, then the mask k-step.
       f32x16 s;
-      const bf16_t* bp = &sB[buf][(wave * 32 + j) * LDV + sub * 32 + 4 * hh];
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const u32x2 w = *reinterpret_cast<const u32x2*>(bp + 8 * g);
-        s[4 * g] = bflo(w.x); s[4 * g + 1] = bfhi(w.x); s[4 * g + 2] = bflo(w.y); s[4 * g + 3] = bfhi(w.y);
-      }
+      for (int r = 0; r < 16; ++r) s[r] = 0.f;
+      const bf16_t* bp = &sB[buf][(wave * 32 + j) * LDB + sub * 32 + 8 * hh];
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+        s = mfma32(idf[st], as_frag(*reinterpret_cast<const u32x4*>(bp + 16 * st)), s);
 #pragma unroll
       for (int ks = 0; ks < 3; ++ks)
         s = mfma32(lds_frag(sK[buf], LDK, sub * 32, ks * 16, lane), qf[ks], s);
@@ -296,13 +311,13 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
       bf16x8 pf[2];
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        float pv[8];
+        float pv8[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          pv[e] = __builtin_amdgcn_exp2f(s[8 * half + e] - m_new);
-          psum += pv[e];
+          pv8[e] = __builtin_amdgcn_exp2f(s[8 * half + e] - m_new);
+          psum += pv8[e];
         }
-        pf[half] = as_frag(pack8(pv));
+        pf[half] = as_frag(pack8(pv8));
       }
       l_run = l_run * alpha + psum;
       if (__any(alpha != 1.f)) {
