@@ -178,10 +178,15 @@ constexpr int LDB = KT + 8;  // sB row: 144 B, 16-byte aligned for the 16-byte f
 constexpr int QW = 128;      // queries per workgroup
 constexpr uint32_t BF16_ONE = 0x3F80u, BF16_NEG_INF = 0xFF80u, BF16_NEG_1E9 = 0xCE6Eu;
 
-__global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
-  __shared__ __attribute__((aligned(16))) bf16_t sK[2][KT * LDK];
-  __shared__ __attribute__((aligned(16))) bf16_t sVt[2][D * LDV];
-  __shared__ __attribute__((aligned(16))) bf16_t sB[2][QW * LDB];
+// LDS tiles are single-buffered (30 KB): the next tile waits in registers while
+// the current one is consumed, at the price of a second barrier per tile; in
+// exchange three workgroups fit on a CU, and with head dim 32 it is the number
+// of waves available to hide the MFMA -> softmax -> MFMA dependency chain that
+// sets the pace, not the barrier count.
+__global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t sK[1][KT * LDK];
+  __shared__ __attribute__((aligned(16))) bf16_t sVt[1][D * LDV];
+  __shared__ __attribute__((aligned(16))) bf16_t sB[1][QW * LDB];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hh = lane >> 5, j = lane & 31;
@@ -282,60 +287,71 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
   lds_barrier();
 
   for (int kt = 0; kt < nkt; ++kt) {
-    const int buf = kt & 1;
+    constexpr int buf = 0;
     if (kt + 1 < nkt) gload((kt + 1) * KT);
+    // Both 32-key halves of the tile go through the matrix unit first (two
+    // independent accumulator chains), then one online-softmax update covers
+    // all 64 keys, then both halves feed O.  A half that lies wholly beyond N
+    // has every key at -inf (mask column) and contributes exactly zero.
+    // s[u][4g + e] <-> key 32u + 8g + 4hh + e of this tile, query j.
+    f32x16 s[2];
 #pragma unroll
-    for (int sub = 0; sub < 2; ++sub) {
-      if (kt * KT + sub * 32 >= N) break;  // uniform across the workgroup
-      // logits, transposed: s[4g + e] <-> key 8g + 4hh + e of this sub-tile, query j.
-      // bias via the identity product, then K Q^T, then the mask k-step.
-      f32x16 s;
+    for (int u = 0; u < 2; ++u) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[r] = 0.f;
-      const bf16_t* bp = &sB[buf][(wave * 32 + j) * LDB + sub * 32 + 8 * hh];
+      for (int r = 0; r < 16; ++r) s[u][r] = 0.f;
+      const bf16_t* bp = &sB[buf][(wave * 32 + j) * LDB + u * 32 + 8 * hh];
 #pragma unroll
       for (int st = 0; st < 2; ++st)
-        s = mfma32(idf[st], as_frag(*reinterpret_cast<const u32x4*>(bp + 16 * st)), s);
+        s[u] = mfma32(idf[st], as_frag(*reinterpret_cast<const u32x4*>(bp + 16 * st)), s[u]);
 #pragma unroll
       for (int ks = 0; ks < 3; ++ks)
-        s = mfma32(lds_frag(sK[buf], LDK, sub * 32, ks * 16, lane), qf[ks], s);
-
-      float mx = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+        s[u] = mfma32(lds_frag(sK[buf], LDK, u * 32, ks * 16, lane), qf[ks], s[u]);
+    }
+    float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
 #pragma unroll
-      for (int g = 1; g < 4; ++g) mx = fmaxf(mx, fmaxf(fmaxf(s[4 * g], s[4 * g + 1]), fmaxf(s[4 * g + 2], s[4 * g + 3])));
-      mx = fmaxf(mx, half_swap(xaddr, mx));
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-      m_run = m_new;
-      float psum = 0.f;
-      bf16x8 pf[2];
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int g = (u == 0 ? 1 : 0); g < 4; ++g)
+        mx = fmaxf(mx, fmaxf(fmaxf(s[u][4 * g], s[u][4 * g + 1]), fmaxf(s[u][4 * g + 2], s[u][4 * g + 3])));
+    mx = fmaxf(mx, half_swap(xaddr, mx));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    m_run = m_new;
+    float psum = 0.f;
+    bf16x8 pf[2][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         float pv8[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          pv8[e] = __builtin_amdgcn_exp2f(s[8 * half + e] - m_new);
+          pv8[e] = __builtin_amdgcn_exp2f(s[u][8 * half + e] - m_new);
           psum += pv8[e];
         }
-        pf[half] = as_frag(pack8(pv8));
+        pf[u][half] = as_frag(pack8(pv8));
       }
-      l_run = l_run * alpha + psum;
-      if (__any(alpha != 1.f)) {
+    l_run = l_run * alpha + psum;
+    if (__any(alpha != 1.f)) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[r] *= alpha;
-      }
+      for (int r = 0; r < 16; ++r) o[r] *= alpha;
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        const bf16_t* vp = &sVt[buf][j * LDV + sub * 32 + 16 * half + 4 * hh];
+        const bf16_t* vp = &sVt[buf][j * LDV + u * 32 + 16 * half + 4 * hh];
         const u32x2 lo = *reinterpret_cast<const u32x2*>(vp);
         const u32x2 hi = *reinterpret_cast<const u32x2*>(vp + 8);
         u32x4 vv;
         vv.x = lo.x; vv.y = lo.y; vv.z = hi.x; vv.w = hi.y;
-        o = mfma32(as_frag(vv), pf[half], o);
+        o = mfma32(as_frag(vv), pf[u][half], o);
       }
+    if (kt + 1 < nkt) {
+      lds_barrier();  // every wave is done reading this tile
+      sstore(0);
+      lds_barrier();
     }
-    if (kt + 1 < nkt) sstore(buf ^ 1);
-    lds_barrier();
   }
 
   const float inv = 1.f / (l_run + half_swap(xaddr, l_run));
