@@ -176,9 +176,8 @@ def main():
     t_buf = torch.empty_like(a)
     q_, k_, g_ = ((torch.randn(n, 4, n, 32, generator=g) * 0.5).to(dev).bfloat16() for _ in range(3))
     vt_ = (torch.randn(n, 4, 32, npad, generator=g) * 0.5).to(dev).bfloat16()
-    nb = torch.randn(4, n, npad, generator=g).to(dev).bfloat16()
+    nb = pkg.ops.pack_pair_bias(torch.randn(4, n, npad, generator=g).to(dev).bfloat16())
     vt_[..., n:] = 0
-    nb[..., n:] = 0
     og = torch.empty((n * n, 128), dtype=torch.bfloat16, device=dev)
     ms_contract = gpu_time_ms(lambda: pkg.ops.triangle_contraction(a, b, t_buf), it)
     ms_attn = gpu_time_ms(lambda: pkg.ops.grid_attention_core(q_, k_, vt_, g_, nb, pair_mask, og), it)

@@ -98,7 +98,7 @@ size_t af3_grid_self_attn_workspace_bytes(int64_t n, int num_head) {
   const size_t e = sizeof(bf16_t), ldn = (size_t)pad8(n);
   // fast path: q, k, g planes, vt, og, bf16 bias
   const size_t fast = 3 * align_up((size_t)n * n * C_PAIR * e, 256) + align_up((size_t)n * C_PAIR * ldn * e, 256) +
-                      align_up((size_t)n * n * C_PAIR * e, 256) + align_up((size_t)num_head * n * ldn * e, 256);
+                      align_up((size_t)n * n * C_PAIR * e, 256) + align_up((size_t)tri_bias_elems(n, num_head) * e, 256);
   // general path (external fp32 bias): qkvg + og
   const size_t general = align_up((size_t)n * n * 4 * C_PAIR * e, 256) + align_up((size_t)n * n * C_PAIR * e, 256);
   return fast > general ? fast : general;
@@ -131,7 +131,7 @@ int af3_grid_self_attn_forward(
     bf16_t* g = ws.take<bf16_t>((size_t)n * n * C_PAIR);
     bf16_t* vt = ws.take<bf16_t>((size_t)n * C_PAIR * ldn);
     og = ws.take<bf16_t>((size_t)n * n * C_PAIR);
-    bf16_t* bias = ws.take<bf16_t>((size_t)num_head * n * ldn);
+    bf16_t* bias = ws.take<bf16_t>((size_t)tri_bias_elems(n, num_head));
     if (!ws.ok) return AF3_ERR_WORKSPACE;
     TriAttnProjArgs p;
     p.pair = pair; p.io_f32 = io_dtype == AF3_F32; p.N = (int)n; p.transpose = transpose != 0;

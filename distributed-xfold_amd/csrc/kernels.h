@@ -124,6 +124,22 @@ int launch_flash_attention(const FlashArgs& a, hipStream_t stream);
 // ---------------------------------------------------------------- triattn.hip
 // Head-major scratch of the triangle-attention fast path (all bf16):
 //   q, k, g [b][h][s][32];  vt [b][h][32][ldn];  bias [h][q][ldn] (times log2 e, pad columns zero)
+// Pair bias of the triangle attention in MFMA-fragment order.  The attention
+// core adds the bias through the matrix unit (S^T += I * bias^T) and wants, per
+// (head, 32-query block, 64-key tile), the four B fragments of that product as
+// four contiguous 1 KB runs: element (h, q, k) lives at
+//   ((((h * QB + q / 32) * KT + k / 64) * 4 + (k % 64) / 16) * 32 + q % 32) * 16 + k % 16
+// with QB = ceil(N / 32), KT = ceil(N / 64); entries whose key is >= N are zero.
+__host__ __device__ inline int64_t tri_bias_qblocks(int64_t n) { return (n + 31) / 32; }
+__host__ __device__ inline int64_t tri_bias_ktiles(int64_t n) { return (n + 63) / 64; }
+__host__ __device__ inline int64_t tri_bias_elems(int64_t n, int64_t heads) {
+  return heads * tri_bias_qblocks(n) * tri_bias_ktiles(n) * 2048;
+}
+__host__ __device__ inline int64_t tri_bias_offset(int64_t n, int h, int q, int k) {
+  return ((((int64_t)h * tri_bias_qblocks(n) + (q >> 5)) * tri_bias_ktiles(n) + (k >> 6)) * 4 + ((k & 63) >> 4)) * 512 +
+         (q & 31) * 16 + (k & 15);
+}
+
 struct TriAttnProjArgs {
   const void* pair = nullptr;  // [N][N][128]
   int io_f32 = 0, N = 0, transpose = 0, skip_ln = 0;
@@ -132,14 +148,15 @@ struct TriAttnProjArgs {
   const bf16_t* w_bias = nullptr;  // [32][128], rows >= 4 zero
   int n_bias = 0;                  // 0 or 4
   float q_scale = 1.f, bias_scale = 1.f;
-  bf16_t *q = nullptr, *k = nullptr, *vt = nullptr, *g = nullptr, *bias = nullptr;
+  bf16_t *q = nullptr, *k = nullptr, *vt = nullptr, *g = nullptr;
+  bf16_t* bias = nullptr;  // fragment order, tri_bias_elems(N, 4) elements
   int64_t ldn = 0;
 };
 int launch_triattn_proj(const TriAttnProjArgs& a, hipStream_t stream);
 
 struct TriAttnArgs {
   const bf16_t *q = nullptr, *k = nullptr, *vt = nullptr, *g = nullptr;
-  const bf16_t* bias = nullptr;  // or null
+  const bf16_t* bias = nullptr;  // fragment order (tri_bias_offset), or null
   const float* mask = nullptr;   // [N][N] 0/1 or null
   bf16_t* og = nullptr;          // [(b*N + s)][128]
   int N = 0;

@@ -4,7 +4,7 @@
 // Scratch layout (bf16), for rows b of the (possibly transposed) operator:
 //   Q, K, G : [b][h][s][32]          one 4 KB-contiguous slab per 64 positions
 //   Vt      : [b][h][32][ldn]        V transposed (keys contiguous), ldn = N up to 8
-//   bias    : [h][q][ldn]            pair bias * log2(e); columns N..ldn-1 are zero
+//   bias    : MFMA-fragment order     pair bias * log2(e) (tri_bias_offset); keys >= N zero
 // so every tile the flash kernel stages is a run of full 16-byte chunks with no
 // transposition and no boundary code.
 //
@@ -23,6 +23,8 @@
 //     XCD's L2.
 #include "common.h"
 #include "kernels.h"
+#include <type_traits>
+
 #include "tile_common.h"
 
 namespace {
@@ -53,8 +55,10 @@ __global__ __launch_bounds__(256, 2) void triattn_proj_kernel(TriAttnProjArgs a)
   const int64_t bh0 = (int64_t)t.o * H;  // (b * H + h) for h = 0
   // chunk order q, k, v, g as packed in w_qkvg; v takes the channel-major route.
   // Two 32-row weight tiles at a time keep the live accumulators at 32 registers.
-#pragma unroll 1
-  for (int chunk = 0; chunk < 4; ++chunk) {
+  // The chunk index is a compile-time constant of the body: with a run-time
+  // index the compiler evaluates the sigmoid for every chunk and selects.
+  auto do_chunk = [&](auto chunk_c) {
+    constexpr int chunk = decltype(chunk_c)::value;
     // The next weights are requested BEFORE this chunk's results are stored:
     // vector memory operations retire in order, so a load issued behind the
     // stores would make its consumer wait for the stores' round trip to HBM.
@@ -137,7 +141,11 @@ __global__ __launch_bounds__(256, 2) void triattn_proj_kernel(TriAttnProjArgs a)
       }
     }
     lds_barrier();
-  }
+  };
+  do_chunk(std::integral_constant<int, 0>{});
+  do_chunk(std::integral_constant<int, 1>{});
+  do_chunk(std::integral_constant<int, 2>{});
+  do_chunk(std::integral_constant<int, 3>{});
 
   // pair-bias heads (T form: lane = pixel, rows = heads): bias[h][q][k] with
   // (q, k) the pixel's own (row, col) in the un-transposed pair tensor
@@ -147,21 +155,21 @@ __global__ __launch_bounds__(256, 2) void triattn_proj_kernel(TriAttnProjArgs a)
     if ((lane >> 5) == 0) {  // heads 0..3 are accumulator rows 0..3: registers 0..3 of the low half
       const int p = wave * 32 + lane;
       const int r = t.r0 + p;
+      const int kpad = (int)tri_bias_ktiles(a.N) * 64;  // keys N..kpad-1 are padding: zero bias
       if (!a.transpose) {
-        // q = o, k = r: consecutive lanes write consecutive keys; pad columns get zeros
-        if (r < a.ldn) {
+        // q = o, k = r
+        if (r < kpad) {
 #pragma unroll
           for (int h = 0; h < H; ++h)
-            a.bias[((int64_t)h * a.N + t.o) * a.ldn + r] = f2bf(t.valid(p) ? acc[0][h] * a.bias_scale : 0.f);
+            a.bias[tri_bias_offset(a.N, h, t.o, r)] = f2bf(t.valid(p) ? acc[0][h] * a.bias_scale : 0.f);
         }
       } else if (t.valid(p)) {
         // q = r, k = o
 #pragma unroll
         for (int h = 0; h < H; ++h) {
-          bf16_t* row = a.bias + ((int64_t)h * a.N + r) * a.ldn;
-          row[t.o] = f2bf(acc[0][h] * a.bias_scale);
+          a.bias[tri_bias_offset(a.N, h, r, t.o)] = f2bf(acc[0][h] * a.bias_scale);
           if (t.o == a.N - 1)
-            for (int k = a.N; k < a.ldn; ++k) row[k] = 0;
+            for (int k = a.N; k < kpad; ++k) a.bias[tri_bias_offset(a.N, h, r, k)] = 0;
         }
       }
     }
@@ -174,19 +182,25 @@ __global__ __launch_bounds__(256, 2) void triattn_proj_kernel(TriAttnProjArgs a)
 constexpr int KT = 64;       // keys per LDS tile
 constexpr int LDK = 56;      // sK row: 32 head-dim + 16 mask k-step + 8 pad (bf16); 112 B
 constexpr int LDV = KT + 4;  // sVt row: 136 B = 34 dwords, so 32 lanes' 8-byte reads hit 32 bank pairs
-constexpr int LDB = KT + 8;  // sB row: 144 B, 16-byte aligned for the 16-byte fragment reads
 constexpr int QW = 128;      // queries per workgroup
 constexpr uint32_t BF16_ONE = 0x3F80u, BF16_NEG_INF = 0xFF80u, BF16_NEG_1E9 = 0xCE6Eu;
 
-// LDS tiles are single-buffered (30 KB): the next tile waits in registers while
-// the current one is consumed, at the price of a second barrier per tile; in
-// exchange three workgroups fit on a CU, and with head dim 32 it is the number
-// of waves available to hide the MFMA -> softmax -> MFMA dependency chain that
-// sets the pace, not the barrier count.
+// One workgroup = (row b, head h, 128 queries); a wave owns 32 queries, lane
+// (j, hh) holds query j's scores for half of the keys of each 32-key tile.
+//
+// S^T = K Q^T runs on the matrix unit with three k-steps: the two halves of the
+// head dimension and a mask step (K column 32 = 0, -1e9 or -inf per key, times a
+// Q entry of 1.0).  The pair bias is added on the matrix unit too,
+// S^T += I * bias^T; its B fragments are 16 contiguous bytes per lane and come
+// straight from global memory, where the bias is stored in fragment order: each
+// load instruction covers one contiguous 1 KB run (the bias is shared by every
+// row b and stays L2-resident), fetched one tile ahead.  Only K and V^T go
+// through LDS, double-buffered (23 KB), with one barrier per tile; three
+// workgroups fit on a CU, and with head dim 32 it is the number of waves
+// available to hide the MFMA -> softmax -> MFMA dependency chain that sets the pace.
 __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
-  __shared__ __attribute__((aligned(16))) bf16_t sK[1][KT * LDK];
-  __shared__ __attribute__((aligned(16))) bf16_t sVt[1][D * LDV];
-  __shared__ __attribute__((aligned(16))) bf16_t sB[1][QW * LDB];
+  __shared__ __attribute__((aligned(16))) bf16_t sK[2][KT * LDK];
+  __shared__ __attribute__((aligned(16))) bf16_t sVt[2][D * LDV];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hh = lane >> 5, j = lane & 31;
@@ -206,6 +220,7 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   const int qw = q0 + wave * 32 + j;
   const int qi = min(qw, N - 1);
   const int64_t bh = (int64_t)b * H + h;
+  const int ldn = (int)a.ldn;
 
   bf16x8 qf[3];
   {
@@ -215,51 +230,49 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
     u32x4 one = {hh == 0 ? BF16_ONE : 0u, 0u, 0u, 0u};
     qf[2] = as_frag(one);
   }
-  // Identity fragments: S^T += I * bias^T adds the pair bias inside the matrix
-  // unit.  A-fragment of k-step `st`: lane (row i = j, half hh) holds
-  // I[i][16 st + 8 hh + e], e = 0..7, i.e. a single 1.0 where 16 st + 8 hh + e == i.
+  // Identity fragments: A-fragment of k-step `st`: lane (row i = j, half hh)
+  // holds I[i][16 st + 8 hh + e], e = 0..7: a single 1.0 where 16 st + 8 hh + e == i.
   bf16x8 idf[2];
 #pragma unroll
   for (int st = 0; st < 2; ++st) {
-    const int e1 = j - 16 * st - 8 * hh;  // position of the 1.0 inside this lane's 8 elements, if any
+    const int e1 = j - 16 * st - 8 * hh;
     uint32_t w[4] = {0u, 0u, 0u, 0u};
     if (e1 >= 0 && e1 < 8) w[e1 >> 1] = (e1 & 1) ? (BF16_ONE << 16) : BF16_ONE;
     idf[st] = as_frag(u32x4{w[0], w[1], w[2], w[3]});
   }
 
-  // loaders, one 16-byte chunk each per tile:
-  //   K   thread (key = tid / 4, c = tid % 4)            + the mask k-step by c < 2
+  // LDS loaders, one 16-byte chunk each per tile:
+  //   K   thread (key = tid / 4, c = tid % 4)   + the mask k-step by c < 2
   //   Vt  thread (d = tid / 8, kc = tid % 8)
-  //   bias: four chunks, idx = tid + 256 i -> (q = idx / 8, kc = idx % 8)
-  // Pointers are set up once and advance by one tile per iteration.
   const int k_key = tid >> 2, k_c = tid & 3;
   const int v_d = tid >> 3, c8 = (tid & 7) * 8;
   const bf16_t* pk = a.k + (bh * N + k_key) * D + k_c * 8;
   const bf16_t* pv = a.vt + (bh * D + v_d) * a.ldn + c8;
   const float* pm = (a.mask && k_c == 0) ? a.mask + (int64_t)b * N + k_key : nullptr;
-  const bf16_t* pb = a.bias ? a.bias + ((int64_t)h * N + q0 + (tid >> 3)) * a.ldn + c8 : nullptr;
-  const int64_t brow = (int64_t)32 * a.ldn;  // bias chunks i and i + 1 are 32 query rows apart
-  bool bq_ok[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) bq_ok[i] = pb != nullptr && q0 + (tid >> 3) + 32 * i < N;
-  const int ldn = (int)a.ldn;
+  // bias B-fragment i = 2 u + st of a tile: keys 32 u + 16 st + 8 hh .. + 8 of this
+  // lane's query.  Queries beyond N have no (initialised) entries and take zeros.
+  const bool has_bias = a.bias != nullptr;
+  const bool lane_bias = has_bias && qw < N;
+  const bf16_t* pb = lane_bias ? a.bias + tri_bias_offset(N, h, qw, 8 * hh) : nullptr;
 
   u32x4 rk, rv, rb[4];
   uint32_t rmask;
-  auto gload = [&](int k0) {
+  auto gload_kv = [&](int k0) {
     const u32x4 z = {0, 0, 0, 0};
     const bool key_ok = k0 + k_key < N;
     rk = key_ok ? *reinterpret_cast<const u32x4*>(pk) : z;
     rmask = key_ok ? 0u : BF16_NEG_INF;
     if (pm && key_ok && *pm == 0.f) rmask = BF16_NEG_1E9;
-    const bool col_ok = k0 + c8 < ldn;
-    rv = col_ok ? *reinterpret_cast<const u32x4*>(pv) : z;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) rb[i] = (bq_ok[i] && col_ok) ? *reinterpret_cast<const u32x4*>(pb + i * brow) : z;
+    rv = k0 + c8 < ldn ? *reinterpret_cast<const u32x4*>(pv) : z;
     pk += KT * D;
     pv += KT;
     if (pm) pm += KT;
-    if (pb) pb += KT;
+  };
+  auto gload_bias = [&]() {
+    const u32x4 z = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rb[i] = lane_bias ? *reinterpret_cast<const u32x4*>(pb + 512 * i) : z;
+    if (lane_bias) pb += 2048;
   };
   auto sstore = [&](int buf) {
     *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + k_c * 8]) = rk;
@@ -271,9 +284,6 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
     u32x2* pvs = reinterpret_cast<u32x2*>(&sVt[buf][v_d * LDV + c8]);
     pvs[0] = u32x2{rv.x, rv.y};
     pvs[1] = u32x2{rv.z, rv.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      *reinterpret_cast<u32x4*>(&sB[buf][((tid >> 3) + 32 * i) * LDB + c8]) = rb[i];
   };
 
   f32x16 o;
@@ -282,13 +292,15 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   float m_run = -__builtin_huge_valf(), l_run = 0.f;
 
   const int nkt = (N + KT - 1) / KT;
-  gload(0);
+  gload_kv(0);
+  gload_bias();
   sstore(0);
   lds_barrier();
 
   for (int kt = 0; kt < nkt; ++kt) {
-    constexpr int buf = 0;
-    if (kt + 1 < nkt) gload((kt + 1) * KT);
+    const int buf = kt & 1;
+    const bool more = kt + 1 < nkt;
+    if (more) gload_kv((kt + 1) * KT);
     // Both 32-key halves of the tile go through the matrix unit first (two
     // independent accumulator chains), then one online-softmax update covers
     // all 64 keys, then both halves feed O.  A half that lies wholly beyond N
@@ -299,14 +311,16 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
     for (int u = 0; u < 2; ++u) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[u][r] = 0.f;
-      const bf16_t* bp = &sB[buf][(wave * 32 + j) * LDB + u * 32 + 8 * hh];
-#pragma unroll
-      for (int st = 0; st < 2; ++st)
-        s[u] = mfma32(idf[st], as_frag(*reinterpret_cast<const u32x4*>(bp + 16 * st)), s[u]);
+      if (has_bias) {
+        s[u] = mfma32(idf[0], as_frag(rb[2 * u]), s[u]);
+        s[u] = mfma32(idf[1], as_frag(rb[2 * u + 1]), s[u]);
+      }
 #pragma unroll
       for (int ks = 0; ks < 3; ++ks)
         s[u] = mfma32(lds_frag(sK[buf], LDK, u * 32, ks * 16, lane), qf[ks], s[u]);
     }
+    // this tile's bias fragments are consumed: request the next tile's
+    if (more) gload_bias();
     float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
 #pragma unroll
     for (int u = 0; u < 2; ++u)
@@ -347,9 +361,10 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
         vv.x = lo.x; vv.y = lo.y; vv.z = hi.x; vv.w = hi.y;
         o = mfma32(as_frag(vv), pf[u][half], o);
       }
-    if (kt + 1 < nkt) {
-      lds_barrier();  // every wave is done reading this tile
-      sstore(0);
+    if (more) {
+      // buffer buf ^ 1 was last read in the previous iteration, which every
+      // wave left through the barrier below
+      sstore(buf ^ 1);
       lds_barrier();
     }
   }

@@ -337,12 +337,26 @@ def triangle_contraction(a, b, out=None):
     return out
 
 
+def pack_pair_bias(bias):
+    """[4, N, >=N] pair bias (already multiplied by log2(e)) -> the MFMA-fragment
+    order the attention core reads: [4, ceil(N/32), ceil(N/64), 4, 32, 16] bf16 with
+    packed[h, qb, kt, i, j, c] = bias[h, 32 qb + j, 64 kt + 16 i + c], zero where
+    the query or key index is >= N."""
+    if bias.dim() != 3 or bias.shape[0] != 4 or bias.shape[2] < bias.shape[1]:
+        raise ValueError("bias: expected [4, N, >=N]")
+    n = bias.shape[1]
+    qb, kt = (n + 31) // 32, (n + 63) // 64
+    full = torch.zeros((4, qb * 32, kt * 64), dtype=torch.bfloat16, device=bias.device)
+    full[:, :n, :n] = bias[:, :, :n].to(torch.bfloat16)
+    return full.view(4, qb, 32, kt, 4, 16).permute(0, 1, 3, 4, 2, 5).contiguous()
+
+
 def grid_attention_core(q, k, vt, g, pair_bias, mask, out=None):
     """The flash-attention stage of the triangle attention on projected, head-major
     bf16 operands in base-2 form: q, k, g [N, 4, N, 32] (q and the bias
-    pre-multiplied by log2(e); g = sigmoid gate), vt [N, 4, 32, ld], pair_bias
-    [4, N, ld] or None, ld = N rounded up to 8 with zero padding.  Returns the
-    gated output [N*N, 128] bf16."""
+    pre-multiplied by log2(e); g = sigmoid gate), vt [N, 4, 32, ld] with ld = N
+    rounded up to 8 and zero padding, pair_bias from pack_pair_bias() or None.
+    Returns the gated output [N*N, 128] bf16."""
     lib = _L.load()
     _gpu(q, "q", torch.bfloat16)
     if q.dim() != 4 or q.shape[1] != 4 or q.shape[3] != 32 or q.shape[0] != q.shape[2]:
@@ -353,7 +367,7 @@ def grid_attention_core(q, k, vt, g, pair_bias, mask, out=None):
     _gpu(g, "g", torch.bfloat16, q.shape)
     _gpu(vt, "vt", torch.bfloat16, (n, 4, 32, ld))
     if pair_bias is not None:
-        _gpu(pair_bias, "pair_bias", torch.bfloat16, (4, n, ld))
+        _gpu(pair_bias, "pair_bias", torch.bfloat16, (4, (n + 31) // 32, (n + 63) // 64, 4, 32, 16))
     maskf = _mask_f32(mask, (n, n), "mask")
     if out is None:
         out = torch.empty((n * n, 128), dtype=torch.bfloat16, device=q.device)

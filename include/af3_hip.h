@@ -227,7 +227,11 @@ int af3_linear_forward(
  *   rounded up to 8):
  *     q  [b][h][s][32] = query * log2(e)/sqrt(32);  k, g [b][h][s][32] (g = sigmoid gate);
  *     vt [b][h][32][ld] = value transposed, columns n_token..ld-1 zero;
- *     pair_bias [h][q][ld] = bias * log2(e), pad columns zero, or NULL;
+ *     pair_bias = bias * log2(e) in MFMA-fragment order, or NULL: element (h, q, k) at
+ *       ((((h*QB + q/32)*KT + k/64)*4 + (k%64)/16)*32 + q%32)*16 + k%16,
+ *       QB = ceil(N/32), KT = ceil(N/64), 4*QB*KT*2048 elements, keys >= N zero
+ *       (per head, 32-query block and 64-key tile: four contiguous 1 KB runs, each
+ *       the B operand of one identity-matrix MFMA that adds the bias to the logits);
  *   key mask [N][N] fp32 0/1 or NULL;
  *   og [(b*N + s)][128] = gate * softmax(q k^T + bias) v.
  */

@@ -436,7 +436,8 @@ def test_kernel_level_attention_core(gpu_pkg, n):
     vt = torch.zeros(n, 4, 32, npad)
     vt[..., :n] = hm(2).transpose(-1, -2)
     t = lambda x: x.to(dev()).bfloat16()
-    og = gpu_pkg.ops.grid_attention_core(t(hm(0)), t(hm(1)), t(vt), t(hm(3)), t(bias), mask.to(dev()))
+    og = gpu_pkg.ops.grid_attention_core(t(hm(0)), t(hm(1)), t(vt), t(hm(3)),
+                                         gpu_pkg.ops.pack_pair_bias(t(bias)), mask.to(dev()))
     q, k, v, gt = (qkvg[:, :, i].permute(0, 2, 1, 3).double() for i in range(4))   # [b, h, s, d]
     logits = (q @ k.transpose(-1, -2) + bias[None, :, :, :n].double()) / log2e
     logits = logits.masked_fill(mask[:, None, None, :] == 0, -1e9)
