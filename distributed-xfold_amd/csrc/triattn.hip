@@ -198,6 +198,7 @@ constexpr uint32_t BF16_ONE = 0x3F80u, BF16_NEG_INF = 0xFF80u, BF16_NEG_1E9 = 0x
 // through LDS, double-buffered (23 KB), with one barrier per tile; three
 // workgroups fit on a CU, and with head dim 32 it is the number of waves
 // available to hide the MFMA -> softmax -> MFMA dependency chain that sets the pace.
+template <bool HAS_BIAS>
 __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t sK[2][KT * LDK];
   __shared__ __attribute__((aligned(16))) bf16_t sVt[2][D * LDV];
@@ -246,44 +247,56 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   //   Vt  thread (d = tid / 8, kc = tid % 8)
   const int k_key = tid >> 2, k_c = tid & 3;
   const int v_d = tid >> 3, c8 = (tid & 7) * 8;
-  const bf16_t* pk = a.k + (bh * N + k_key) * D + k_c * 8;
-  const bf16_t* pv = a.vt + (bh * D + v_d) * a.ldn + c8;
-  const float* pm = (a.mask && k_c == 0) ? a.mask + (int64_t)b * N + k_key : nullptr;
-  // bias B-fragment i = 2 u + st of a tile: keys 32 u + 16 st + 8 hh .. + 8 of this
-  // lane's query.  Queries beyond N have no (initialised) entries and take zeros.
-  const bool has_bias = a.bias != nullptr;
-  const bool lane_bias = has_bias && qw < N;
-  const bf16_t* pb = lane_bias ? a.bias + tri_bias_offset(N, h, qw, 8 * hh) : nullptr;
-
-  u32x4 rk, rv, rb[4];
-  uint32_t rmask;
+  // All global loads are unconditional, from clamped addresses, and nothing is
+  // decided from a loaded value until the LDS store one tile later: a load
+  // under a lane mask, or a value inspected right after its load, would put a
+  // full memory round trip (behind every load queued before it) into each tile.
+  // Addresses are a wave-uniform 64-bit base plus a 32-bit lane offset.
+  u32x4 rk, rv, rb[4];  // rb: bias fragments, fetched one tile ahead
+  float rm = 1.f;
+  bool key_ok = false, col_ok = false;
+  const char* kbase = reinterpret_cast<const char*>(a.k + bh * N * D);
+  const char* vbase = reinterpret_cast<const char*>(a.vt + bh * D * a.ldn);
+  const char* mbase = reinterpret_cast<const char*>(a.mask ? a.mask + (int64_t)b * N : nullptr);
+  const uint32_t v_row = (uint32_t)(v_d * ldn) * 2u;
   auto gload_kv = [&](int k0) {
-    const u32x4 z = {0, 0, 0, 0};
-    const bool key_ok = k0 + k_key < N;
-    rk = key_ok ? *reinterpret_cast<const u32x4*>(pk) : z;
-    rmask = key_ok ? 0u : BF16_NEG_INF;
-    if (pm && key_ok && *pm == 0.f) rmask = BF16_NEG_1E9;
-    rv = k0 + c8 < ldn ? *reinterpret_cast<const u32x4*>(pv) : z;
-    pk += KT * D;
-    pv += KT;
-    if (pm) pm += KT;
+    key_ok = k0 + k_key < N;
+    col_ok = k0 + c8 < ldn;
+    const uint32_t key = (uint32_t)min(k0 + k_key, N - 1);
+    rk = *reinterpret_cast<const u32x4*>(kbase + (key * (D * 2u) + k_c * 16u));
+    if (mbase) rm = *reinterpret_cast<const float*>(mbase + key * 4u);
+    rv = *reinterpret_cast<const u32x4*>(vbase + (v_row + (col_ok ? (uint32_t)(k0 + c8) * 2u : 0u)));
   };
-  auto gload_bias = [&]() {
-    const u32x4 z = {0, 0, 0, 0};
+  // bias B-fragment i = 2 u + st of a tile: keys 32 u + 16 st + 8 hh .. + 8 of this
+  // lane's query.  A query beyond N reads its (uninitialised) slot of the padded
+  // block, or block 0 if its whole block lies beyond N; whatever it reads only
+  // reaches its own, discarded, column of S.
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int qblock = q0 + wave_u * 32 < N ? (q0 >> 5) + wave_u : 0;
+  const char* bbase = HAS_BIAS ? reinterpret_cast<const char*>(a.bias + tri_bias_offset(N, h, qblock * 32, 0)) : nullptr;
+  const uint32_t b_lane = (uint32_t)(j * 16 + 8 * hh) * 2u;
+  const int bias_tiles = (int)tri_bias_ktiles(N);
+  int bias_next = 0;  // tile the next gload_bias fetches; stops at the last one
+  auto gload_bias = [&](u32x4* dst) {
+    if (!HAS_BIAS) return;
+    const char* p = bbase + (size_t)min(bias_next, bias_tiles - 1) * 4096u;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) rb[i] = lane_bias ? *reinterpret_cast<const u32x4*>(pb + 512 * i) : z;
-    if (lane_bias) pb += 2048;
+    for (int i = 0; i < 4; ++i) dst[i] = *reinterpret_cast<const u32x4*>(p + (b_lane + 1024u * i));
+    ++bias_next;
   };
   auto sstore = [&](int buf) {
-    *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + k_c * 8]) = rk;
+    const u32x4 z = {0, 0, 0, 0};
+    *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + k_c * 8]) = key_ok ? rk : z;
     if (k_c < 2) {
+      const uint32_t rmask = !key_ok ? BF16_NEG_INF : (rm == 0.f ? BF16_NEG_1E9 : 0u);
       u32x4 m = {k_c == 0 ? rmask : 0u, 0u, 0u, 0u};
       *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + 32 + k_c * 8]) = m;
     }
     // rows of sVt are 8-byte aligned only: two 8-byte stores
+    const u32x4 v = col_ok ? rv : z;
     u32x2* pvs = reinterpret_cast<u32x2*>(&sVt[buf][v_d * LDV + c8]);
-    pvs[0] = u32x2{rv.x, rv.y};
-    pvs[1] = u32x2{rv.z, rv.w};
+    pvs[0] = u32x2{v.x, v.y};
+    pvs[1] = u32x2{v.z, v.w};
   };
 
   f32x16 o;
@@ -293,14 +306,13 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
 
   const int nkt = (N + KT - 1) / KT;
   gload_kv(0);
-  gload_bias();
+  gload_bias(rb);
   sstore(0);
   lds_barrier();
 
   for (int kt = 0; kt < nkt; ++kt) {
     const int buf = kt & 1;
     const bool more = kt + 1 < nkt;
-    if (more) gload_kv((kt + 1) * KT);
     // Both 32-key halves of the tile go through the matrix unit first (two
     // independent accumulator chains), then one online-softmax update covers
     // all 64 keys, then both halves feed O.  A half that lies wholly beyond N
@@ -311,7 +323,7 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
     for (int u = 0; u < 2; ++u) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[u][r] = 0.f;
-      if (has_bias) {
+      if (HAS_BIAS) {
         s[u] = mfma32(idf[0], as_frag(rb[2 * u]), s[u]);
         s[u] = mfma32(idf[1], as_frag(rb[2 * u + 1]), s[u]);
       }
@@ -319,8 +331,12 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
       for (int ks = 0; ks < 3; ++ks)
         s[u] = mfma32(lds_frag(sK[buf], LDK, u * 32, ks * 16, lane), qf[ks], s[u]);
     }
-    // this tile's bias fragments are consumed: request the next tile's
-    if (more) gload_bias();
+    // Global loads are issued here, behind the score MFMAs: the bias registers
+    // are free again, and the K / V loads come first so that their consumer (the
+    // LDS store at the end of this tile) does not have to wait for the bias
+    // loads queued behind them (vector memory operations retire in order).
+    gload_kv((kt + 1) * KT);
+    gload_bias(rb);
     float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
 #pragma unroll
     for (int u = 0; u < 2; ++u)
@@ -373,12 +389,14 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   if (qw >= N) return;
   const bf16_t* gp = a.g + (bh * N + qw) * D + 4 * hh;
   bf16_t* op = a.og + ((int64_t)b * N + qw) * 128 + h * D + 4 * hh;
+  u32x2 gw[4];  // all gate loads before the first store (which they could alias as far as the compiler knows)
+#pragma unroll
+  for (int g = 0; g < 4; ++g) gw[g] = *reinterpret_cast<const u32x2*>(gp + 8 * g);
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    const u32x2 gw = *reinterpret_cast<const u32x2*>(gp + 8 * g);
     u32x2 w;
-    w.x = pack2bf(o[4 * g] * inv * bflo(gw.x), o[4 * g + 1] * inv * bfhi(gw.x));
-    w.y = pack2bf(o[4 * g + 2] * inv * bflo(gw.y), o[4 * g + 3] * inv * bfhi(gw.y));
+    w.x = pack2bf(o[4 * g] * inv * bflo(gw[g].x), o[4 * g + 1] * inv * bfhi(gw[g].x));
+    w.y = pack2bf(o[4 * g + 2] * inv * bflo(gw[g].y), o[4 * g + 3] * inv * bfhi(gw[g].y));
     *reinterpret_cast<u32x2*>(op + 8 * g) = w;
   }
 }
@@ -408,6 +426,7 @@ int launch_triattn_flash(const TriAttnArgs& a, hipStream_t stream) {
   const int64_t total = (int64_t)((a.N + QW - 1) / QW) * H * a.N;
   const int64_t blocks = (total + 7) / 8 * 8;
   if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
-  hipLaunchKernelGGL(triattn_flash_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  if (a.bias) hipLaunchKernelGGL(triattn_flash_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL(triattn_flash_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
   return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }
