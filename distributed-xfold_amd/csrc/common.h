@@ -64,6 +64,12 @@ template <> struct Elem<bf16_t> {
   }
   static __device__ __forceinline__ float load(const bf16_t* p) { return bf2f(*p); }
   static __device__ __forceinline__ void store(bf16_t* p, float v) { *p = f2bf(v); }
+  // 8 elements as loaded, conversion deferred: lets a kernel put a batch of
+  // loads in flight before the first value is touched
+  struct Raw { u32x4 v; };
+  static constexpr int kBatch = 8;  // 8-element groups to keep in flight at a time (4 VGPRs each)
+  static __device__ __forceinline__ Raw load_raw(const bf16_t* p) { return Raw{*reinterpret_cast<const u32x4*>(p)}; }
+  static __device__ __forceinline__ void unpack_raw(const Raw& r, float* f) { unpack8(r.v, f); }
 };
 template <> struct Elem<float> {
   static __device__ __forceinline__ void load8(const float* p, float* f) {
@@ -79,6 +85,15 @@ template <> struct Elem<float> {
   }
   static __device__ __forceinline__ float load(const float* p) { return *p; }
   static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+  struct Raw { f32x4 a, b; };
+  static constexpr int kBatch = 4;  // 8 VGPRs per group
+  static __device__ __forceinline__ Raw load_raw(const float* p) {
+    return Raw{*reinterpret_cast<const f32x4*>(p), *reinterpret_cast<const f32x4*>(p + 4)};
+  }
+  static __device__ __forceinline__ void unpack_raw(const Raw& r, float* f) {
+    f[0] = r.a.x; f[1] = r.a.y; f[2] = r.a.z; f[3] = r.a.w;
+    f[4] = r.b.x; f[5] = r.b.y; f[6] = r.b.z; f[7] = r.b.w;
+  }
 };
 
 // sigmoid through the hardware exp2 / reciprocal (about 1 ulp each): four

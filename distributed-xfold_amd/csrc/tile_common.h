@@ -30,50 +30,61 @@ __device__ __forceinline__ Tile make_tile(int N, bool column_mode) {
   return t;
 }
 
+// Eight consecutive fp32 parameters (LayerNorm weight / bias slice of a thread),
+// or a constant when the pointer is null.
+__device__ __forceinline__ void load_param8(const float* p, float fill, float* out) {
+  if (p) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p);
+    const f32x4 b = *reinterpret_cast<const f32x4*>(p + 4);
+    out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+    out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = fill;
+  }
+}
+
 // LayerNorm of a tile of pixels from global memory into sX[p][c] (bf16).
 // Thread (prow = tid / 16, chunk = tid % 16) handles channels 8*chunk..+7 of
 // pixels prow, prow + 16, ...; 16 lanes cooperate on one pixel's statistics.
-// Out-of-range pixels become zero rows.
+// Out-of-range pixels become zero rows.  The loads of a batch of pixels are
+// unconditional (an out-of-range pixel re-reads the tile's first one) and all
+// issued before any value is converted: a load under a lane mask, or one whose
+// value is touched at once, costs a full memory round trip per pixel.
 template <typename TIO>
 __device__ __forceinline__ void load_ln_tile(const TIO* x, const Tile& t, const float* lnw,
                                              const float* lnb, bf16_t* sX, int tid, bool skip_ln = false) {
+  using E = Elem<TIO>;
+  constexpr int NB = E::kBatch;
   const int chunk = tid & 15, prow = tid >> 4;
   float w[8], b[8];
+  load_param8(lnw ? lnw + chunk * 8 : nullptr, 1.f, w);
+  load_param8(lnb ? lnb + chunk * 8 : nullptr, 0.f, b);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    w[e] = lnw ? lnw[chunk * 8 + e] : 1.f;
-    b[e] = lnb ? lnb[chunk * 8 + e] : 0.f;
-  }
-  // two batches of four pixels per thread: the global loads of a batch are all
-  // in flight before its statistics start, at half the registers of one batch of eight
+  for (int base = 0; base < 8; base += NB) {
+    typename E::Raw raw[NB];
 #pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    float v[4][8];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int p = (half * 4 + i) * 16 + prow;
-      if (t.valid(p)) {
-        Elem<TIO>::load8(x + t.pix(p) * C + chunk * 8, v[i]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[i][e] = 0.f;
-      }
+    for (int i = 0; i < NB; ++i) {
+      const int p = (base + i) * 16 + prow;
+      raw[i] = E::load_raw(x + t.pix(t.valid(p) ? p : 0) * C + chunk * 8);
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int p = (half * 4 + i) * 16 + prow;
+    for (int i = 0; i < NB; ++i) {
+      const int p = (base + i) * 16 + prow;
+      float v[8];
+      E::unpack_raw(raw[i], v);
       float s = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) s += v[i][e];
+      for (int e = 0; e < 8; ++e) s += v[e];
       const float mean = group16_sum(s) * (1.f / C);
       float q = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) { const float d = v[i][e] - mean; q += d * d; }
+      for (int e = 0; e < 8; ++e) { const float d = v[e] - mean; q += d * d; }
       const float rstd = rsqrtf(group16_sum(q) * (1.f / C) + LN_EPS);
       float o[8];
       const bool ok = t.valid(p);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] = ok ? (skip_ln ? v[i][e] : (v[i][e] - mean) * rstd * w[e] + b[e]) : 0.f;
+      for (int e = 0; e < 8; ++e) o[e] = ok ? (skip_ln ? v[e] : (v[e] - mean) * rstd * w[e] + b[e]) : 0.f;
       *reinterpret_cast<u32x4*>(sX + p * LDX + chunk * 8) = pack8(o);
     }
   }
@@ -82,6 +93,9 @@ __device__ __forceinline__ void load_ln_tile(const TIO* x, const Tile& t, const 
 // In-place LayerNorm of the rows of sX (bf16 in LDS), same thread mapping.
 __device__ __forceinline__ void ln_inplace_tile(bf16_t* sX, const float* lnw, const float* lnb, int tid) {
   const int chunk = tid & 15, prow = tid >> 4;
+  float w[8], b[8];
+  load_param8(lnw + chunk * 8, 1.f, w);
+  load_param8(lnb + chunk * 8, 0.f, b);
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
     const int p = it * 16 + prow;
@@ -97,7 +111,7 @@ __device__ __forceinline__ void ln_inplace_tile(bf16_t* sX, const float* lnw, co
     const float rstd = rsqrtf(group16_sum(q) * (1.f / C) + LN_EPS);
     float o[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) o[e] = (v[e] - mean) * rstd * lnw[chunk * 8 + e] + lnb[chunk * 8 + e];
+    for (int e = 0; e < 8; ++e) o[e] = (v[e] - mean) * rstd * w[e] + b[e];
     *reinterpret_cast<u32x4*>(sX + p * LDX + chunk * 8) = pack8(o);
   }
 }
@@ -162,26 +176,40 @@ __device__ __forceinline__ void stage_t_bf16(const f32x16* acc, bf16_t* sS, int 
     }
 }
 
-// Staged fp32 tile -> residual stream: out[pix] = (res ? res[pix] : 0) + tile
+// Staged fp32 tile -> residual stream: out[pix] = (res ? res[pix] : 0) + tile.
+// The residual rows of a batch of pixels are loaded (unconditionally, from a
+// clamped pixel) before the batch's first store: out may alias res, so the
+// compiler cannot move a load above a store on its own.
 template <typename TIO>
 __device__ __forceinline__ void store_tile_f32(const float* sS, const Tile& t, TIO* out, const TIO* res, int tid) {
+  using E = Elem<TIO>;
+  constexpr int NB = E::kBatch;
   const int chunk = tid & 15, prow = tid >> 4;
 #pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int p = it * 16 + prow;
-    if (!t.valid(p)) continue;
-    float v[8];
-    const f32x4 a = *reinterpret_cast<const f32x4*>(sS + p * LDS_F + chunk * 8);
-    const f32x4 b = *reinterpret_cast<const f32x4*>(sS + p * LDS_F + chunk * 8 + 4);
-    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-    const int64_t off = t.pix(p) * C + chunk * 8;
+  for (int base = 0; base < 8; base += NB) {
+    typename E::Raw raw[NB];
     if (res) {
-      float rr[8];
-      Elem<TIO>::load8(res + off, rr);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] += rr[e];
+      for (int i = 0; i < NB; ++i) {
+        const int p = (base + i) * 16 + prow;
+        raw[i] = E::load_raw(res + t.pix(t.valid(p) ? p : 0) * C + chunk * 8);
+      }
     }
-    Elem<TIO>::store8(out + off, v);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int p = (base + i) * 16 + prow;
+      float v[8];
+      const f32x4 a = *reinterpret_cast<const f32x4*>(sS + p * LDS_F + chunk * 8);
+      const f32x4 b = *reinterpret_cast<const f32x4*>(sS + p * LDS_F + chunk * 8 + 4);
+      v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+      if (res) {
+        float rr[8];
+        E::unpack_raw(raw[i], rr);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += rr[e];
+      }
+      if (t.valid(p)) E::store8(out + t.pix(p) * C + chunk * 8, v);
+    }
   }
 }
 
