@@ -182,7 +182,7 @@ def main():
     ms_contract = gpu_time_ms(lambda: pkg.ops.triangle_contraction(a, b, t_buf), it)
     ms_attn = gpu_time_ms(lambda: pkg.ops.grid_attention_core(q_, k_, vt_, g_, nb, pair_mask, og), it)
     kernels = {
-        "gemm_nt_kernel (triangle contraction)": (ms_contract, flops_contraction(n)),
+        "contract_kernel (triangle contraction)": (ms_contract, flops_contraction(n)),
         "triattn_flash_kernel (triangle attention core)": (ms_attn, flops_attention_core(n)),
     }
     dom = max(kernels, key=lambda k: kernels[k][0])      # each runs twice per block

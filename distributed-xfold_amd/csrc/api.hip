@@ -46,6 +46,14 @@ const char* af3_error_string(int code) {
 }
 
 // ------------------------------------------------------ triangle multiplication
+// The N x N x N contraction of the triangle multiplication: the 256x256-tile
+// kernel once a token count fills at least part of a second 128-row tile,
+// the general 128x128-tile GEMM below that.
+static int contraction(const GemmArgs& g, hipStream_t s) {
+  if (g.M > 128 && contract_supported(g)) return launch_contract(g, s);
+  return launch_gemm_nt(g, s);
+}
+
 size_t af3_triangle_multiplication_workspace_bytes(int64_t n) {
   if (n <= 0) return 0;
   return 3 * align_up((size_t)C_PAIR * n * pad8(n) * sizeof(bf16_t), 256);
@@ -87,7 +95,7 @@ int af3_triangle_multiplication_forward(
   g.M = g.N = (int)n; g.K = (int)np; g.batch = C_PAIR;
   g.lda = g.ldb = g.ldc = np;
   g.sA = g.sB = g.sC = n * np;
-  rc = launch_gemm_nt(g, s);
+  rc = contraction(g, s);
   if (rc) return rc;
   return launch_trimul_epilogue(a, s);
 }
@@ -354,7 +362,7 @@ int af3_triangle_contraction_forward(
   g.M = g.N = (int)n; g.K = (int)np; g.batch = C_PAIR;
   g.lda = g.ldb = g.ldc = np;
   g.sA = g.sB = g.sC = n * np;
-  return launch_gemm_nt(g, static_cast<hipStream_t>(stream));
+  return contraction(g, static_cast<hipStream_t>(stream));
 }
 
 int af3_grid_attention_core_forward(

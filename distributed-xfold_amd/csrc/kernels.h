@@ -28,6 +28,9 @@ struct GemmArgs {
   int vec_ok = 0, res_vec_ok = 0;  // set by launch_gemm_nt: rows aligned for 16-byte stores / loads
 };
 int launch_gemm_nt(const GemmArgs& g, hipStream_t stream);
+// contract.hip: the same product, plain bf16 output, 256x256 tiles (large M, N)
+bool contract_supported(const GemmArgs& g);
+int launch_contract(const GemmArgs& g, hipStream_t stream);
 
 // ---------------------------------------------------------------- rowops.hip
 // y = LN(x) [* weight + bias] ; then, if scale: y = sigmoid(scale[r]) * y + shift[r]

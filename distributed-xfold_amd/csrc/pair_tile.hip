@@ -243,18 +243,28 @@ __global__ __launch_bounds__(256) void attn_out_kernel(AttnOutArgs a) {
   float* sS = reinterpret_cast<float*>(smem);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const Tile t = make_tile(a.N, a.transpose != 0);  // where the result lands in the pair tensor
-  {
-    const int ck = tid & 15, prow = tid >> 4;
+  // Everything the tile needs is requested up front, unconditionally (rows past
+  // the end re-read a valid one and are zeroed / skipped later): the gated
+  // attention output, the output weights and the residual rows.
+  const int ck = tid & 15, prow = tid >> 4;
+  u32x4 og[8];
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      const int p = it * 16 + prow;
-      u32x4 v = {0, 0, 0, 0};
-      if (t.valid(p))
-        v = *reinterpret_cast<const u32x4*>(a.og + ((int64_t)t.o * a.N + t.r0 + p) * a.ld_og + ck * 8);
-      *reinterpret_cast<u32x4*>(sX + p * LDX + ck * 8) = v;
-    }
+  for (int it = 0; it < 8; ++it) {
+    const int p = it * 16 + prow;
+    og[it] = *reinterpret_cast<const u32x4*>(a.og + ((int64_t)t.o * a.N + t.r0 + (t.valid(p) ? p : 0)) * a.ld_og + ck * 8);
   }
-  load_w_rows(a.w_out, sW, TM, tid);
+  WChunkRegs wr;
+  wr.load(a.w_out, tid);
+  const bool add = a.residual != 0;
+  typename Elem<TIO>::Raw res[8];
+  prefetch_tile_rows<TIO>(reinterpret_cast<const TIO*>(add ? a.pair : a.out), t, tid, res);
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int p = it * 16 + prow;
+    const u32x4 z = {0, 0, 0, 0};
+    *reinterpret_cast<u32x4*>(sX + p * LDX + ck * 8) = t.valid(p) ? og[it] : z;
+  }
+  wr.store(sW, tid);
   lds_barrier();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
@@ -263,8 +273,7 @@ __global__ __launch_bounds__(256) void attn_out_kernel(AttnOutArgs a) {
   lds_barrier();
   stage_t_f32(acc, sS, wave, lane);
   lds_barrier();
-  store_tile_f32<TIO>(sS, t, reinterpret_cast<TIO*>(a.out),
-                      a.residual ? reinterpret_cast<const TIO*>(a.pair) : nullptr, tid);
+  store_tile_f32_pre<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), res, add, tid);
 }
 
 // ============================================================================

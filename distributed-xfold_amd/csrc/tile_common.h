@@ -214,6 +214,35 @@ __device__ __forceinline__ void store_tile_f32(const float* sS, const Tile& t, T
 }
 
 
+// The same with the residual rows fetched by the caller ahead of time
+// (prefetch_tile_rows at kernel entry, so their latency hides behind the MFMAs).
+template <typename TIO>
+__device__ __forceinline__ void prefetch_tile_rows(const TIO* src, const Tile& t, int tid, typename Elem<TIO>::Raw* raw) {
+  const int chunk = tid & 15, prow = tid >> 4;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int p = i * 16 + prow;
+    raw[i] = Elem<TIO>::load_raw(src + t.pix(t.valid(p) ? p : 0) * C + chunk * 8);
+  }
+}
+template <typename TIO>
+__device__ __forceinline__ void store_tile_f32_pre(const float* sS, const Tile& t, TIO* out,
+                                                   const typename Elem<TIO>::Raw* raw, bool add, int tid) {
+  const int chunk = tid & 15, prow = tid >> 4;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int p = i * 16 + prow;
+    float v[8], rr[8];
+    const f32x4 a = *reinterpret_cast<const f32x4*>(sS + p * LDS_F + chunk * 8);
+    const f32x4 b = *reinterpret_cast<const f32x4*>(sS + p * LDS_F + chunk * 8 + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    Elem<TIO>::unpack_raw(raw[i], rr);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] += add ? rr[e] : 0.f;
+    if (t.valid(p)) Elem<TIO>::store8(out + t.pix(p) * C + chunk * 8, v);
+  }
+}
+
 // 128 x 128 bf16 weight chunk held in registers between a global load and the
 // LDS store, so the load overlaps the MFMA work on the previous chunk.
 struct WChunkRegs {
