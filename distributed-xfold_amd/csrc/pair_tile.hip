@@ -279,7 +279,8 @@ __global__ __launch_bounds__(256) void attn_out_kernel(AttnOutArgs a) {
 // ============================================================================
 // SwiGLU transition, c = 128, hidden = 128 * factor, all in one kernel
 // ============================================================================
-constexpr int LDW2 = 72;  // LDS row stride (bf16) of a [128 out][64 hidden] W2 slab
+constexpr int LDW2 = 68;  // LDS row stride (bf16) of a [128 out][64 hidden] W2 slab: 136 B = 34 dwords, so
+                          // the 32 rows of an 8-byte fragment read fall on 32 different bank pairs
 
 template <typename TIO>
 __global__ __launch_bounds__(256, 2) void transition_kernel(TransitionArgs a) {
@@ -322,7 +323,10 @@ __global__ __launch_bounds__(256, 2) void transition_kernel(TransitionArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int idx = tid + 256 * i;
-      *reinterpret_cast<u32x4*>(sW2 + (idx >> 3) * LDW2 + (idx & 7) * 8) = w2r[i];
+      // rows are 8-byte aligned only: two 8-byte stores
+      u32x2* dst = reinterpret_cast<u32x2*>(sW2 + (idx >> 3) * LDW2 + (idx & 7) * 8);
+      dst[0] = u32x2{w2r[i].x, w2r[i].y};
+      dst[1] = u32x2{w2r[i].z, w2r[i].w};
     }
   };
   fetch(0);
