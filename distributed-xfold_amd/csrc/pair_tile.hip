@@ -99,6 +99,7 @@ __global__ __launch_bounds__(256, 2) void trimul_epilogue_kernel(TriMulArgs a) {
   bf16_t* sW = smem + TM * LDX;
   float* sS = reinterpret_cast<float*>(smem);  // [TM][LDS_F] fp32 over both, after the last MFMA
   static_assert(TM * LDS_F * 4 <= 2 * TM * LDX * 2, "staging tile must fit");
+  __shared__ __attribute__((aligned(16))) float sP[2 * C];  // center LayerNorm weight | bias
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const Tile t = make_tile(a.N, false);
   const TIO* x = reinterpret_cast<const TIO*>(a.pair);
@@ -108,12 +109,12 @@ __global__ __launch_bounds__(256, 2) void trimul_epilogue_kernel(TriMulArgs a) {
   wr.load(a.w_gl, tid);
   u32x4 rt[8];  // contraction result t[c][i][j0 + 8 pc ..], c = 16 it + tid / 16
   const int pc = tid & 15, crow = tid >> 4;
-  const int nvalid = min(max(a.N - (t.r0 + pc * 8), 0), 8);
+  // (a chunk that starts past the row's end re-reads the tile's first one; its pixels are zeroed later)
+  const int j_chunk = t.r0 + pc * 8 < a.Np ? t.r0 + pc * 8 : t.r0;
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
     const int c = it * 16 + crow;
-    const u32x4 z = {0, 0, 0, 0};
-    rt[it] = nvalid > 0 ? *reinterpret_cast<const u32x4*>(a.t_buf + ((int64_t)c * a.N + t.o) * a.Np + t.r0 + pc * 8) : z;
+    rt[it] = *reinterpret_cast<const u32x4*>(a.t_buf + ((int64_t)c * a.N + t.o) * a.Np + j_chunk);
   }
 
   // 1. output gate from the LayerNorm-ed input: sigmoid(LN(x) Wgl^T), T form, kept in registers
@@ -131,23 +132,59 @@ __global__ __launch_bounds__(256, 2) void trimul_epilogue_kernel(TriMulArgs a) {
     for (int r = 0; r < 16; ++r) gate[nt][r] = sigmoidf_(gate[nt][r]);
   lds_barrier();
 
-  // 2. contraction result -> sX[j][c] (transposed), then center LayerNorm
+  // 2. center LayerNorm of the contraction result, without a transposed copy:
+  // the channel-major chunks go to LDS as they are (sT[c][j], 16-byte stores),
+  // and every lane gathers, for its own pixel, exactly the 64 channels that
+  // its eight MFMA B-fragments hold (channels 16 ks + 8 hh + e; the other half
+  // of the wave holds the other 64 of the same pixel).  Lanes of a half-wave
+  // read consecutive pixels of one channel row: conflict-free, where a
+  // transposing 2-byte scatter would put a whole wave on two banks.
+  bf16_t* sT = sX;
 #pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int c = it * 16 + crow;
-    const uint32_t w4[4] = {rt[it].x, rt[it].y, rt[it].z, rt[it].w};
+  for (int it = 0; it < 8; ++it) *reinterpret_cast<u32x4*>(sT + (it * 16 + crow) * LDX + pc * 8) = rt[it];
+  wr.store(sW, tid);
+  if (tid < C) {
+    sP[tid] = a.ln_c_w[tid];
+    sP[C + tid] = a.ln_c_b[tid];
+  }
+  lds_barrier();
+  {
+    const int j = lane & 31, hh = lane >> 5;
+    const int px = wave * 32 + j;
+    const int xaddr = half_swap_addr();
+    float v[8][8];
+    float s1 = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      bf16_t h = (bf16_t)((e & 1) ? (w4[e >> 1] >> 16) : (w4[e >> 1] & 0xffffu));
-      if (e >= nvalid) h = 0;
-      sX[(pc * 8 + e) * LDX + c] = h;
+    for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        v[ks][e] = bf2f(sT[(16 * ks + 8 * hh + e) * LDX + px]);
+        s1 += v[ks][e];
+      }
+    s1 += half_swap(xaddr, s1);
+    const float mean = s1 * (1.f / C);
+    float s2 = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { const float d = v[ks][e] - mean; s2 += d * d; }
+    s2 += half_swap(xaddr, s2);
+    const float rstd = rsqrtf(s2 * (1.f / C) + LN_EPS);
+    const bool ok = t.valid(px);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const f32x4 w0 = *reinterpret_cast<const f32x4*>(sP + 16 * ks + 8 * hh);
+      const f32x4 w1 = *reinterpret_cast<const f32x4*>(sP + 16 * ks + 8 * hh + 4);
+      const f32x4 b0 = *reinterpret_cast<const f32x4*>(sP + C + 16 * ks + 8 * hh);
+      const f32x4 b1 = *reinterpret_cast<const f32x4*>(sP + C + 16 * ks + 8 * hh + 4);
+      const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+      const float bb[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = ok ? (v[ks][e] - mean) * rstd * w[e] + bb[e] : 0.f;
+      xf[ks] = as_frag(pack8(o));
     }
   }
-  wr.store(sW, tid);
-  lds_barrier();
-  ln_inplace_tile(sX, a.ln_c_w, a.ln_c_b, tid);
-  lds_barrier();
-  load_x_frags(sX, wave, lane, xf);
   f32x16 acc[4];
   mfma_chunk<true, 4>(xf, sW, lane, acc);
 #pragma unroll
