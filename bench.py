@@ -111,6 +111,9 @@ def main():
     ap.add_argument("--n-token", type=int, default=768)
     ap.add_argument("--io", choices=["bf16", "f32"], default="bf16", help="dtype of the residual stream")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run a plain elementwise kernel that reads and writes 256 MiB, three times: the "
+                         "reference against which the FETCH_SIZE / WRITE_SIZE counters of a profiler run are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build keeps the whole pair tensor on ONE GPU (no sharding, no collectives); "
@@ -195,6 +198,14 @@ def main():
         "others": {k: {"launch_ms": round(v[0], 4), "tflops": round(v[1] / v[0] / 1e9, 2)}
                    for k, v in kernels.items() if k != dom},
     }
+
+    if args.calibrate:
+        cx = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device=dev)   # 256 MiB in, 256 MiB out
+        cy = torch.empty_like(cx)
+        for _ in range(3):
+            torch.add(cx, 1.0, out=cy)
+        torch.cuda.synchronize()
+        del cx, cy
 
     out = {
         "metric": "Pairformer ms/block at N=%d bf16" % n,

@@ -10,8 +10,11 @@
 // 256x256 block with a 64-deep k slab, each wave a 128x128 quadrant = 4x4 MFMA
 // tiles = 256 fp32 accumulators (the unified 512-entry register file of a lone
 // wave per SIMD), half a fragment read per MFMA and twice the FLOPs per byte
-// fetched from L2.  Slabs are double-buffered in LDS (144 KB), prefetched
-// through registers one slab ahead, one barrier per slab.
+// fetched from L2.  Slabs are double-buffered in LDS (144 KB) and prefetched
+// through two register sets (two slabs ahead of the MFMAs), one barrier per
+// slab; global loads, LDS fragment reads and LDS stores are interleaved with
+// the MFMA stream explicitly, because the lone wave of a SIMD has nobody to
+// cover for it while one of them blocks its instruction stream.
 //
 // The accumulators hold T^T tiles (B fragments as the MFMA's A operand), so a
 // lane owns one output row i and four consecutive columns j per register quad:

@@ -372,20 +372,27 @@ __global__ __launch_bounds__(256, 2) void transition_kernel(TransitionArgs a) {
 #pragma unroll 1
   for (int hs = 0; hs < n_slabs; ++hs) {
     if (hs + 1 < n_slabs) fetch(hs + 1);
-    // GEMM1, T form: acc[0..1] = a^T (64 hidden x 32 px), acc[2..3] = b^T
-    f32x16 acc[4];
-    mfma_chunk<true, 4>(xf, sW1, lane, acc);
-    // h^T = silu(a) * b; registers 8s..8s+7 of tile nt are, as they stand, the
-    // B fragment of k-step s of GEMM2 provided W2's k index is permuted alike:
-    // element e of lane-half hh is hidden unit 32*nt + 16*s + 8*(e >> 2) + 4*hh + (e & 3).
+    // GEMM1, T form, one 32-unit half of the slab at a time (32 live
+    // accumulators instead of 64): ab[0] = a^T (32 hidden x 32 px), ab[1] = b^T.
+    // h^T = silu(a) * b; registers 8s..8s+7 are, as they stand, the B fragment of
+    // k-step s of GEMM2 provided W2's k index is permuted alike: element e of
+    // lane-half hh is hidden unit 32*nt + 16*s + 8*(e >> 2) + 4*hh + (e & 3).
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
+      f32x16 ab[2];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) ab[0][r] = ab[1][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        ab[0] = mfma32(lds_frag(sW1, LDX, nt * 32, ks * 16, lane), xf[ks], ab[0]);
+        ab[1] = mfma32(lds_frag(sW1, LDX, 64 + nt * 32, ks * 16, lane), xf[ks], ab[1]);
+      }
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         float hv[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const float av = acc[nt][8 * s + e], bv = acc[nt + 2][8 * s + e];
+          const float av = ab[0][8 * s + e], bv = ab[1][8 * s + e];
           hv[e] = av * sigmoidf_(av) * bv;
         }
         const bf16x8 hf = as_frag(pack8(hv));
