@@ -32,6 +32,10 @@ if ROOT not in sys.path:
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel from rocprofv3 counters (FETCH_SIZE x 2.000 +
+# WRITE_SIZE x 1.000, scaled by a plain elementwise kernel of known size in the same run, see
+# --calibrate); measured offline, per N_token: profiles/pairformer_block_n768_bf16_hbm_traffic.txt
+MEASURED_TRAFFIC_BYTES = {("triattn_flash_kernel", 768): 786.6e6, ("contract_kernel", 768): 517.2e6}
 
 
 def flops_trimul(n):      # one direction
@@ -193,7 +197,8 @@ def main():
     achieved = dom_flops / dom_ms / 1e9
     roofline = {
         "kernel": dom, "bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
-        "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+        "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
+        "traffic": MEASURED_TRAFFIC_BYTES.get((dom.split(" ")[0], n)),
         "launch_ms": round(dom_ms, 4),
         "others": {k: {"launch_ms": round(v[0], 4), "tflops": round(v[1] / v[0] / 1e9, 2)}
                    for k, v in kernels.items() if k != dom},
