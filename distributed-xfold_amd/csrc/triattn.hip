@@ -184,25 +184,13 @@ constexpr int LDK = 56;      // sK row: 32 head-dim + 16 mask k-step + 8 pad (bf
 constexpr int LDV = KT + 4;  // sVt row: 136 B = 34 dwords, so 32 lanes' 8-byte reads hit 32 bank pairs
 constexpr int QW = 128;      // queries per workgroup
 constexpr uint32_t BF16_ONE = 0x3F80u, BF16_NEG_INF = 0xFF80u, BF16_NEG_1E9 = 0xCE6Eu;
-constexpr float LAZY_MAX = 6.f;  // a score may exceed its query's reference by this much (base-2 exponent)
 
 // One workgroup = (row b, head h, 128 queries); a wave owns 32 queries, lane
 // (j, hh) holds query j's scores for half of the keys of each 32-key tile.
 //
 // S^T = K Q^T runs on the matrix unit with three k-steps: the two halves of the
-// head dimension and an extension step whose K columns are
-//   [key mask value (0, -1e9 or -inf), 1.0, 1.0, 0 ...]   and whose Q entries are
-//   [1.0, -ref_hi(query), -ref_lo(query), 0 ...],
-// so the mask AND the softmax reference come out of the MFMA already applied.
-// Vector ALU and matrix unit together are busy all the time in this kernel
-// (head dim 32: one exp2 per 64 flops), so what counts is the number of vector
-// instructions per score.  m_ref = ref_hi + ref_lo (two bf16 terms, 17
-// significant bits) follows the query's running maximum but is only moved (and
-// o, l rescaled) when some score exceeds it by more than LAZY_MAX, which after
-// the first tile is rare: the common tile is exp2(S') -> bf16 with no
-// subtraction, no cross-lane maximum and no rescaling of O.  A tile that moves
-// a reference recomputes S without the reference term (adding then removing a
-// reference as far away as -1e9 would lose the score's low bits).  The pair bias is added on the matrix unit too,
+// head dimension and a mask step (K column 32 = 0, -1e9 or -inf per key, times a
+// Q entry of 1.0).  The pair bias is added on the matrix unit too,
 // S^T += I * bias^T; its B fragments are 16 contiguous bytes per lane and come
 // straight from global memory, where the bias is stored in fragment order: each
 // load instruction covers one contiguous 1 KB run (the bias is shared by every
@@ -214,7 +202,6 @@ template <bool HAS_BIAS>
 __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t sK[2][KT * LDK];
   __shared__ __attribute__((aligned(16))) bf16_t sVt[2][D * LDV];
-  __shared__ int sAnyKey;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hh = lane >> 5, j = lane & 31;
@@ -236,37 +223,14 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   const int64_t bh = (int64_t)b * H + h;
   const int ldn = (int)a.ldn;
 
-  // A row whose keys are ALL masked attends uniformly (every logit is absorbed
-  // by -1e9).  Once a reference of -1e9 sits in the extension step that
-  // absorption would depend on the order in which the matrix unit adds the
-  // products, so such a row drops q and the bias altogether: S is then the mask
-  // column alone and exactly uniform.
-  bool row_live = true;
-  if (a.mask) {
-    if (tid == 0) sAnyKey = 0;
-    __syncthreads();
-    bool any_on = false;
-    for (int k = tid; k < N; k += 256) any_on |= a.mask[(int64_t)b * N + k] != 0.f;
-    if (any_on) sAnyKey = 1;
-    __syncthreads();
-    row_live = sAnyKey != 0;
-  }
-  bf16x8 qf[2];
+  bf16x8 qf[3];
   {
     const bf16_t* qp = a.q + (bh * N + qi) * D + 8 * hh;
-    const u32x4 z = {0u, 0u, 0u, 0u};
-    qf[0] = as_frag(row_live ? *reinterpret_cast<const u32x4*>(qp) : z);
-    qf[1] = as_frag(row_live ? *reinterpret_cast<const u32x4*>(qp + 16) : z);
+    qf[0] = as_frag(*reinterpret_cast<const u32x4*>(qp));
+    qf[1] = as_frag(*reinterpret_cast<const u32x4*>(qp + 16));
+    u32x4 one = {hh == 0 ? BF16_ONE : 0u, 0u, 0u, 0u};
+    qf[2] = as_frag(one);
   }
-  // extension fragment of Q: [1.0, -ref_hi, -ref_lo] in the low half-wave, zeros in the high one
-  auto ext_frag = [&](float ref_hi, float ref_lo) {
-    u32x4 e = {0u, 0u, 0u, 0u};
-    if (hh == 0) {
-      e.x = BF16_ONE | ((uint32_t)f2bf(-ref_hi) << 16);
-      e.y = (uint32_t)f2bf(-ref_lo);
-    }
-    return as_frag(e);
-  };
   // Identity fragments: A-fragment of k-step `st`: lane (row i = j, half hh)
   // holds I[i][16 st + 8 hh + e], e = 0..7: a single 1.0 where 16 st + 8 hh + e == i.
   bf16x8 idf[2];
@@ -320,11 +284,6 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
     const char* p = bbase + (size_t)min(bias_next, bias_tiles - 1) * 4096u;
 #pragma unroll
     for (int i = 0; i < 4; ++i) dst[i] = *reinterpret_cast<const u32x4*>(p + (b_lane + 1024u * i));
-    if (!row_live) {  // workgroup-uniform
-      const u32x4 z = {0, 0, 0, 0};
-#pragma unroll
-      for (int i = 0; i < 4; ++i) dst[i] = z;
-    }
     ++bias_next;
   };
   auto sstore = [&](int buf) {
@@ -332,7 +291,7 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
     *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + k_c * 8]) = key_ok ? rk : z;
     if (k_c < 2) {
       const uint32_t rmask = !key_ok ? BF16_NEG_INF : (rm == 0.f ? BF16_NEG_1E9 : 0u);
-      u32x4 m = {k_c == 0 ? (rmask | (BF16_ONE << 16)) : 0u, k_c == 0 ? BF16_ONE : 0u, 0u, 0u};
+      u32x4 m = {k_c == 0 ? rmask : 0u, 0u, 0u, 0u};
       *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + 32 + k_c * 8]) = m;
     }
     // rows of sVt are 8-byte aligned only: two 8-byte stores
@@ -345,9 +304,7 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   f32x16 o;
 #pragma unroll
   for (int r = 0; r < 16; ++r) o[r] = 0.f;
-  float m_ref = -__builtin_huge_valf(), l_run = 0.f;
-  bf16x8 qext = ext_frag(0.f, 0.f);
-  bool first = true;
+  float m_run = -__builtin_huge_valf(), l_run = 0.f;
 
   const int nkt = (N + KT - 1) / KT;
   gload_kv(0);
@@ -364,52 +321,17 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
     // has every key at -inf (mask column) and contributes exactly zero.
     // s[u][4g + e] <-> key 32u + 8g + 4hh + e of this tile, query j.
     f32x16 s[2];
-    auto scores = [&](const bf16x8& ext) {
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < 2; ++u) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[u][r] = 0.f;
-        if (HAS_BIAS) {
-          s[u] = mfma32(idf[0], as_frag(rb[2 * u]), s[u]);
-          s[u] = mfma32(idf[1], as_frag(rb[2 * u + 1]), s[u]);
-        }
-        s[u] = mfma32(lds_frag(sK[buf], LDK, u * 32, 0, lane), qf[0], s[u]);
-        s[u] = mfma32(lds_frag(sK[buf], LDK, u * 32, 16, lane), qf[1], s[u]);
-        s[u] = mfma32(lds_frag(sK[buf], LDK, u * 32, 32, lane), ext, s[u]);
+      for (int r = 0; r < 16; ++r) s[u][r] = 0.f;
+      if (HAS_BIAS) {
+        s[u] = mfma32(idf[0], as_frag(rb[2 * u]), s[u]);
+        s[u] = mfma32(idf[1], as_frag(rb[2 * u + 1]), s[u]);
       }
-    };
-    auto lane_max = [&]() {
-      float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int g = (u == 0 ? 1 : 0); g < 4; ++g)
-          mx = fmaxf(mx, fmaxf(fmaxf(s[u][4 * g], s[u][4 * g + 1]), fmaxf(s[u][4 * g + 2], s[u][4 * g + 3])));
-      return mx;
-    };
-    scores(qext);
-    float alpha = 1.f;
-    if (first || __any(lane_max() > LAZY_MAX)) {
-      // move the references: scores without the reference term, ordinary online-softmax update
-      if (!first) scores(ext_frag(0.f, 0.f));
-      float mx = lane_max();
-      mx = fmaxf(mx, half_swap(xaddr, mx));
-      // the new reference is the running maximum to two bf16 terms, so that the
-      // largest probability of this tile is 1 up to 2^-17 and rounds to 1 exactly
-      const float m_new = fmaxf(m_ref, mx);
-      const float ref_hi = bf2f(f2bf(m_new));
-      const float ref_lo = bf2f(f2bf(m_new - ref_hi));
-      const float new_ref = ref_hi + ref_lo;
-      alpha = __builtin_amdgcn_exp2f(m_ref - new_ref);
-      m_ref = new_ref;
-      qext = ext_frag(ref_hi, ref_lo);
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[u][r] -= new_ref;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o[r] *= alpha;
-      first = false;
+      for (int ks = 0; ks < 3; ++ks)
+        s[u] = mfma32(lds_frag(sK[buf], LDK, u * 32, ks * 16, lane), qf[ks], s[u]);
     }
     // Global loads are issued here, behind the score MFMAs: the bias registers
     // are free again, and the K / V loads come first so that their consumer (the
@@ -417,6 +339,16 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
     // loads queued behind them (vector memory operations retire in order).
     gload_kv((kt + 1) * KT);
     gload_bias(rb);
+    float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int g = (u == 0 ? 1 : 0); g < 4; ++g)
+        mx = fmaxf(mx, fmaxf(fmaxf(s[u][4 * g], s[u][4 * g + 1]), fmaxf(s[u][4 * g + 2], s[u][4 * g + 3])));
+    mx = fmaxf(mx, half_swap(xaddr, mx));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    m_run = m_new;
     bf16x8 pf[2][2];
 #pragma unroll
     for (int u = 0; u < 2; ++u)
@@ -424,7 +356,7 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
       for (int half = 0; half < 2; ++half) {
         float pv8[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) pv8[e] = __builtin_amdgcn_exp2f(s[u][8 * half + e]);
+        for (int e = 0; e < 8; ++e) pv8[e] = __builtin_amdgcn_exp2f(s[u][8 * half + e] - m_new);
         pf[u][half] = as_frag(pack8(pv8));
       }
     // Row sums on the matrix unit: ones * P sums the bf16 probabilities of all
@@ -438,6 +370,10 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
 #pragma unroll
       for (int half = 0; half < 2; ++half) lsum = mfma32(onesf, pf[u][half], lsum);
     l_run = l_run * alpha + lsum[0];
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[r] *= alpha;
+    }
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
