@@ -23,8 +23,11 @@
 namespace {
 
 constexpr int KT = 64;        // keys per LDS tile
-constexpr int LDV = KT + 8;   // sVt row stride (bf16)
+constexpr int LDV = KT + 4;   // sVt row stride (bf16): 34 dwords, 32 rows' 8-byte reads hit 32 bank pairs
 constexpr float NEG_INF = -__builtin_huge_valf();
+constexpr float LOG2E = 1.4426950408889634f;
+// per-key code staged in LDS next to the K tile
+constexpr int KEY_MASKED = 1, KEY_PAD = 2, KEY_BEYOND = 4;
 
 template <int KSTEPS, int DVT, int NW>
 __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
@@ -33,6 +36,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
   constexpr int NT = NW * 64;
   __shared__ __attribute__((aligned(16))) bf16_t sK[2][KT * LDK];
   __shared__ __attribute__((aligned(16))) bf16_t sVt[2][DVT * 32 * LDV];
+  __shared__ __attribute__((aligned(16))) int sCode[2][KT];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hh = lane >> 5, j = lane & 31;
@@ -53,47 +57,69 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       const int c = 16 * ks + 8 * hh;
-      u32x4 v = {0, 0, 0, 0};
-      if (c < d) v = *reinterpret_cast<const u32x4*>(qp + c);
-      qf[ks] = as_frag(v);
+      const u32x4 z = {0, 0, 0, 0};
+      const u32x4 v = *reinterpret_cast<const u32x4*>(qp + (c < d ? c : 0));
+      qf[ks] = as_frag(c < d ? v : z);
     }
   }
+  const bf16x8 onesf = as_frag(u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
 
   const bf16_t* kg = a.k + (int64_t)b * a.k_sb + h * d;
   const bf16_t* vg = a.v + (int64_t)b * a.v_sb + h * d;
   const int dch = d / 8;  // 16-byte chunks per real key row
 
-  // tile loaders (global -> registers -> LDS), chunk id = key * (KD/8) + c
+  // Tile loaders (global -> registers -> LDS).  Every load is unconditional,
+  // from a clamped address, and nothing is decided from a loaded value before
+  // the LDS store one tile later: a load under a lane mask, or a value
+  // inspected right after its load, costs a full memory round trip per tile.
+  //   K: chunk id = key * (KD/8) + c, c fastest (one key row is contiguous)
+  //   V: chunk id = c * KT + key, key fastest, so that the transposing 2-byte
+  //      LDS stores of a wave walk along a V^T row instead of down a column
   constexpr int KCH = KT * (KD / 8);
   constexpr int NLD = (KCH + NT - 1) / NT;
   u32x4 rk[NLD], rv[NLD];
+  float rkm = 1.f, rkp = 1.f;  // key mask / key padding flag of key tid (threads 0..63)
+  const int bb = a.bias_mod > 0 ? b % a.bias_mod : b;  // batch index of bias / padding masks
+  const float* kmask = a.key_mask ? a.key_mask + (int64_t)b * a.km_sb : nullptr;
+  const float* kpad = a.kpad ? a.kpad + (int64_t)bb * a.kp_sb : nullptr;
+  int k0_loaded = 0;
   auto gload = [&](int k0) {
+    k0_loaded = k0;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-      const int idx = tid + i * NT;
-      const int key = idx / (KD / 8), c = idx % (KD / 8);
-      const u32x4 z = {0, 0, 0, 0};
-      rk[i] = z; rv[i] = z;
-      if (idx < KCH && k0 + key < a.Sk && c < dch) {
-        rk[i] = *reinterpret_cast<const u32x4*>(kg + (int64_t)(k0 + key) * a.k_ss + c * 8);
-        rv[i] = *reinterpret_cast<const u32x4*>(vg + (int64_t)(k0 + key) * a.v_ss + c * 8);
-      }
+      const int idx = min(tid + i * NT, KCH - 1);
+      const int key = min(k0 + idx / (KD / 8), a.Sk - 1), c = idx % (KD / 8);
+      rk[i] = *reinterpret_cast<const u32x4*>(kg + (int64_t)key * a.k_ss + (c < dch ? c : 0) * 8);
+      const int vkey = min(k0 + idx % KT, a.Sk - 1), vc = idx / KT;
+      rv[i] = *reinterpret_cast<const u32x4*>(vg + (int64_t)vkey * a.v_ss + (vc < dch ? vc : 0) * 8);
+    }
+    if (tid < KT) {
+      const int key = min(k0 + tid, a.Sk - 1);
+      if (kmask) rkm = kmask[key];
+      if (kpad) rkp = kpad[key];
     }
   };
   auto sstore = [&](int buf) {
+    const u32x4 z = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int idx = tid + i * NT;
       if (idx >= KCH) continue;
       const int key = idx / (KD / 8), c = idx % (KD / 8);
-      *reinterpret_cast<u32x4*>(&sK[buf][key * LDK + c * 8]) = rk[i];
-      if (c * 8 < DVT * 32) {
+      *reinterpret_cast<u32x4*>(&sK[buf][key * LDK + c * 8]) = (k0_loaded + key < a.Sk && c < dch) ? rk[i] : z;
+      const int vkey = idx % KT, vc = idx / KT;
+      if (vc * 8 < DVT * 32) {
+        const bool ok = k0_loaded + vkey < a.Sk && vc < dch;
         const uint32_t w4[4] = {rv[i].x, rv[i].y, rv[i].z, rv[i].w};
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          sVt[buf][(c * 8 + e) * LDV + key] = (bf16_t)((e & 1) ? (w4[e >> 1] >> 16) : (w4[e >> 1] & 0xffffu));
+        for (int e = 0; e < 8; ++e) {
+          const bf16_t x = (bf16_t)((e & 1) ? (w4[e >> 1] >> 16) : (w4[e >> 1] & 0xffffu));
+          sVt[buf][(vc * 8 + e) * LDV + vkey] = ok ? x : (bf16_t)0;
+        }
       }
     }
+    if (tid < KT)
+      sCode[buf][tid] = (k0_loaded + tid >= a.Sk ? KEY_BEYOND : 0) | (rkm == 0.f ? KEY_MASKED : 0) | (rkp == 0.f ? KEY_PAD : 0);
   };
   // V^T rows that no chunk covers (head dim padding) must read as zero
   for (int idx = tid; idx < 2 * DVT * 32 * LDV; idx += NT) (&sVt[0][0])[idx] = 0;
@@ -104,112 +130,141 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
   for (int t = 0; t < DVT; ++t)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
-  float m_run = NEG_INF, l_run = 0.f;
+  float m_run = NEG_INF, l_run = 0.f;  // running maximum in base-2 units
 
-  const int bb = a.bias_mod > 0 ? b % a.bias_mod : b;  // batch index of bias / padding masks
+  // Pair bias (fp32, one row per query): the 8 quads of a 64-key tile are
+  // fetched one tile ahead, unconditionally, from addresses clamped into the
+  // row (a clamped quad belongs to keys >= Sk, which are masked anyway).
   const float* bias_row = a.bias ? a.bias + (int64_t)bb * a.bias_sb + (int64_t)h * a.bias_sh + (int64_t)qi * a.bias_sq : nullptr;
-  const float* kmask = a.key_mask ? a.key_mask + (int64_t)b * a.km_sb : nullptr;
-  const float* kpad = a.kpad ? a.kpad + (int64_t)bb * a.kp_sb : nullptr;
   const bool q_is_pad = a.qpad ? (a.qpad[(int64_t)bb * a.qp_sb + qi] == 0.f) : false;
-  const bool bias_vec = a.bias && ((a.bias_sq & 3) == 0) && ((a.bias_sb & 3) == 0) && ((a.bias_sh & 3) == 0) &&
-                        (((uintptr_t)a.bias & 15) == 0);
+  const bool bias_vec = a.bias && a.Sk >= 4 && ((a.bias_sq & 3) == 0) && ((a.bias_sb & 3) == 0) &&
+                        ((a.bias_sh & 3) == 0) && (((uintptr_t)a.bias & 15) == 0);
+  const int last_quad = (a.Sk - 1) & ~3;
+  f32x4 rbias[2][4];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) rbias[u][g] = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto gload_bias = [&](int k0) {
+    if (!bias_vec) return;  // workgroup-uniform
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        rbias[u][g] = *reinterpret_cast<const f32x4*>(bias_row + min(k0 + u * 32 + 8 * g + 4 * hh, last_quad));
+  };
 
   const int nkt = (a.Sk + KT - 1) / KT;
   gload(0);
+  gload_bias(0);
   sstore(0);
   lds_barrier();
 
   for (int kt = 0; kt < nkt; ++kt) {
     const int buf = kt & 1;
-    if (kt + 1 < nkt) gload((kt + 1) * KT);
+    const int k0 = kt * KT;
+    // both 32-key halves through the matrix unit first (two independent chains);
+    // s[u][4g + e] = logit(query j, key k0 + 32u + 8g + 4hh + e)
+    f32x16 s[2];
 #pragma unroll
-    for (int sub = 0; sub < 2; ++sub) {
-      const int kbase = kt * KT + sub * 32;
-      if (kbase >= a.Sk) break;  // uniform across the workgroup
-      f32x16 s;
+    for (int u = 0; u < 2; ++u) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[r] = 0.f;
+      for (int r = 0; r < 16; ++r) s[u][r] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks)
-        s = mfma32(lds_frag(sK[buf], LDK, sub * 32, ks * 16, lane), qf[ks], s);
-      // s[4g + e] = logit(query j, key kbase + 8g + 4hh + e)
+        s[u] = mfma32(lds_frag(sK[buf], LDK, u * 32, ks * 16, lane), qf[ks], s[u]);
+    }
+    // bias, then the next tile's loads into the registers just freed
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const int key0 = kbase + 8 * g + 4 * hh;
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (bias_row) {
-          if (bias_vec && key0 + 3 < a.Sk) {
-            const f32x4 t4 = *reinterpret_cast<const f32x4*>(bias_row + key0);
-            bv[0] = t4.x; bv[1] = t4.y; bv[2] = t4.z; bv[3] = t4.w;
-          } else {
+        if (bias_vec) {
+          s[u][4 * g] += rbias[u][g].x; s[u][4 * g + 1] += rbias[u][g].y;
+          s[u][4 * g + 2] += rbias[u][g].z; s[u][4 * g + 3] += rbias[u][g].w;
+        } else if (bias_row) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (key0 + e < a.Sk) bv[e] = bias_row[key0 + e];
+          for (int e = 0; e < 4; ++e) {
+            const int key = k0 + u * 32 + 8 * g + 4 * hh + e;
+            s[u][4 * g + e] += bias_row[min(key, a.Sk - 1)];
           }
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int key = key0 + e;
-          float v = s[4 * g + e] + bv[e];
-          if (key >= a.Sk) {
-            v = NEG_INF;
-          } else {
-            if (kmask && kmask[key] == 0.f) v = -1e9f;
-            if (q_is_pad && kpad[key] == 0.f) v += 1e9f;
-          }
-          s[4 * g + e] = v;
         }
       }
-      float mx = s[0];
+    gload((kt + 1) * KT);
+    gload_bias((kt + 1) * KT);
+    // masks from the per-key codes, logits to base 2
 #pragma unroll
-      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[r]);
-      mx = fmaxf(mx, half_swap(xaddr, mx));
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = __expf(m_run - m_new);  // 0 on the first tile (m_run = -inf, m_new finite)
-      m_run = m_new;
-      float psum = 0.f;
-      bf16x8 pf[2];
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int* cp = &sCode[buf][u * 32 + 8 * g + 4 * hh];
+        const int code[4] = {cp[0], cp[1], cp[2], cp[3]};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float v = s[u][4 * g + e];
+          if (code[e] & KEY_MASKED) v = -1e9f;
+          if (q_is_pad && (code[e] & KEY_PAD)) v += 1e9f;
+          v *= LOG2E;
+          if (code[e] & KEY_BEYOND) v = NEG_INF;
+          s[u][4 * g + e] = v;
+        }
+      }
+    float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int g = (u == 0 ? 1 : 0); g < 4; ++g)
+        mx = fmaxf(mx, fmaxf(fmaxf(s[u][4 * g], s[u][4 * g + 1]), fmaxf(s[u][4 * g + 2], s[u][4 * g + 3])));
+    mx = fmaxf(mx, half_swap(xaddr, mx));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first tile (m_run = -inf, m_new finite)
+    m_run = m_new;
+    bf16x8 pf[2][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         float pv[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) pv[e] = __expf(s[8 * half + e] - m_new);
-        const u32x4 pk = pack8(pv);
-        // the row sum uses the rounded probabilities so that the weights that
-        // multiply V sum to exactly one after normalisation
-        float back[8];
-        unpack8(pk, back);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) psum += back[e];
-        pf[half] = as_frag(pk);
+        for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(s[u][8 * half + e] - m_new);
+        pf[u][half] = as_frag(pack8(pv));
       }
-      l_run = l_run * alpha + psum;
-      if (__any(alpha != 1.f)) {
+    // row sums of the ROUNDED probabilities on the matrix unit (ones * P), so
+    // that the weights that multiply V sum to exactly one after normalisation
+    f32x16 lsum;
 #pragma unroll
-        for (int t = 0; t < DVT; ++t)
+    for (int r = 0; r < 16; ++r) lsum[r] = 0.f;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
-      }
-      // O^T[dd][query] += sum_key V^T[dd][key] P^T[key][query]; fragment element e
-      // of lane-half hh in k-step `half` is key kbase + 16*half + 8*(e>>2) + 4*hh + (e&3)
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int half = 0; half < 2; ++half) lsum = mfma32(onesf, pf[u][half], lsum);
+    l_run = l_run * alpha + lsum[0];
+    if (__any(alpha != 1.f)) {
 #pragma unroll
       for (int t = 0; t < DVT; ++t)
 #pragma unroll
+        for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
+    }
+    // O^T[dd][query] += sum_key V^T[dd][key] P^T[key][query]; fragment element e
+    // of lane-half hh in k-step `half` is key 32u + 16*half + 8*(e>>2) + 4*hh + (e&3)
+#pragma unroll
+    for (int t = 0; t < DVT; ++t)
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
         for (int half = 0; half < 2; ++half) {
-          const bf16_t* vp = &sVt[buf][(t * 32 + j) * LDV + sub * 32 + 16 * half + 4 * hh];
+          const bf16_t* vp = &sVt[buf][(t * 32 + j) * LDV + u * 32 + 16 * half + 4 * hh];
           const u32x2 lo = *reinterpret_cast<const u32x2*>(vp);
           const u32x2 hi = *reinterpret_cast<const u32x2*>(vp + 8);
           u32x4 vv;
           vv.x = lo.x; vv.y = lo.y; vv.z = hi.x; vv.w = hi.y;
-          o[t] = mfma32(as_frag(vv), pf[half], o[t]);
+          o[t] = mfma32(as_frag(vv), pf[u][half], o[t]);
         }
-    }
     if (kt + 1 < nkt) sstore(buf ^ 1);
     lds_barrier();
   }
 
-  const float l_tot = l_run + half_swap(xaddr, l_run);
-  const float inv = 1.f / l_tot;
+  const float inv = 1.f / l_run;  // the ones * P sums cover both half-waves' keys
   if (!q_ok) return;
   // o[t][4g + e] = out(query j, head-dim 32t + 8g + 4hh + e)
 #pragma unroll
@@ -238,13 +293,17 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
     }
 }
 
+// Queries per workgroup: 128 (four waves share the K / V tiles), or 64 when
+// that would leave the 256 CUs with too few workgroups, or 32 for the short
+// query windows of the atom cross-attention.
 template <int KSTEPS, int DVT>
 int launch_nw(const FlashArgs& a, hipStream_t stream) {
-  const bool small = a.Sq <= 32;
-  const int qper = small ? 32 : 128;
-  const int64_t blocks = (int64_t)((a.Sq + qper - 1) / qper) * a.H * a.B;
+  const int64_t heads = (int64_t)a.H * a.B;
+  const int nw = a.Sq <= 32 ? 1 : (((a.Sq + 127) / 128) * heads < 1024 ? 2 : 4);
+  const int64_t blocks = (int64_t)((a.Sq + nw * 32 - 1) / (nw * 32)) * heads;
   if (blocks <= 0 || blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
-  if (small) hipLaunchKernelGGL((flash_kernel<KSTEPS, DVT, 1>), dim3((unsigned)blocks), dim3(64), 0, stream, a);
+  if (nw == 1) hipLaunchKernelGGL((flash_kernel<KSTEPS, DVT, 1>), dim3((unsigned)blocks), dim3(64), 0, stream, a);
+  else if (nw == 2) hipLaunchKernelGGL((flash_kernel<KSTEPS, DVT, 2>), dim3((unsigned)blocks), dim3(128), 0, stream, a);
   else hipLaunchKernelGGL((flash_kernel<KSTEPS, DVT, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
   return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }
