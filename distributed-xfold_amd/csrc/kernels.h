@@ -46,6 +46,7 @@ struct RowNormArgs {
   const float* scale = nullptr;   // [cond_rows][ld_cond] pre-sigmoid, or null
   const float* shift = nullptr;
   int64_t cond_rows = 0, ld_cond = 0;
+  int param_vec = 0, cond_vec = 0;  // set by launch_row_norm: arrays aligned for 16-byte loads
 };
 int launch_row_norm(const RowNormArgs& a, hipStream_t stream);
 

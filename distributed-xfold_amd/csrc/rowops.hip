@@ -1,13 +1,48 @@
 // Row-wise LayerNorm / adaptive LayerNorm for the single, diffusion and atom
 // activations (any channel count that is a multiple of 8).  One wave owns one
-// row: 16-byte loads, two-pass statistics in registers, a 64-lane reduction,
-// bf16 output ready to be an MFMA operand.  HBM-bound.
+// row (or, for narrow rows, a group of 1..16 lanes does): 16-byte loads,
+// two-pass statistics in registers, a shuffle reduction, bf16 output ready to
+// be an MFMA operand.  HBM-bound.
 #include "common.h"
 #include "kernels.h"
 
 namespace {
 
 constexpr int MAX_CHUNKS = 4;  // 64 lanes * 8 channels * 4 = 2048 channels at most
+
+// Eight consecutive fp32 parameters (the channel offset is a multiple of 8):
+// two 16-byte loads when the launcher found the array aligned for them.
+__device__ __forceinline__ void load8f(const float* p, bool vec, float* out) {
+  if (vec) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p);
+    const f32x4 b = *reinterpret_cast<const f32x4*>(p + 4);
+    out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+    out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = p[e];
+  }
+}
+
+// y = LN(x) [* weight] [+ bias], then [sigmoid(scale) * y + shift], 8 channels
+__device__ __forceinline__ void finish8(const RowNormArgs& a, const float* v, float mean, float rstd, int c,
+                                        int64_t crow, float* o) {
+  float w[8], b[8], sc[8], sh[8];
+  if (a.weight) load8f(a.weight + c, a.param_vec, w);
+  if (a.bias) load8f(a.bias + c, a.param_vec, b);
+  if (a.scale) {
+    load8f(a.scale + crow * a.ld_cond + c, a.cond_vec, sc);
+    load8f(a.shift + crow * a.ld_cond + c, a.cond_vec, sh);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float t = (v[e] - mean) * rstd;
+    if (a.weight) t *= w[e];
+    if (a.bias) t += b[e];
+    if (a.scale) t = sigmoidf_(sc[e]) * t + sh[e];
+    o[e] = t;
+  }
+}
 
 template <typename TIn>
 __global__ __launch_bounds__(256) void ln_rows_kernel(RowNormArgs a) {
@@ -44,26 +79,74 @@ __global__ __launch_bounds__(256) void ln_rows_kernel(RowNormArgs a) {
     const int c = (i * 64 + lane) * 8;
     if (c < a.C) {
       float o[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float t = (v[i][e] - mean) * rstd;
-        if (a.weight) t *= a.weight[c + e];
-        if (a.bias) t += a.bias[c + e];
-        if (a.scale) t = sigmoidf_(a.scale[crow * a.ld_cond + c + e]) * t + a.shift[crow * a.ld_cond + c + e];
-        o[e] = t;
-      }
+      finish8(a, v[i], mean, rstd, c, crow, o);
       *reinterpret_cast<u32x4*>(y + c) = pack8(o);
     }
   }
 }
 
+// Narrow rows (C <= 128, e.g. the 16-channel atom pair conditioning with its
+// millions of rows): G lanes per row, 64 / G rows per wave, so a wave still
+// moves a full kilobyte per instruction instead of one lane group's worth.
+template <typename TIn, int G>
+__global__ __launch_bounds__(256) void ln_rows_small_kernel(RowNormArgs a) {
+  constexpr int RPW = 64 / G;
+  const int lane = threadIdx.x & 63, sub = lane % G;
+  const int64_t row = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW + lane / G;
+  const bool ok = row < a.rows && sub * 8 < a.C;
+  const int64_t rr = row < a.rows ? row : a.rows - 1;
+  const int c = sub * 8 < a.C ? sub * 8 : 0;
+  float v[8];
+  Elem<TIn>::load8(reinterpret_cast<const TIn*>(a.x) + rr * a.ldx + c, v);
+  float s = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) { v[e] = ok ? v[e] : 0.f; s += v[e]; }
+#pragma unroll
+  for (int m = 1; m < G; m <<= 1) s += __shfl_xor(s, m);
+  const float mean = s / (float)a.C;
+  float q = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) { const float d = ok ? v[e] - mean : 0.f; q += d * d; }
+#pragma unroll
+  for (int m = 1; m < G; m <<= 1) q += __shfl_xor(q, m);
+  const float rstd = rsqrtf(q / (float)a.C + LN_EPS);
+  if (!ok) return;
+  const int64_t crow = a.cond_rows > 0 ? row % a.cond_rows : 0;
+  float o[8];
+  finish8(a, v, mean, rstd, c, crow, o);
+  *reinterpret_cast<u32x4*>(a.y + row * a.ldy + c) = pack8(o);
+}
+
+template <typename TIn>
+int launch_small(const RowNormArgs& a, hipStream_t stream) {
+  const int chunks = a.C / 8;
+  const int g = chunks <= 1 ? 1 : chunks <= 2 ? 2 : chunks <= 4 ? 4 : chunks <= 8 ? 8 : 16;
+  const int64_t rows_per_block = 4 * (64 / g);
+  const int64_t blocks = (a.rows + rows_per_block - 1) / rows_per_block;
+  if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  const dim3 grid((unsigned)blocks), block(256);
+  switch (g) {
+    case 1: hipLaunchKernelGGL((ln_rows_small_kernel<TIn, 1>), grid, block, 0, stream, a); break;
+    case 2: hipLaunchKernelGGL((ln_rows_small_kernel<TIn, 2>), grid, block, 0, stream, a); break;
+    case 4: hipLaunchKernelGGL((ln_rows_small_kernel<TIn, 4>), grid, block, 0, stream, a); break;
+    case 8: hipLaunchKernelGGL((ln_rows_small_kernel<TIn, 8>), grid, block, 0, stream, a); break;
+    default: hipLaunchKernelGGL((ln_rows_small_kernel<TIn, 16>), grid, block, 0, stream, a); break;
+  }
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
 }  // namespace
 
-int launch_row_norm(const RowNormArgs& a, hipStream_t stream) {
+int launch_row_norm(const RowNormArgs& a_in, hipStream_t stream) {
+  RowNormArgs a = a_in;
+  auto al16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+  a.param_vec = al16(a.weight) && al16(a.bias);
+  a.cond_vec = al16(a.scale) && al16(a.shift) && (a.ld_cond & 3) == 0;
   if (a.rows <= 0 || a.C <= 0 || (a.C & 7) || a.C > 64 * 8 * MAX_CHUNKS) return AF3_ERR_BAD_ARG;
   if ((a.ldx & 7) || (a.ldy & 7) || ((uintptr_t)a.x & 15) || ((uintptr_t)a.y & 15)) return AF3_ERR_BAD_ARG;
   if ((a.scale == nullptr) != (a.shift == nullptr)) return AF3_ERR_BAD_ARG;
   if (a.scale && a.cond_rows <= 0) return AF3_ERR_BAD_ARG;
+  if (a.C <= 128) return a.x_f32 ? launch_small<float>(a, stream) : launch_small<bf16_t>(a, stream);
   const unsigned blocks = (unsigned)((a.rows + 3) / 4);
   if (a.x_f32) hipLaunchKernelGGL(ln_rows_kernel<float>, dim3(blocks), dim3(256), 0, stream, a);
   else hipLaunchKernelGGL(ln_rows_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, a);

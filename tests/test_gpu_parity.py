@@ -152,7 +152,7 @@ def test_linear_swiglu_and_gate_res(gpu_pkg):
     assert e < 1e-5
 
 
-@pytest.mark.parametrize("c", [16, 128, 384, 768])
+@pytest.mark.parametrize("c", [8, 16, 40, 128, 384, 768])
 def test_layer_norm_and_adaln(gpu_pkg, c):
     note(f"test_layer_norm_and_adaln c={c}")
     g = gen(c)
