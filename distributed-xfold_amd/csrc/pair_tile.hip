@@ -29,9 +29,11 @@ namespace {
 // triangle multiplication, prologue
 // ============================================================================
 template <typename TIO>
-__global__ __launch_bounds__(256, 2) void trimul_prologue_kernel(TriMulArgs a) {
-  __shared__ __attribute__((aligned(16))) bf16_t sX[TM * LDX];  // LN tile, then the [64 ch][px] staging tile
-  __shared__ __attribute__((aligned(16))) bf16_t sW[TM * LDX];
+__global__ __launch_bounds__(256, 3) void trimul_prologue_kernel(TriMulArgs a) {
+  // 34.8 KB + 17.4 KB + 0.5 KB of LDS and at most 168 registers: three workgroups per CU.  The kernel is
+  // a chain of short dependent phases (load, LayerNorm, MFMA, stage, store), so what it needs is company.
+  __shared__ __attribute__((aligned(16))) bf16_t sX[TM * LDX];  // LN tile, then the [32 ch][px] staging tile
+  __shared__ __attribute__((aligned(16))) bf16_t sW[64 * LDX];  // 32 projection rows | the 32 matching gate rows
   __shared__ float sMask[TM];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // outgoing: tiles run along k for fixed i (a[c][i][k]); incoming: along k for
@@ -39,35 +41,50 @@ __global__ __launch_bounds__(256, 2) void trimul_prologue_kernel(TriMulArgs a) {
   const Tile t = make_tile(a.N, !a.outgoing);
   const TIO* x = reinterpret_cast<const TIO*>(a.pair);
 
-  WChunkRegs wr;
-  wr.load(a.w_pg, tid);
+  // Weight chunks in memory: [P(64 ch) | G(64 ch)] for a ch 0-63, a ch 64-127, b ch 0-63, b ch 64-127.
+  // Step s = 2 * chunk + half takes projection rows 32 half .. +31 and gate rows 64 + 32 half .. +31 of
+  // its chunk: 64 rows x 128, four 16-byte pieces per thread.
+  u32x4 wr[4];
+  auto wload = [&](int s) {
+    const bf16_t* base = a.w_pg + ((int64_t)(s >> 1) * TM + (s & 1) * 32) * C;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + 256 * i, row = idx >> 4;  // 0..63
+      wr[i] = *reinterpret_cast<const u32x4*>(base + ((row & 31) + (row >> 5) * 64) * C + (idx & 15) * 8);
+    }
+  };
+  auto wstore = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + 256 * i;
+      *reinterpret_cast<u32x4*>(sW + (idx >> 4) * LDX + (idx & 15) * 8) = wr[i];
+    }
+  };
+  wload(0);
   if (tid < TM) sMask[tid] = (t.valid(tid) ? (a.mask ? a.mask[t.pix(tid)] : 1.f) : 0.f);
   load_ln_tile<TIO>(x, t, a.ln_in_w, a.ln_in_b, sX, tid);
-  wr.store(sW, tid);
+  wstore();
   lds_barrier();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
   lds_barrier();  // sX is free from here on
 
-  // weight chunks: [P(64 ch) | G(64 ch)] for a ch 0-63, a ch 64-127, b ch 0-63, b ch 64-127
 #pragma unroll 1
-  for (int chunk = 0; chunk < 4; ++chunk) {
-    // request the next weights before this chunk's stores go out (vector
+  for (int s = 0; s < 8; ++s) {
+    // request the next weights before this step's stores go out (vector
     // memory operations retire in order)
-    if (chunk < 3) wr.load(a.w_pg + (int64_t)(chunk + 1) * TM * C, tid);
-    f32x16 acc[4];
-    mfma_chunk<false, 4>(xf, sW, lane, acc);
-    // D form: lane owns channel (lane & 31) of tiles 0/1 (P) and 2/3 (G)
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-      const int ch = nt * 32 + (lane & 31);
+    if (s < 7) wload(s + 1);
+    f32x16 acc[2];
+    mfma_chunk<false, 2>(xf, sW, lane, acc);
+    // D form: lane owns channel (lane & 31) of tile 0 (P) and tile 1 (G)
+    {
+      const int ch = lane & 31;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int p0 = wave * 32 + 8 * g + 4 * (lane >> 5);
         float v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          v[e] = acc[nt][4 * g + e] * sMask[p0 + e] * sigmoidf_(acc[nt + 2][4 * g + e]);
+        for (int e = 0; e < 4; ++e) v[e] = acc[0][4 * g + e] * sMask[p0 + e] * sigmoidf_(acc[1][4 * g + e]);
         u32x2 pk;
         pk.x = pack2bf(v[0], v[1]);
         pk.y = pack2bf(v[2], v[3]);
@@ -75,10 +92,11 @@ __global__ __launch_bounds__(256, 2) void trimul_prologue_kernel(TriMulArgs a) {
       }
     }
     lds_barrier();  // staging visible; every wave is done with sW
-    if (chunk < 3) wr.store(sW, tid);
-    bf16_t* dst = (chunk < 2 ? a.a_buf : a.b_buf) + ((int64_t)(chunk & 1) * 64 * a.N + t.o) * a.Np;
+    if (s < 7) wstore();
+    // 32 channels x 128 positions: two 16-byte pieces per thread
+    bf16_t* dst = (s < 4 ? a.a_buf : a.b_buf) + ((int64_t)(((s >> 1) & 1) * 64 + (s & 1) * 32) * a.N + t.o) * a.Np;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 2; ++i) {
       const int idx = tid + 256 * i, ch = idx >> 4, pc = idx & 15;
       const int r = t.r0 + pc * 8;
       if (r < a.Np)
