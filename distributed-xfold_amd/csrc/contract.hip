@@ -2,19 +2,34 @@
 // for a batch of channels c, bf16 in and out, fp32 accumulation.
 //
 // Both operands are k-contiguous (the natural fragment order of
-// v_mfma_f32_32x32x16_bf16).  What bounds this product on a CU is not the matrix
-// unit but the operand traffic per MFMA, out of LDS and out of L2: a wave that
-// owns a 64x64 corner reads one 16-byte fragment per MFMA and with eight such
-// waves on a CU the LDS pipe is as busy as the matrix unit.  So the tile is as
-// large as the register file allows: one workgroup of four waves per CU, a
-// 256x256 block with a 64-deep k slab, each wave a 128x128 quadrant = 4x4 MFMA
-// tiles = 256 fp32 accumulators (the unified 512-entry register file of a lone
-// wave per SIMD), half a fragment read per MFMA and twice the FLOPs per byte
-// fetched from L2.  Slabs are double-buffered in LDS (144 KB) and prefetched
-// through two register sets (two slabs ahead of the MFMAs), one barrier per
-// slab; global loads, LDS fragment reads and LDS stores are interleaved with
-// the MFMA stream explicitly, because the lone wave of a SIMD has nobody to
-// cover for it while one of them blocks its instruction stream.
+// v_mfma_f32_32x32x16_bf16).  The tile is as large as the register file
+// allows: one workgroup of four waves per CU, a 256x256 block, each wave a
+// 128x128 quadrant = 4x4 MFMA tiles = 256 fp32 accumulators (the unified
+// 512-entry register file of a lone wave per SIMD), half a 16-byte fragment
+// read per MFMA and 128 FLOPs per byte fetched from L2.
+//
+// What paces the kernel is the CU's vector memory path: it accepts 64 bytes
+// per cycle, so the 32 KB of operands that go with 32 MFMAs per wave (1024
+// cycles of the matrix unit) occupy it for 512 cycles, and a wave that issues
+// a load into a full queue stalls with its MFMAs behind it.  A lone wave per
+// SIMD has nobody to cover for it.  So:
+//   * slabs (32 k deep) go from global memory straight into LDS
+//     (global_load_lds_dwordx4: no staging registers, no LDS stores in the
+//     instruction stream);
+//   * the loads are spread evenly, one per four MFMAs per wave, which keeps the
+//     memory path half busy all the time instead of saturated in bursts;
+//   * four LDS buffers: a load is issued two to three slabs (2000-3000 cycles)
+//     before anybody waits for it, about the latency of a miss that goes to HBM;
+//   * the one barrier per slab sits between its two k-steps, after the wave has
+//     read all its fragments of the slab: the MFMAs of the second k-step cover
+//     the barrier and the first fragment reads of the next slab, and the
+//     buffer is free for refill the moment the barrier is passed.
+// A load puts lane l's 16 bytes at LDS base + 16 l, so rows cannot be padded;
+// instead the four 16-byte chunks of a 64-byte row are permuted, chunk c of row
+// r living at position c ^ ((r >> 2) & 3), which makes the fragment reads (32
+// rows x one chunk per half-wave) conflict-free over the 64 banks.  The
+// permutation is applied on the global side, where a lane is free to fetch
+// any chunk.
 //
 // The accumulators hold T^T tiles (B fragments as the MFMA's A operand), so a
 // lane owns one output row i and four consecutive columns j per register quad:
@@ -27,16 +42,43 @@
 
 namespace {
 
-constexpr int CM = 256, CN = 256, CK = 64;
-constexpr int LDT = CK + 8;      // LDS row stride of a slab (bf16): 144 B keeps the 16-byte reads conflict-free
-constexpr int LDE = 128 + 8;     // LDS row stride of a wave's staged output quadrant (bf16)
-constexpr int STAGE = (CM + CN) * LDT;
+constexpr int CM = 256, CN = 256, CK = 32;
+constexpr int ROWB = CK * 2;            // bytes of a slab row in LDS (unpadded)
+constexpr int SLAB_A = CM * ROWB;       // A rows first, then B rows
+constexpr int SLAB = (CM + CN) * ROWB;  // 32 KB
+constexpr int LDE = 128 + 8;            // LDS row stride of a wave's staged output quadrant (bf16)
+constexpr int EPI_BYTES = 128 * LDE * 2;  // one wave's output quadrant
+constexpr int BUF_BYTES = SLAB > EPI_BYTES ? SLAB : EPI_BYTES;
+constexpr int NBUF = 4;
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+// 64 lanes x 16 bytes from global (uniform base + per-lane byte offset) to
+// 1 KB of LDS starting at the wave-uniform address dst
+__device__ __forceinline__ void load_to_lds(const char* base, uint32_t off, char* dst) {
+  __builtin_amdgcn_global_load_lds((gptr_t)(base + off), (lptr_t)dst, 16, 0, 0);
+}
+
+// s_waitcnt with vmcnt = n, lgkmcnt = 0 (expcnt left alone)
+template <int N>
+__device__ __forceinline__ void wait_loads_but() {
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x70);
+}
 
 __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
-  __shared__ __attribute__((aligned(16))) bf16_t smem[2 * STAGE];
-  static_assert(4 * 128 * LDE <= 2 * STAGE, "output staging must fit");
+  // Four arrays, not one: the compiler then knows that a load in flight to one
+  // buffer cannot alias a fragment read from another and does not make the
+  // read wait for it.
+  __shared__ __attribute__((aligned(1024))) char sb0[BUF_BYTES];
+  __shared__ __attribute__((aligned(1024))) char sb1[BUF_BYTES];
+  __shared__ __attribute__((aligned(1024))) char sb2[BUF_BYTES];
+  __shared__ __attribute__((aligned(1024))) char sb3[BUF_BYTES];
+  auto buf = [&](int i) -> char* { return (i & 3) == 0 ? sb0 : (i & 3) == 1 ? sb1 : (i & 3) == 2 ? sb2 : sb3; };
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hh = lane >> 5, l31 = lane & 31;
   const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
 
@@ -56,53 +98,54 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   const char* A = reinterpret_cast<const char*>(g.A + (int64_t)bz * g.sA);
   const char* B = reinterpret_cast<const char*>(g.B + (int64_t)bz * g.sB);
 
-  // Per slab each thread moves eight 16-byte chunks of A and eight of B:
-  // rows ld_row + 32 i, chunk ld_c.  Loads are unconditional from clamped rows:
-  // a row past the end repeats the last one, and what it produces lands in
-  // output rows that are never stored or in columns N..ldc-1 of T, which no
-  // consumer reads.  Only a k chunk past K must contribute nothing; it is
-  // zeroed on its way to LDS, in the one slab that can contain it.
-  const int ld_row = tid >> 3, ld_c = tid & 7;
-  uint32_t offa[8], offb[8];
+  // Per slab a wave issues four loads for A and four for B: load i covers rows
+  // 64 wave + 16 i .. + 16 (one 64-byte row per 4 lanes).  The lane at position
+  // pc of row r fetches chunk pc ^ ((r >> 2) & 3) = pc ^ (lane >> 4).  Rows past
+  // the end repeat the last one (what they produce lands in output rows that
+  // are never stored or in columns N..ldc-1 of T, which no consumer reads); a
+  // chunk past K is fetched from the row's first slab instead and zeroed in
+  // LDS before the slab is used.
+  const int ld_r = lane >> 2;
+  const int ld_c = (lane & 3) ^ (lane >> 4);
+  uint32_t offa[4], offb[4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = ld_row + 32 * i;
+  for (int i = 0; i < 4; ++i) {
+    const int row = 64 * wave + 16 * i + ld_r;
     offa[i] = ((uint32_t)min(m0 + row, g.M - 1) * (uint32_t)g.lda + ld_c * 8) * 2u;
     offb[i] = ((uint32_t)min(n0 + row, g.N - 1) * (uint32_t)g.ldb + ld_c * 8) * 2u;
   }
-  // Two register sets: while slab kt is multiplied out of LDS, slab kt + 1
-  // waits in one set for its turn in the idle LDS buffer and slab kt + 2 is in
-  // flight to the other, so a load has a whole slab of MFMA work (about 1 us)
-  // plus its own issue time to come back before anything waits for it.
-  u32x4 ra[2][8], rb[2][8];
-  bool k_ok[2] = {true, true};
-  uint32_t kb[2] = {0, 0};
-  auto gload_begin = [&](int set, int kt) {  // kt may run past the last slab: such a slab is all zeros
+  // Half a slab: `first` = the wave's four loads of A, else its four of B.
+  // kt may run past the last slab (such loads re-read slab 0 and are never used).
+  auto slab_load = [&](char* dst, int kt, bool first) {
     const int k0 = kt * CK;
-    k_ok[set] = k0 + ld_c * 8 < g.K;
-    kb[set] = k_ok[set] ? (uint32_t)k0 * 2u : 0u;
-  };
-  // chunk q of a slab: q < 8 is row group q of A, q >= 8 row group q - 8 of B
-  auto gload = [&](int set, int q0, int q1) {
+    const uint32_t kb = k0 + ld_c * 8 < g.K ? (uint32_t)k0 * 2u : 0u;
 #pragma unroll
-    for (int q = q0; q < q1; ++q) {
-      if (q < 8) ra[set][q] = *reinterpret_cast<const u32x4*>(A + (offa[q] + kb[set]));
-      else rb[set][q - 8] = *reinterpret_cast<const u32x4*>(B + (offb[q - 8] + kb[set]));
+    for (int i = 0; i < 4; ++i) {
+      if (first) load_to_lds(A, offa[i] + kb, dst + (64 * wave + 16 * i) * ROWB);
+      else load_to_lds(B, offb[i] + kb, dst + SLAB_A + (64 * wave + 16 * i) * ROWB);
     }
   };
-  auto sstore = [&](int set, int buf) {
-    bf16_t* sA = smem + buf * STAGE;
-    bf16_t* sB = sA + CM * LDT;
-    if (!k_ok[set]) {
-      const u32x4 z = {0, 0, 0, 0};
-#pragma unroll
-      for (int i = 0; i < 8; ++i) ra[set][i] = rb[set][i] = z;
+  // Chunks at or past K of slab kt (the last slab, and the all-zero slabs that
+  // pad the slab count to a multiple of four): thread t clears them in row t
+  // of A and row t of B.  Every wave's loads of the slab must have landed.
+  auto slab_clear_tail = [&](char* b, int kt) {
+    const int valid = max(0, min(4, (g.K - kt * CK) >> 3));
+    const u32x4 z = {0, 0, 0, 0};
+    const int swz = (tid >> 2) & 3;
+    for (int c = valid; c < 4; ++c) {
+      *reinterpret_cast<u32x4*>(b + tid * ROWB + ((c ^ swz) << 4)) = z;
+      *reinterpret_cast<u32x4*>(b + SLAB_A + tid * ROWB + ((c ^ swz) << 4)) = z;
     }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(sA + (ld_row + 32 * i) * LDT + ld_c * 8) = ra[set][i];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(sB + (ld_row + 32 * i) * LDT + ld_c * 8) = rb[set][i];
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   };
+
+  // Fragment (row R = base + 32 t + l31, k-step ks, half hh) is chunk 2 ks + hh
+  // of row R, at position (2 ks + hh) ^ ((R >> 2) & 3); the bases are multiples
+  // of 32, so the permutation depends on l31 only.
+  uint32_t fo[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) fo[ks] = (uint32_t)(l31 * ROWB + (((2 * ks + hh) ^ ((l31 >> 2) & 3)) << 4));
+  const uint32_t a_base = (uint32_t)(wm * ROWB), b_base = (uint32_t)(SLAB_A + wn * ROWB);
 
   // acc[jt][it] = (T^T) tile: rows j = wn + 32 jt + .., columns i = wm + 32 it + ..
   f32x16 acc[4][4];
@@ -113,102 +156,95 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[jt][it][r] = 0.f;
 
-  const int nk = (g.K + CK - 1) / CK;
-  gload_begin(0, 0);
-  gload(0, 0, 16);
-  gload_begin(1, 1);
-  gload(1, 0, 16);
-  sstore(0, 0);
-  lds_barrier();
-
-  // One slab = four k-steps of 16 MFMAs.  A lone wave per SIMD has nobody to
-  // cover for it, and a burst of 16 global loads or 16 LDS stores blocks the
-  // wave's instruction stream for longer than a k-step of MFMAs takes (the
-  // memory pipeline accepts a CU's 64 KB slab no faster than 64 B per cycle).
-  // So everything is spread over the MFMA stream, and the scheduler is told the
-  // interleave explicitly:
-  //   k-steps 0-2: a third of slab kt + 2's loads + the next step's fragments
-  //                between the MFMAs
-  //   k-step 3: slab kt + 1 goes from its registers to the idle LDS buffer
-  // No load or store is decided by a branch: slabs past the end are fetched
-  // from offset 0 and stored as zeros.
-  auto stage = [&](int kt, auto par_c) {
-    constexpr int par = decltype(par_c)::value;  // kt & 1: LDS buffer read, register set refilled
-    const bf16_t* sA = smem + par * STAGE;
-    const bf16_t* sB = sA + CM * LDT;
-    bf16x8 fa[2][4], fb[2][4];
-    auto frags = [&](int set, int ks) {
+  bf16x8 fa[2][4], fb[2][4];  // set 0: first k-step of a slab, set 1: second
+  auto frags = [&](int set, const char* b, int ks) {
 #pragma unroll
-      for (int it = 0; it < 4; ++it) fa[set][it] = lds_frag(sA, LDT, wm + 32 * it, ks * 16, lane);
+    for (int it = 0; it < 4; ++it)
+      fa[set][it] = as_frag(*reinterpret_cast<const u32x4*>(b + a_base + it * (32 * ROWB) + fo[ks]));
 #pragma unroll
-      for (int jt = 0; jt < 4; ++jt) fb[set][jt] = lds_frag(sB, LDT, wn + 32 * jt, ks * 16, lane);
-    };
-    auto mfmas = [&](int set) {
-#pragma unroll
-      for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-        for (int it = 0; it < 4; ++it) acc[jt][it] = mfma32(fb[set][jt], fa[set][it], acc[jt][it]);
-    };
-    frags(0, 0);
-    gload_begin(par, kt + 2);
-    __builtin_amdgcn_sched_barrier(0);
-    // k-step 0
-    gload(par, 0, 6);
-    frags(1, 1);
-    mfmas(0);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);             // two MFMAs
-      if (i < 6) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // one LDS read
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    // k-step 1
-    gload(par, 6, 11);
-    frags(0, 2);
-    mfmas(1);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      if (i < 5) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    // k-step 2
-    gload(par, 11, 16);
-    frags(1, 3);
-    mfmas(0);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      if (i < 5) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    // k-step 3
-    mfmas(1);
-    sstore(par ^ 1, par ^ 1);
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // one LDS store
-    }
-    lds_barrier();
+    for (int jt = 0; jt < 4; ++jt)
+      fb[set][jt] = as_frag(*reinterpret_cast<const u32x4*>(b + b_base + jt * (32 * ROWB) + fo[ks]));
   };
-  // Two stages per trip (the register sets and LDS buffers are addressed
-  // statically); an odd slab count runs one extra stage on an all-zero slab.
-  for (int kt = 0; kt < nk; kt += 2) {
+  auto mfmas = [&](int set) {
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+      for (int it = 0; it < 4; ++it) acc[jt][it] = mfma32(fb[set][jt], fa[set][it], acc[jt][it]);
+  };
+  // 16 MFMAs with 8 fragment reads and 4 loads between them
+  auto interleave = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // two MFMAs
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+  };
+
+  const int nk = (g.K + CK - 1) / CK;
+  const int nk4 = (nk + 3) & ~3;  // stages come in fours (the buffers are addressed statically)
+  // Loads in flight, oldest first, whenever a wave reaches the barrier of
+  // slab kt: [slab kt + 1] [slab kt + 2] [slab kt + 3]; the barrier needs the
+  // first group, so 16 may stay outstanding.
+  slab_load(sb0, 0, true);
+  slab_load(sb0, 0, false);
+  slab_load(sb1, 1, true);
+  slab_load(sb1, 1, false);
+  slab_load(sb2, 2, true);
+  slab_load(sb2, 2, false);
+  slab_load(sb3, 3, true);
+  wait_loads_but<20>();
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  if (CK > g.K) slab_clear_tail(sb0, 0);
+  frags(0, sb0, 0);
+
+  auto stage = [&](int kt, auto b_c) {
+    constexpr int b = decltype(b_c)::value;  // kt & 3
+    char* cur = buf(b);
+    char* nxt = buf(b + 1);
+    // first k-step (fragments already in set 0); meanwhile the second k-step's
+    // fragments and the B half of slab kt + 3
+    frags(1, cur, 1);
+    slab_load(buf(b + 3), kt + 3, false);
+    mfmas(0);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    // This wave has read all it needs of slab kt; its share of slab kt + 1 has
+    // landed once at most 16 younger loads are outstanding.  Past the barrier
+    // that holds for every wave: slab kt + 1 is complete, buffer b is free.
+    wait_loads_but<16>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if ((kt + 2) * CK > g.K && kt + 1 < nk4) slab_clear_tail(nxt, kt + 1);
+    // second k-step; meanwhile the next slab's first fragments and the A half
+    // of slab kt + 4 into the buffer just freed
+    frags(0, nxt, 0);
+    slab_load(cur, kt + 4, true);
+    mfmas(1);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  for (int kt = 0; kt < nk4; kt += 4) {
     stage(kt, std::integral_constant<int, 0>{});
     stage(kt + 1, std::integral_constant<int, 1>{});
+    stage(kt + 2, std::integral_constant<int, 2>{});
+    stage(kt + 3, std::integral_constant<int, 3>{});
   }
 
   // ------------------------------------------------------------- epilogue
-  // Every wave has passed the last barrier, so the slabs are dead.  A wave
-  // stages its own 128x128 quadrant (rows i, columns j) and reads it back
-  // itself (a wave's LDS operations execute in order): no further barrier.
+  // Drain the loads that ran ahead (they target the buffers about to be
+  // reused) and let every wave finish its fragment reads.  Then a wave stages
+  // its own 128x128 quadrant (rows i, columns j) in buffer `wave` and reads it
+  // back itself (a wave's LDS operations execute in order): no further barrier.
   // Lane (l31, hh), register quad q of tile (jt, it): row i = 32 it + l31,
   // columns j = 32 jt + 8 q + 4 hh + 0..3.
-  bf16_t* sE = smem + wave * (128 * LDE);
+  wait_loads_but<0>();
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  bf16_t* sE = reinterpret_cast<bf16_t*>(buf(wave));
 #pragma unroll
   for (int jt = 0; jt < 4; ++jt)
 #pragma unroll

@@ -310,11 +310,17 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   gload_kv(0);
   gload_bias(rb);
   sstore(0);
+  gload_kv(KT);
   lds_barrier();
 
   for (int kt = 0; kt < nkt; ++kt) {
     const int buf = kt & 1;
-    const bool more = kt + 1 < nkt;
+    // Tile kt + 1, fetched during the previous iteration, goes to the other
+    // buffer (last read in iteration kt - 1, which every wave left through the
+    // barrier at its end); its registers then take tile kt + 2.  Past the last
+    // tile both are clamped re-reads whose stores nobody reads.
+    sstore(buf ^ 1);
+    gload_kv((kt + 2) * KT);
     // Both 32-key halves of the tile go through the matrix unit first (two
     // independent accumulator chains), then one online-softmax update covers
     // all 64 keys, then both halves feed O.  A half that lies wholly beyond N
@@ -333,11 +339,9 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
       for (int ks = 0; ks < 3; ++ks)
         s[u] = mfma32(lds_frag(sK[buf], LDK, u * 32, ks * 16, lane), qf[ks], s[u]);
     }
-    // Global loads are issued here, behind the score MFMAs: the bias registers
-    // are free again, and the K / V loads come first so that their consumer (the
-    // LDS store at the end of this tile) does not have to wait for the bias
-    // loads queued behind them (vector memory operations retire in order).
-    gload_kv((kt + 1) * KT);
+    // The next tile's bias is fetched here, behind the score MFMAs, when its
+    // registers are free again; like the K / V loads at the top of the loop it
+    // is first looked at at the top of the next iteration.
     gload_bias(rb);
     float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
 #pragma unroll
@@ -385,12 +389,7 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
         vv.x = lo.x; vv.y = lo.y; vv.z = hi.x; vv.w = hi.y;
         o = mfma32(as_frag(vv), pf[u][half], o);
       }
-    if (more) {
-      // buffer buf ^ 1 was last read in the previous iteration, which every
-      // wave left through the barrier below
-      sstore(buf ^ 1);
-      lds_barrier();
-    }
+    lds_barrier();
   }
 
   const float inv = 1.f / l_run;  // l_run already holds the sum over both half-waves' keys

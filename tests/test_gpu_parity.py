@@ -404,7 +404,7 @@ def test_bad_shape_is_rejected(gpu_pkg):
 
 
 # ---------------------------------------------------------- kernel-level entries
-@pytest.mark.parametrize("n", [70, 130, 256, 300, 520])
+@pytest.mark.parametrize("n", [70, 130, 256, 300, 360, 520])
 def test_kernel_level_contraction(gpu_pkg, n):
     note(f"test_kernel_level_contraction n={n}")
     g = gen(n)
