@@ -9,6 +9,8 @@
 // This kernel carries the triangle-multiplication contraction (batch = 128
 // channels, M = N = K = N_token) and every dense projection outside the
 // 128-channel pair path (single / diffusion / atom attention and transitions).
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -46,9 +48,13 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
   const bf16_t* A = g.A + (int64_t)bz * g.sA;
   const bf16_t* B = g.B + (int64_t)bz * g.sB;
 
-  // each thread moves 4 16-byte chunks of A and 4 of B per k slab
+  // each thread moves 4 16-byte chunks of A and 4 of B per k slab.  Two register
+  // sets: a slab is requested two iterations before it goes to LDS.  The small
+  // products this kernel is mostly used for (a few hundred rows, K = 384 ...
+  // 1536) run on fewer workgroups than there are CUs, so each workgroup is one
+  // chain of K / 64 memory round trips and nothing else covers their latency.
   const int ld_row = tid >> 3, ld_kc = (tid & 7) * 8;  // + 32 rows per step
-  u32x4 ra[4], rb[4];
+  u32x4 ra[2][4], rb[2][4];
   const bf16_t* pa[4];
   const bf16_t* pb[4];
 #pragma unroll
@@ -57,21 +63,25 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
     pa[i] = A + (int64_t)min(m0 + row, g.M - 1) * g.lda + ld_kc;
     pb[i] = B + (int64_t)min(n0 + row, g.N - 1) * g.ldb + ld_kc;
   }
-  auto gload = [&](int k0) {
-    const bool ok = k0 + ld_kc < g.K;
+  // unconditional loads (a chunk past K re-reads the row's first one) whose
+  // values are zeroed on their way to LDS
+  bool k_ok[2] = {true, true};
+  auto gload = [&](int set, int k0) {
+    k_ok[set] = k0 + ld_kc < g.K;
+    const int kk = k_ok[set] ? k0 : -ld_kc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ra[set][i] = *reinterpret_cast<const u32x4*>(pa[i] + kk);
+      rb[set][i] = *reinterpret_cast<const u32x4*>(pb[i] + kk);
+    }
+  };
+  auto sstore = [&](int set, int buf) {
     const u32x4 z = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      ra[i] = ok ? *reinterpret_cast<const u32x4*>(pa[i] + k0) : z;
-      rb[i] = ok ? *reinterpret_cast<const u32x4*>(pb[i] + k0) : z;
-    }
-  };
-  auto sstore = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
       const int row = ld_row + 32 * i;
-      *reinterpret_cast<u32x4*>(smem + buf * STAGE + row * LDT + ld_kc) = ra[i];
-      *reinterpret_cast<u32x4*>(smem + buf * STAGE + (BM + row) * LDT + ld_kc) = rb[i];
+      *reinterpret_cast<u32x4*>(smem + buf * STAGE + row * LDT + ld_kc) = k_ok[set] ? ra[set][i] : z;
+      *reinterpret_cast<u32x4*>(smem + buf * STAGE + (BM + row) * LDT + ld_kc) = k_ok[set] ? rb[set][i] : z;
     }
   };
 
@@ -84,27 +94,34 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   const int nk = (g.K + BK - 1) / BK;
-  gload(0);
-  sstore(0);
+  gload(0, 0);
+  gload(1, BK);  // past K when nk == 1: a clamped re-read, never stored
+  sstore(0, 0);
   lds_barrier();
 
-  for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < nk) gload((kt + 1) * BK);
+  // slab kt is in LDS buffer kt & 1, slab kt + 1 in register set (kt + 1) & 1,
+  // and set kt & 1 (just stored) takes slab kt + 2
+  auto stage = [&](int kt, auto par_c) {
+    constexpr int par = decltype(par_c)::value;
+    if (kt + 2 < nk) gload(par, (kt + 2) * BK);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       bf16x8 fa[2], fb[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) fa[i] = lds_frag(smem + buf * STAGE, LDT, wm + 32 * i, ks * 16, lane);
+      for (int i = 0; i < 2; ++i) fa[i] = lds_frag(smem + par * STAGE, LDT, wm + 32 * i, ks * 16, lane);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) fb[j] = lds_frag(smem + buf * STAGE + BM * LDT, LDT, wn + 32 * j, ks * 16, lane);
+      for (int j = 0; j < 2; ++j) fb[j] = lds_frag(smem + par * STAGE + BM * LDT, LDT, wn + 32 * j, ks * 16, lane);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(fa[i], fb[j], acc[i][j]);
     }
-    if (kt + 1 < nk) sstore(buf ^ 1);
+    if (kt + 1 < nk) sstore(par ^ 1, par ^ 1);
     lds_barrier();
+  };
+  for (int kt = 0; kt < nk; kt += 2) {
+    stage(kt, std::integral_constant<int, 0>{});
+    if (kt + 1 < nk) stage(kt + 1, std::integral_constant<int, 1>{});
   }
 
   // ------------------------------------------------------------- epilogue
