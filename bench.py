@@ -59,13 +59,20 @@ def flops_attention_core(n):  # QK^T and PV for N rows x 4 heads x d=32
     return 512.0 * n ** 3
 
 
-def gpu_time_ms(fn, iters, warmup=2):
+def gpu_time_ms(fn, iters, warmup=2, warm_ms=0.0):
     """Average duration of fn() in ms, timed with HIP events on torch's current
-    stream (the stream handed to the C ABI)."""
+    stream (the stream handed to the C ABI).  `warm_ms`: keep launching untimed
+    until that much wall time has passed (after an idle stretch the GPU clock
+    takes some tens of milliseconds to come back to its sustained level)."""
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < warm_ms:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(iters):
@@ -186,8 +193,9 @@ def main():
     nb = pkg.ops.pack_pair_bias(torch.randn(4, n, npad, generator=g).to(dev).bfloat16())
     vt_[..., n:] = 0
     og = torch.empty((n * n, 128), dtype=torch.bfloat16, device=dev)
-    ms_contract = gpu_time_ms(lambda: pkg.ops.triangle_contraction(a, b, t_buf), it)
-    ms_attn = gpu_time_ms(lambda: pkg.ops.grid_attention_core(q_, k_, vt_, g_, nb, pair_mask, og), it)
+    # (the operands above are generated on the host, during which the GPU idles and its clock drops)
+    ms_contract = gpu_time_ms(lambda: pkg.ops.triangle_contraction(a, b, t_buf), 30, warm_ms=40.0)
+    ms_attn = gpu_time_ms(lambda: pkg.ops.grid_attention_core(q_, k_, vt_, g_, nb, pair_mask, og), 30, warm_ms=40.0)
     kernels = {
         "contract_kernel (triangle contraction)": (ms_contract, flops_contraction(n)),
         "triattn_flash_kernel (triangle attention core)": (ms_attn, flops_attention_core(n)),
