@@ -37,12 +37,18 @@ class AdaptiveLayerNorm(HipModule):
         b = torch.cat([self.single_cond_scale.bias, torch.zeros_like(self.single_cond_scale.bias)])
         return dict(cond_ln_w=f32(self.single_cond_layer_norm.weight), w_ss=bf16(w), b_ss=f32(b))
 
-    def forward(self, x: torch.Tensor, single_cond: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, single_cond: Optional[torch.Tensor] = None,
+                scale_shift: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """`scale_shift`: fp32 [cond_rows, 2 c_x] view (unit column stride) holding
+        what the two conditioning projections of this module give for
+        `single_cond`, computed by the caller for many modules at once."""
         assert (single_cond is None) == (self.use_single_cond is False)
         if in_check_mode():
             return check.adaptive_layer_norm(self, x, single_cond)
-        p = self.packed()
         x = x.contiguous()
+        if scale_shift is not None:
+            return ops.layer_norm(x, scale=scale_shift[:, :self.c_x], shift=scale_shift[:, self.c_x:])
+        p = self.packed()
         if not self.use_single_cond:
             return ops.layer_norm(x, p["ln_w"], p["ln_b"])
         s = ops.layer_norm(single_cond.contiguous(), p["cond_ln_w"])
@@ -74,12 +80,13 @@ class AdaLNZero(HipModule):
             d["b_cond"] = f32(self.adaptive_zero_cond.bias)
         return d
 
-    def run(self, x, single_cond, out_dtype, residual=None):
+    def run(self, x, single_cond, out_dtype, residual=None, gate=None):
         """x bf16 [..., c_in] -> [..., c_out]; `residual` (same shape as the
-        result) is added and overwritten in place when given."""
+        result) is added and overwritten in place when given.  `gate`: the
+        sigmoid of this module's conditioning projection, fp32 [cond_rows,
+        c_out] contiguous, when the caller has computed it already."""
         p = self.packed()
-        gate = None
-        if self.use_single_cond:
+        if self.use_single_cond and gate is None:
             gate = ops.linear(single_cond.to(torch.bfloat16).contiguous(), p["w_cond"], bias=p["b_cond"],
                               out_dtype=torch.float32, sigmoid=True)
         return ops.linear(x, p["w"], out_dtype=out_dtype, mode=L.LINEAR_GATE_RES, gate=gate,
@@ -111,10 +118,12 @@ class DiffusionTransition(HipModule):
     def _pack(self):
         return dict(w1=bf16(pack_swiglu(self.transition1.weight, 32)))
 
-    def run(self, x, single_cond, residual: bool):
-        xa = self.adaptive_layernorm(x, single_cond)
+    def run(self, x, single_cond, residual: bool, cond=None):
+        """`cond` = (scale_shift, gate) computed by the caller, see AdaptiveLayerNorm / AdaLNZero."""
+        ss, gate = cond if cond is not None else (None, None)
+        xa = self.adaptive_layernorm(x, single_cond, scale_shift=ss)
         h = ops.linear(xa, self.packed()["w1"], mode=L.LINEAR_SWIGLU)
-        return self.adaptive_zero_init.run(h, single_cond, x.dtype, residual=x if residual else None)
+        return self.adaptive_zero_init.run(h, single_cond, x.dtype, residual=x if residual else None, gate=gate)
 
     def forward(self, x: torch.Tensor, single_cond: Optional[torch.Tensor] = None) -> torch.Tensor:
         if in_check_mode():
@@ -150,9 +159,11 @@ class SelfAttention(HipModule):
                        self.gating_query.weight], dim=0)
         return dict(w_qkvg=bf16(w), q_b=f32(self.q_projection.bias))
 
-    def run(self, x, mask, pair_logits, single_cond, residual: bool):
+    def run(self, x, mask, pair_logits, single_cond, residual: bool, cond=None):
+        """`cond` = (scale_shift, gate) computed by the caller, see AdaptiveLayerNorm / AdaLNZero."""
         p = self.packed()
-        xa = self.adaptive_layernorm(x, single_cond)
+        ss, gate = cond if cond is not None else (None, None)
+        xa = self.adaptive_layernorm(x, single_cond, scale_shift=ss)
         batched = xa.dim() == 3
         xb = xa if batched else xa.unsqueeze(0)
         if pair_logits is not None:
@@ -161,7 +172,7 @@ class SelfAttention(HipModule):
         avg = avg.reshape(xb.shape)
         if not batched:
             avg = avg.squeeze(0)
-        return self.adaptive_zero_init.run(avg, single_cond, x.dtype, residual=x if residual else None)
+        return self.adaptive_zero_init.run(avg, single_cond, x.dtype, residual=x if residual else None, gate=gate)
 
     def forward(self, x: torch.Tensor, mask: torch.Tensor, pair_logits: Optional[torch.Tensor] = None,
                 single_cond: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -201,8 +212,27 @@ class DiffusionTransformer(HipModule):
              for _ in range(num_blocks)])
 
     def _pack(self):
+        # Every block conditions on the same single_cond, so the 4 conditioning
+        # projections of each block (adaptive LayerNorm scale | shift and the
+        # AdaLN-Zero gate, for the attention and for the transition) are taken
+        # out of the blocks: two products for all blocks before the first one.
+        # Each adaptive LayerNorm normalises single_cond with its own weight and
+        # no bias, LN_w(s) W^T = LN_1(s) (W diag(w))^T, so the weight goes into
+        # the projection and one plain normalisation serves them all.
+        w_ss, b_ss, w_gate, b_gate = [], [], [], []
+        for att, tr in zip(self.self_attention, self.transition_block):
+            for m in (att, tr):
+                aln, az = m.adaptive_layernorm, m.adaptive_zero_init
+                lnw = aln.single_cond_layer_norm.weight.detach().float()
+                w = torch.cat([aln.single_cond_scale.weight, aln.single_cond_bias.weight], dim=0).detach().float()
+                w_ss.append(w * lnw[None, :])
+                b_ss.append(torch.cat([aln.single_cond_scale.bias, torch.zeros_like(aln.single_cond_scale.bias)]))
+                w_gate.append(az.adaptive_zero_cond.weight)
+                b_gate.append(az.adaptive_zero_cond.bias)
         return dict(ln_w=f32(self.pair_input_layer_norm.weight),
-                    w_logits=[pad_rows(bf16(m.weight), 32) for m in self.pair_logits_projection])
+                    w_logits=[pad_rows(bf16(m.weight), 32) for m in self.pair_logits_projection],
+                    w_ss=bf16(torch.cat(w_ss, dim=0)), b_ss=f32(torch.cat(b_ss)),
+                    w_gate=bf16(torch.cat(w_gate, dim=0)), b_gate=f32(torch.cat(b_gate)))
 
     def forward(self, act: torch.Tensor, mask: torch.Tensor, single_cond: torch.Tensor,
                 pair_cond: torch.Tensor) -> torch.Tensor:
@@ -215,13 +245,23 @@ class DiffusionTransformer(HipModule):
         if not act.is_contiguous():
             raise ValueError("act must be contiguous (it is updated in place)")
         n_out = self.super_block_size * self.num_head
+        c, n_mod = self.c_act, 2 * self.num_blocks
+        sc = single_cond.contiguous()
+        rows = sc.numel() // sc.shape[-1]
+        ss_all = ops.linear(ops.layer_norm(sc), p["w_ss"], bias=p["b_ss"], out_dtype=torch.float32)
+        ss_all = ss_all.view(rows, n_mod, 2 * c)                       # column slices, read in place
+        gate_all = ops.linear(sc.to(torch.bfloat16), p["w_gate"], bias=p["b_gate"], out_dtype=torch.float32,
+                              sigmoid=True)
+        gate_all = gate_all.view(rows, n_mod, c).permute(1, 0, 2).contiguous()   # [module][row][c]
         for sb in range(self.num_super_blocks):
             logits = ops.pair_logits(pair_cond, p["ln_w"], None, p["w_logits"][sb], n_out)
             logits = logits.view(self.super_block_size, self.num_head, *logits.shape[1:])  # (b h) n s -> b h n s
             for j in range(self.super_block_size):
                 i = sb * self.super_block_size + j
-                self.self_attention[i].run(act, mask, logits[j], single_cond, residual=True)
-                self.transition_block[i].run(act, single_cond, residual=True)
+                self.self_attention[i].run(act, mask, logits[j], single_cond, residual=True,
+                                           cond=(ss_all[:, 2 * i], gate_all[2 * i]))
+                self.transition_block[i].run(act, single_cond, residual=True,
+                                             cond=(ss_all[:, 2 * i + 1], gate_all[2 * i + 1]))
         return act
 
 
@@ -256,12 +296,14 @@ class CrossAttention(HipModule):
             w_kv=bf16(torch.cat([self.k_projection.weight, self.v_projection.weight], dim=0)),
             q_b=f32(self.q_projection.bias))
 
-    def run(self, x_q, x_k, mask_q, mask_k, pair_logits, single_cond_q, single_cond_k, residual: bool):
+    def run(self, x_q, x_k, mask_q, mask_k, pair_logits, single_cond_q, single_cond_k, residual: bool, cond=None):
+        """`cond` = (scale_shift_q, scale_shift_k, gate) computed by the caller, see AdaptiveLayerNorm / AdaLNZero."""
         p = self.packed()
         n_sub, n_q, c = x_q.shape[-3:]
         n_k = x_k.shape[-2]
-        xq = self.q_adaptive_layernorm(x_q, single_cond_q)
-        xk = self.k_adaptive_layernorm(x_k, single_cond_k)
+        ss_q, ss_k, gate = cond if cond is not None else (None, None, None)
+        xq = self.q_adaptive_layernorm(x_q, single_cond_q, scale_shift=ss_q)
+        xk = self.k_adaptive_layernorm(x_k, single_cond_k, scale_shift=ss_k)
         mq = mask_q.reshape(-1, n_q)
         mk = mask_k.reshape(-1, n_k)
         pl = None
@@ -271,7 +313,8 @@ class CrossAttention(HipModule):
             xq.reshape(-1, n_q, c), xk.reshape(-1, n_k, c), pl, mq, mk, p["w_qg"], p["w_kv"], p["q_b"],
             self.num_head)
         avg = avg.reshape(x_q.shape)
-        return self.adaptive_zero_init.run(avg, single_cond_q, x_q.dtype, residual=x_q if residual else None)
+        return self.adaptive_zero_init.run(avg, single_cond_q, x_q.dtype, residual=x_q if residual else None,
+                                           gate=gate)
 
     def forward(self, x_q, x_k, mask_q, mask_k, pair_logits=None, single_cond_q=None, single_cond_k=None):
         """x_q [(B,) S, Q, c], x_k [(B,) S, K, c], masks [(1,) S, Q] / [(1,) S, K],
@@ -308,7 +351,29 @@ class DiffusionCrossAttTransformer(HipModule):
              for _ in range(num_blocks)])
 
     def _pack(self):
-        return dict(ln_w=f32(self.pair_input_layer_norm.weight), w=bf16(self.pair_logits_projection.weight))
+        # The conditioning inputs are the same for every block: all adaptive
+        # LayerNorm scale | shift projections and AdaLN-Zero gates are computed
+        # before the first block, one product per input (see DiffusionTransformer._pack).
+        def ss(aln):
+            w = torch.cat([aln.single_cond_scale.weight, aln.single_cond_bias.weight], dim=0).detach().float()
+            b = torch.cat([aln.single_cond_scale.bias, torch.zeros_like(aln.single_cond_scale.bias)])
+            return w * aln.single_cond_layer_norm.weight.detach().float()[None, :], b
+        wq, bq, wk, bk, wg, bg = [], [], [], [], [], []
+        for ca, tr in zip(self.cross_attention, self.transition_block):
+            for aln in (ca.q_adaptive_layernorm, tr.adaptive_layernorm):
+                w, b = ss(aln)
+                wq.append(w)
+                bq.append(b)
+            w, b = ss(ca.k_adaptive_layernorm)
+            wk.append(w)
+            bk.append(b)
+            for az in (ca.adaptive_zero_init, tr.adaptive_zero_init):
+                wg.append(az.adaptive_zero_cond.weight)
+                bg.append(az.adaptive_zero_cond.bias)
+        return dict(ln_w=f32(self.pair_input_layer_norm.weight), w=bf16(self.pair_logits_projection.weight),
+                    w_ss_q=bf16(torch.cat(wq, dim=0)), b_ss_q=f32(torch.cat(bq)),
+                    w_ss_k=bf16(torch.cat(wk, dim=0)), b_ss_k=f32(torch.cat(bk)),
+                    w_gate=bf16(torch.cat(wg, dim=0)), b_gate=f32(torch.cat(bg)))
 
     @staticmethod
     def _gather(queries_to_keys, queries_act):
@@ -334,9 +399,21 @@ class DiffusionCrossAttTransformer(HipModule):
         logits = ops.linear(pair_act, p["w"], out_dtype=torch.float32)           # [S, Q, K, (b h)]
         s, q, k, _ = logits.shape
         logits = logits.reshape(s, q, k, self.num_blocks, self.num_head).permute(3, 0, 4, 1, 2).contiguous()
+        c = self.c_query
+        cq = queries_single_cond.contiguous()
+        ck = keys_single_cond.contiguous()
+        rq, rk = cq.numel() // cq.shape[-1], ck.numel() // ck.shape[-1]
+        ss_q = ops.linear(ops.layer_norm(cq), p["w_ss_q"], bias=p["b_ss_q"], out_dtype=torch.float32)
+        ss_q = ss_q.view(rq, 2 * self.num_blocks, 2 * c)                # column slices, read in place
+        ss_k = ops.linear(ops.layer_norm(ck), p["w_ss_k"], bias=p["b_ss_k"], out_dtype=torch.float32)
+        ss_k = ss_k.view(rk, self.num_blocks, 2 * c)
+        gate = ops.linear(cq.to(torch.bfloat16), p["w_gate"], bias=p["b_gate"], out_dtype=torch.float32, sigmoid=True)
+        gate = gate.view(rq, 2 * self.num_blocks, c).permute(1, 0, 2).contiguous()   # [module][row][c]
         for blk in range(self.num_blocks):
             keys_act = self._gather(queries_to_keys, queries_act)
             self.cross_attention[blk].run(queries_act, keys_act, queries_mask, keys_mask, logits[blk],
-                                          queries_single_cond, keys_single_cond, residual=True)
-            self.transition_block[blk].run(queries_act, queries_single_cond, residual=True)
+                                          queries_single_cond, keys_single_cond, residual=True,
+                                          cond=(ss_q[:, 2 * blk], ss_k[:, blk], gate[2 * blk]))
+            self.transition_block[blk].run(queries_act, queries_single_cond, residual=True,
+                                           cond=(ss_q[:, 2 * blk + 1], gate[2 * blk + 1]))
         return queries_act
