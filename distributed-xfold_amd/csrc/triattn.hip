@@ -278,13 +278,11 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   const char* bbase = HAS_BIAS ? reinterpret_cast<const char*>(a.bias + tri_bias_offset(N, h, qblock * 32, 0)) : nullptr;
   const uint32_t b_lane = (uint32_t)(j * 16 + 8 * hh) * 2u;
   const int bias_tiles = (int)tri_bias_ktiles(N);
-  int bias_next = 0;  // tile the next gload_bias fetches; stops at the last one
-  auto gload_bias = [&](u32x4* dst) {
+  auto gload_bias = [&](u32x4* dst, int tile) {  // a tile past the end re-reads the last one
     if (!HAS_BIAS) return;
-    const char* p = bbase + (size_t)min(bias_next, bias_tiles - 1) * 4096u;
+    const char* p = bbase + (size_t)min(tile, bias_tiles - 1) * 4096u;
 #pragma unroll
     for (int i = 0; i < 4; ++i) dst[i] = *reinterpret_cast<const u32x4*>(p + (b_lane + 1024u * i));
-    ++bias_next;
   };
   auto sstore = [&](int buf) {
     const u32x4 z = {0, 0, 0, 0};
@@ -307,20 +305,55 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   float m_run = -__builtin_huge_valf(), l_run = 0.f;
 
   const int nkt = (N + KT - 1) / KT;
-  gload_kv(0);
-  gload_bias(rb);
+  // Key tiles whose 64 keys are all masked contribute exactly nothing to a row
+  // that has an unmasked key anywhere (their probabilities underflow to zero, or
+  // are scaled by exactly zero when the first unmasked key raises the running
+  // maximum), so they are left out: same bits, fewer tiles - with padded inputs
+  // every row skips the padding's tiles.  A row with no unmasked key at all
+  // keeps every tile (its softmax is uniform over the masked keys).  The live
+  // tiles of the row as a bit mask, for up to 64 tiles.
+  uint64_t live = nkt >= 64 ? ~0ull : (1ull << nkt) - 1;
+  if (mbase && nkt <= 64) {
+    uint32_t* sLive = reinterpret_cast<uint32_t*>(&sK[1][0]);  // not yet in use
+    if (tid < 2) sLive[tid] = 0u;
+    lds_barrier();
+    for (int t0 = 0; t0 < nkt; t0 += 4) {
+      const int tile = t0 + wave, key = tile * KT + lane;
+      const float mv = *reinterpret_cast<const float*>(mbase + (uint32_t)min(key, N - 1) * 4u);
+      const bool on = key < N && mv != 0.f;
+      if (__ballot(on) != 0ull && lane == 0) atomicOr(&sLive[tile >> 5], 1u << (tile & 31));
+    }
+    lds_barrier();
+    const uint64_t m = (uint64_t)sLive[0] | ((uint64_t)sLive[1] << 32);
+    lds_barrier();  // sLive is read; the buffer may be written
+    if (m != 0ull) live = m;
+  }
+  const uint32_t live_lo = __builtin_amdgcn_readfirstlane((uint32_t)live);
+  const uint32_t live_hi = __builtin_amdgcn_readfirstlane((uint32_t)(live >> 32));
+  uint64_t rest = (uint64_t)live_lo | ((uint64_t)live_hi << 32);
+  // next live tile, or nkt (a tile past the end: clamped loads, every key at -inf, never used) when none is left
+  auto pop = [&]() {
+    if (rest == 0ull) return nkt;
+    const int tile = __builtin_ctzll(rest);
+    rest &= rest - 1;
+    return tile;
+  };
+  int t_cur = pop(), t_nxt = pop();
+  gload_kv(t_cur * KT);
+  gload_bias(rb, t_cur);
   sstore(0);
-  gload_kv(KT);
+  gload_kv(t_nxt * KT);
   lds_barrier();
 
-  for (int kt = 0; kt < nkt; ++kt) {
+  for (int kt = 0; t_cur < nkt; ++kt) {
     const int buf = kt & 1;
-    // Tile kt + 1, fetched during the previous iteration, goes to the other
-    // buffer (last read in iteration kt - 1, which every wave left through the
-    // barrier at its end); its registers then take tile kt + 2.  Past the last
-    // tile both are clamped re-reads whose stores nobody reads.
+    const int t_nn = pop();
+    // The next live tile, fetched during the previous iteration, goes to the
+    // other buffer (last read in the previous iteration, which every wave left
+    // through the barrier at its end); its registers then take the tile after
+    // it.  Past the last tile both are clamped re-reads whose stores nobody reads.
     sstore(buf ^ 1);
-    gload_kv((kt + 2) * KT);
+    gload_kv(t_nn * KT);
     // Both 32-key halves of the tile go through the matrix unit first (two
     // independent accumulator chains), then one online-softmax update covers
     // all 64 keys, then both halves feed O.  A half that lies wholly beyond N
@@ -342,7 +375,7 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
     // The next tile's bias is fetched here, behind the score MFMAs, when its
     // registers are free again; like the K / V loads at the top of the loop it
     // is first looked at at the top of the next iteration.
-    gload_bias(rb);
+    gload_bias(rb, t_nxt);
     float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
 #pragma unroll
     for (int u = 0; u < 2; ++u)
@@ -390,6 +423,8 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
         o = mfma32(as_frag(vv), pf[u][half], o);
       }
     lds_barrier();
+    t_cur = t_nxt;
+    t_nxt = t_nn;
   }
 
   const float inv = 1.f / l_run;  // l_run already holds the sum over both half-waves' keys

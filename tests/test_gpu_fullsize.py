@@ -52,14 +52,18 @@ def compare(name, got, ref, rms_tol=RMS_TOL, max_tol=MAX_TOL):
     assert rms <= rms_tol and mx <= max_tol, (name, rms, mx)
 
 
-def block_inputs(seed, live):
+def block_inputs(seed, live, trailing=False):
     g = gen(seed)
     p = rparams(O.make_pairformer_block_params(g))
     pair = O.round_bf16(torch.randn(N, N, 128, generator=g))
     single = O.round_bf16(torch.randn(N, 384, generator=g))
-    # padding scattered over the sequence, not only at its end
     seq = torch.ones(N)
-    seq[torch.randperm(N, generator=g)[: N - live]] = 0
+    if trailing:
+        # padding at the end: whole key tiles are masked (the attention core leaves them out)
+        seq[live:] = 0
+    else:
+        # padding scattered over the sequence
+        seq[torch.randperm(N, generator=g)[: N - live]] = 0
     pm = seq[:, None] * seq[None, :]
     return g, p, pair, single, seq, pm
 
@@ -106,8 +110,9 @@ def test_ending_node_attention_is_starting_node_attention_of_the_transpose(gpu_p
     compare("ending node vs transposed starting node", a.cpu(), b.cpu())
 
 
-def test_bf16_block_against_fp32_check_mode(gpu_pkg):
-    g, p, pair, single, seq, pm = block_inputs(13, 700)
+@pytest.mark.parametrize("live,trailing", [(700, False), (600, True)])
+def test_bf16_block_against_fp32_check_mode(gpu_pkg, live, trailing):
+    g, p, pair, single, seq, pm = block_inputs(13, live, trailing)
     blk = gpu_pkg.nn.PairformerBlock()
     blk.load_state_dict(p)
     blk.to(dev())

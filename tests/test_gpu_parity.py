@@ -418,11 +418,13 @@ def test_kernel_level_contraction(gpu_pkg, n):
     assert_within_bf16_ulp("contraction", t[:, :, :n], want, ulps=1.01, atol=1e-3)
 
 
-@pytest.mark.parametrize("n", [40, 200])
-def test_kernel_level_attention_core(gpu_pkg, n):
-    """Base-2 operands in, gate * softmax(q k^T + bias, masked) v out."""
-    note(f"test_kernel_level_attention_core n={n}")
-    g = gen(n)
+@pytest.mark.parametrize("n,tiles", [(40, False), (200, False), (200, True), (330, True)])
+def test_kernel_level_attention_core(gpu_pkg, n, tiles):
+    """Base-2 operands in, gate * softmax(q k^T + bias, masked) v out.  `tiles`:
+    whole 64-key tiles masked (the kernel leaves such tiles out for rows that
+    have an unmasked key elsewhere, which must not change a bit of the result)."""
+    note(f"test_kernel_level_attention_core n={n} tiles={tiles}")
+    g = gen(n + tiles)
     log2e = 1.4426950408889634
     npad = (n + 7) // 8 * 8
     qkvg = rb(torch.randn(n, n, 4, 4, 32, generator=g) * 0.7)       # [b, s, (q k v g), h, d]
@@ -431,6 +433,13 @@ def test_kernel_level_attention_core(gpu_pkg, n):
     bias[:, :, :n] = rb(torch.randn(4, n, n, generator=g))
     mask = (torch.rand(n, n, generator=g) > 0.2).float()
     mask[:, 0] = 1
+    if tiles:
+        mask[:, 64:128] = 0                                         # tile 1 masked for every row ...
+        mask[5, :] = 0
+        mask[5, 100] = 1                                            # ... but the only live one of row 5
+        mask[:, n - 70:] = 0                                        # trailing padding, more than a tile
+        mask[7, :] = 0
+        mask[7, n - 3] = 1                                          # row 7 lives in the last, partial tile only
     mask[3, :] = 0                                                  # one fully masked row
     hm = lambda i: qkvg[:, :, i].permute(0, 2, 1, 3).contiguous()       # [b, h, s, d]
     vt = torch.zeros(n, 4, 32, npad)
