@@ -313,6 +313,7 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   // keeps every tile (its softmax is uniform over the masked keys).  The live
   // tiles of the row as a bit mask, for up to 64 tiles.
   uint64_t live = nkt >= 64 ? ~0ull : (1ull << nkt) - 1;
+  bool row_dead = false;
   if (mbase && nkt <= 64) {
     uint32_t* sLive = reinterpret_cast<uint32_t*>(&sK[1][0]);  // not yet in use
     if (tid < 2) sLive[tid] = 0u;
@@ -327,6 +328,7 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
     const uint64_t m = (uint64_t)sLive[0] | ((uint64_t)sLive[1] << 32);
     lds_barrier();  // sLive is read; the buffer may be written
     if (m != 0ull) live = m;
+    else row_dead = true;
   }
   const uint32_t live_lo = __builtin_amdgcn_readfirstlane((uint32_t)live);
   const uint32_t live_hi = __builtin_amdgcn_readfirstlane((uint32_t)(live >> 32));
@@ -339,11 +341,35 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
     return tile;
   };
   int t_cur = pop(), t_nxt = pop();
+  if (row_dead) {
+    // Every key of the row is masked: the reference replaces all logits by the
+    // same -1e9, the softmax is exactly uniform and every query's output is the
+    // mean of V over the N keys (times its gate).  No attention to compute.
+    float* sMean = reinterpret_cast<float*>(&sK[0][0]);
+    const bf16_t* vrow = a.vt + (bh * D + v_d) * a.ldn;
+    float acc = 0.f;
+    for (int k0 = c8; k0 < N; k0 += 64) {  // rows of V^T hold ldn >= N keys, ldn a multiple of 8
+      float f[8];
+      unpack8(*reinterpret_cast<const u32x4*>(vrow + k0), f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc += k0 + e < N ? f[e] : 0.f;
+    }
+    acc += __shfl_xor(acc, 1);
+    acc += __shfl_xor(acc, 2);
+    acc += __shfl_xor(acc, 4);
+    if ((tid & 7) == 0) sMean[v_d] = acc;
+    lds_barrier();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[r] = sMean[8 * (r >> 2) + 4 * hh + (r & 3)];
+    l_run = (float)N;
+    t_cur = nkt;  // no tile loop
+  } else {
   gload_kv(t_cur * KT);
   gload_bias(rb, t_cur);
   sstore(0);
   gload_kv(t_nxt * KT);
   lds_barrier();
+  }
 
   for (int kt = 0; t_cur < nkt; ++kt) {
     const int buf = kt & 1;
