@@ -60,8 +60,20 @@ __global__ __launch_bounds__(256, 3) void trimul_prologue_kernel(TriMulArgs a) {
       *reinterpret_cast<u32x4*>(sW + (idx >> 4) * LDX + (idx & 15) * 8) = wr[i];
     }
   };
+  const float mk = tid < TM && t.valid(tid) ? (a.mask ? a.mask[t.pix(tid)] : 1.f) : 0.f;
+  if (!__syncthreads_or(mk != 0.f)) {
+    // Every position of the tile is masked (padding): a' and b' are zero there
+    // whatever the activations are.  Write the zeros and skip the rest.
+    const u32x4 z = {0, 0, 0, 0};
+    for (int idx = tid; idx < 2 * C * 16; idx += 256) {
+      const int op = idx >> 11, ch = (idx >> 4) & (C - 1), r = t.r0 + (idx & 15) * 8;
+      if (r < a.Np)
+        *reinterpret_cast<u32x4*>((op ? a.b_buf : a.a_buf) + ((int64_t)ch * a.N + t.o) * a.Np + r) = z;
+    }
+    return;
+  }
   wload(0);
-  if (tid < TM) sMask[tid] = (t.valid(tid) ? (a.mask ? a.mask[t.pix(tid)] : 1.f) : 0.f);
+  if (tid < TM) sMask[tid] = mk;
   load_ln_tile<TIO>(x, t, a.ln_in_w, a.ln_in_b, sX, tid);
   wstore();
   lds_barrier();
