@@ -333,8 +333,11 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   const uint32_t live_lo = __builtin_amdgcn_readfirstlane((uint32_t)live);
   const uint32_t live_hi = __builtin_amdgcn_readfirstlane((uint32_t)(live >> 32));
   uint64_t rest = (uint64_t)live_lo | ((uint64_t)live_hi << 32);
-  // next live tile, or nkt (a tile past the end: clamped loads, every key at -inf, never used) when none is left
+  // next live tile, or nkt (a tile past the end: clamped loads, every key at -inf, never used) when none is
+  // left; more than 64 tiles (N > 4096) are simply taken in order
+  int seq = 0;
   auto pop = [&]() {
+    if (nkt > 64) return seq < nkt ? seq++ : nkt;
     if (rest == 0ull) return nkt;
     const int tile = __builtin_ctzll(rest);
     rest &= rest - 1;
