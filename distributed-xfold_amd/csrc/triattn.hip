@@ -284,19 +284,20 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) dst[i] = *reinterpret_cast<const u32x4*>(p + (b_lane + 1024u * i));
   };
+  // A key at or past N gets -inf in its mask entry, so its probability is
+  // exactly zero whatever its K row and V column hold; the clamped loads gave
+  // them finite values (the last row / the first chunk), which is all it takes.
   auto sstore = [&](int buf) {
-    const u32x4 z = {0, 0, 0, 0};
-    *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + k_c * 8]) = key_ok ? rk : z;
+    *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + k_c * 8]) = rk;
     if (k_c < 2) {
       const uint32_t rmask = !key_ok ? BF16_NEG_INF : (rm == 0.f ? BF16_NEG_1E9 : 0u);
       u32x4 m = {k_c == 0 ? rmask : 0u, 0u, 0u, 0u};
       *reinterpret_cast<u32x4*>(&sK[buf][k_key * LDK + 32 + k_c * 8]) = m;
     }
     // rows of sVt are 8-byte aligned only: two 8-byte stores
-    const u32x4 v = col_ok ? rv : z;
     u32x2* pvs = reinterpret_cast<u32x2*>(&sVt[buf][v_d * LDV + c8]);
-    pvs[0] = u32x2{v.x, v.y};
-    pvs[1] = u32x2{v.z, v.w};
+    pvs[0] = u32x2{rv.x, rv.y};
+    pvs[1] = u32x2{rv.z, rv.w};
   };
 
   f32x16 o;
@@ -405,12 +406,17 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
     // registers are free again; like the K / V loads at the top of the loop it
     // is first looked at at the top of the next iteration.
     gload_bias(rb, t_nxt);
-    float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
+    // maximum of the lane's 32 scores as a tree of three-input maxima (16 instructions, depth 4)
+    float t3[11];
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int g = (u == 0 ? 1 : 0); g < 4; ++g)
-        mx = fmaxf(mx, fmaxf(fmaxf(s[u][4 * g], s[u][4 * g + 1]), fmaxf(s[u][4 * g + 2], s[u][4 * g + 3])));
+    for (int i = 0; i < 10; ++i) {
+      const int e = 3 * i;
+      t3[i] = fmaxf(fmaxf(s[e >> 4][e & 15], s[(e + 1) >> 4][(e + 1) & 15]), s[(e + 2) >> 4][(e + 2) & 15]);
+    }
+    t3[10] = fmaxf(s[1][14], s[1][15]);
+    const float t9a = fmaxf(fmaxf(t3[0], t3[1]), t3[2]), t9b = fmaxf(fmaxf(t3[3], t3[4]), t3[5]);
+    const float t9c = fmaxf(fmaxf(t3[6], t3[7]), t3[8]), t9d = fmaxf(t3[9], t3[10]);
+    float mx = fmaxf(fmaxf(fmaxf(t9a, t9b), t9c), t9d);
     mx = fmaxf(mx, half_swap(xaddr, mx));
     const float m_new = fmaxf(m_run, mx);
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
