@@ -36,46 +36,63 @@ constexpr int H = 4, D = 32;
 // (channel-major), + pair-bias heads
 // ============================================================================
 template <typename TIO>
-__global__ __launch_bounds__(256, 2) void triattn_proj_kernel(TriAttnProjArgs a) {
+__global__ __launch_bounds__(256, 3) void triattn_proj_kernel(TriAttnProjArgs a) {
+  // 34.8 KB + 17.4 KB of LDS and at most 168 registers: three workgroups per CU.  The kernel is a chain of
+  // short dependent phases (load, LayerNorm, MFMA, stage, store), so what it needs is company.
   __shared__ __attribute__((aligned(16))) bf16_t sX[TM * LDX];  // LN tile, then staging
-  __shared__ __attribute__((aligned(16))) bf16_t sW[TM * LDX];
+  __shared__ __attribute__((aligned(16))) bf16_t sW[64 * LDX];  // 64 weight rows at a time
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // (b, s) = (o, r): for the transposed operator a tile is a column segment
   const Tile t = make_tile(a.N, a.transpose != 0);
   const TIO* x = reinterpret_cast<const TIO*>(a.pair);
-  WChunkRegs wr;
-  wr.load(a.w_qkvg, tid);
+  // Step s = 2 * chunk + half: weight rows 64 half .. + 63 of chunk s / 2 (chunks q, k, v, g as packed in
+  // w_qkvg), four 16-byte pieces per thread; the 32 (padded) pair-bias rows ride in the same registers.
+  u32x4 wr[4];
+  auto wload = [&](int s) {
+    const bf16_t* base = a.w_qkvg + (int64_t)s * 64 * C;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + 256 * i;
+      wr[i] = *reinterpret_cast<const u32x4*>(base + (idx >> 4) * C + (idx & 15) * 8);
+    }
+  };
+  auto wload_bias = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int idx = tid + 256 * i;
+      wr[i] = *reinterpret_cast<const u32x4*>(a.w_bias + (idx >> 4) * C + (idx & 15) * 8);
+    }
+  };
+  auto wstore = [&](int n) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + 256 * i;
+      if (i < n) *reinterpret_cast<u32x4*>(sW + (idx >> 4) * LDX + (idx & 15) * 8) = wr[i];
+    }
+  };
+  wload(0);
   load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0);
-  wr.store(sW, tid);
+  wstore(4);
   lds_barrier();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
   lds_barrier();  // sX is free from here on: it becomes the staging tile
 
   const int64_t bh0 = (int64_t)t.o * H;  // (b * H + h) for h = 0
-  // chunk order q, k, v, g as packed in w_qkvg; v takes the channel-major route.
-  // Two 32-row weight tiles at a time keep the live accumulators at 32 registers.
-  // The chunk index is a compile-time constant of the body: with a run-time
-  // index the compiler evaluates the sigmoid for every chunk and selects.
-  auto do_chunk = [&](auto chunk_c) {
-    constexpr int chunk = decltype(chunk_c)::value;
+  // v takes the channel-major route.  The step index is a compile-time constant of the body: with a
+  // run-time index the compiler evaluates the sigmoid for every chunk and selects.
+  auto do_step = [&](auto step_c) {
+    constexpr int step = decltype(step_c)::value, chunk = step >> 1, pairt = step & 1;
     // The next weights are requested BEFORE this chunk's results are stored:
     // vector memory operations retire in order, so a load issued behind the
     // stores would make its consumer wait for the stores' round trip to HBM.
-    if (chunk < 3) wr.load(a.w_qkvg + (int64_t)(chunk + 1) * TM * C, tid);
-    else if (a.n_bias > 0) {
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int idx = tid + 256 * i;
-        wr.r[i] = *reinterpret_cast<const u32x4*>(a.w_bias + (idx >> 4) * C + (idx & 15) * 8);
-      }
-    }
-#pragma unroll
-    for (int pairt = 0; pairt < 2; ++pairt) {
+    if (step < 7) wload(step + 1);
+    else if (a.n_bias > 0) wload_bias();
+    {
       f32x16 acc[2];
       if (chunk == 2) {
         // v: D form, lane owns channel (lane & 31) of a tile, registers walk pixels
-        mfma_chunk<false, 2>(xf, sW + pairt * 64 * LDX, lane, acc);
+        mfma_chunk<false, 2>(xf, sW, lane, acc);
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt) {
           const int ch = (pairt * 2 + nt) * 32 + (lane & 31);
@@ -89,7 +106,7 @@ __global__ __launch_bounds__(256, 2) void triattn_proj_kernel(TriAttnProjArgs a)
           }
         }
       } else {
-        mfma_chunk<true, 2>(xf, sW + pairt * 64 * LDX, lane, acc);
+        mfma_chunk<true, 2>(xf, sW, lane, acc);
         const int px = wave * 32 + (lane & 31);
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
@@ -110,42 +127,43 @@ __global__ __launch_bounds__(256, 2) void triattn_proj_kernel(TriAttnProjArgs a)
       }
     }
     lds_barrier();  // staging visible; every wave is done with sW
-    if (chunk < 3) wr.store(sW, tid);
-    else if (a.n_bias > 0) {
+    if (step < 7) wstore(4);
+    else if (a.n_bias > 0) wstore(2);
+    if (pairt == 1) {
+      // both halves of the chunk are staged: 128 channels per position go out
+      if (chunk == 2) {
+        // Vt[(b*H + h)*32 + d][s]: per channel 128 consecutive positions
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int idx = tid + 256 * i;
-        *reinterpret_cast<u32x4*>(sW + (idx >> 4) * LDX + (idx & 15) * 8) = wr.r[i];
-      }
-    }
-    if (chunk == 2) {
-      // Vt[(b*H + h)*32 + d][s]: per channel 128 consecutive positions
+        for (int i = 0; i < 8; ++i) {
+          const int idx = tid + 256 * i, ch = idx >> 4, pc = idx & 15;
+          const int r = t.r0 + pc * 8;
+          if (r < a.ldn)
+            *reinterpret_cast<u32x4*>(a.vt + (bh0 * D + ch) * a.ldn + r) =
+                *reinterpret_cast<const u32x4*>(sX + ch * LDX + pc * 8);
+        }
+      } else {
+        bf16_t* plane = chunk == 0 ? a.q : (chunk == 1 ? a.k : a.g);
+        const int ck = tid & 15, prow = tid >> 4;
+        const int h = ck >> 2, part = ck & 3;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int idx = tid + 256 * i, ch = idx >> 4, pc = idx & 15;
-        const int r = t.r0 + pc * 8;
-        if (r < a.ldn)
-          *reinterpret_cast<u32x4*>(a.vt + (bh0 * D + ch) * a.ldn + r) =
-              *reinterpret_cast<const u32x4*>(sX + ch * LDX + pc * 8);
-      }
-    } else {
-      bf16_t* plane = chunk == 0 ? a.q : (chunk == 1 ? a.k : a.g);
-      const int ck = tid & 15, prow = tid >> 4;
-      const int h = ck >> 2, part = ck & 3;
-#pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const int p = it * 16 + prow;
-        if (t.valid(p))
-          *reinterpret_cast<u32x4*>(plane + ((bh0 + h) * a.N + t.r0 + p) * D + part * 8) =
-              *reinterpret_cast<const u32x4*>(sX + p * LDX + ck * 8);
+        for (int it = 0; it < 8; ++it) {
+          const int p = it * 16 + prow;
+          if (t.valid(p))
+            *reinterpret_cast<u32x4*>(plane + ((bh0 + h) * a.N + t.r0 + p) * D + part * 8) =
+                *reinterpret_cast<const u32x4*>(sX + p * LDX + ck * 8);
+        }
       }
     }
     lds_barrier();
   };
-  do_chunk(std::integral_constant<int, 0>{});
-  do_chunk(std::integral_constant<int, 1>{});
-  do_chunk(std::integral_constant<int, 2>{});
-  do_chunk(std::integral_constant<int, 3>{});
+  do_step(std::integral_constant<int, 0>{});
+  do_step(std::integral_constant<int, 1>{});
+  do_step(std::integral_constant<int, 2>{});
+  do_step(std::integral_constant<int, 3>{});
+  do_step(std::integral_constant<int, 4>{});
+  do_step(std::integral_constant<int, 5>{});
+  do_step(std::integral_constant<int, 6>{});
+  do_step(std::integral_constant<int, 7>{});
 
   // pair-bias heads (T form: lane = pixel, rows = heads): bias[h][q][k] with
   // (q, k) the pixel's own (row, col) in the un-transposed pair tensor
