@@ -412,31 +412,55 @@ __global__ __launch_bounds__(256, 2) void transition_kernel(TransitionArgs a) {
       f32x16 ab[2];
 #pragma unroll
       for (int r = 0; r < 16; ++r) ab[0][r] = ab[1][r] = 0.f;
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
         ab[0] = mfma32(lds_frag(sW1, LDX, nt * 32, ks * 16, lane), xf[ks], ab[0]);
         ab[1] = mfma32(lds_frag(sW1, LDX, 64 + nt * 32, ks * 16, lane), xf[ks], ab[1]);
       }
+      // fragment reads four ahead of the MFMAs that use them (left to itself the
+      // compiler reads each one right in front of its MFMA and waits for it)
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
+      for (int i = 0; i < 12; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // GEMM2: the W2 fragments of a step are requested before its silu, not
+      // in front of each MFMA
+      auto w2_frags = [&](int s, u32x4* wv) {
+        const int kbase = 32 * nt + 16 * s + 4 * (lane >> 5);
+#pragma unroll
+        for (int ot = 0; ot < 4; ++ot) {
+          const bf16_t* wp = sW2 + (ot * 32 + (lane & 31)) * LDW2 + kbase;
+          const u32x2 lo = *reinterpret_cast<const u32x2*>(wp);
+          const u32x2 hi = *reinterpret_cast<const u32x2*>(wp + 8);
+          wv[ot].x = lo.x; wv[ot].y = lo.y; wv[ot].z = hi.x; wv[ot].w = hi.y;
+        }
+      };
+      auto silu_frag = [&](int s) {
         float hv[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float av = ab[0][8 * s + e], bv = ab[1][8 * s + e];
           hv[e] = av * sigmoidf_(av) * bv;
         }
-        const bf16x8 hf = as_frag(pack8(hv));
-        const int kbase = 32 * nt + 16 * s + 4 * (lane >> 5);
+        return as_frag(pack8(hv));
+      };
+      u32x4 wv0[4], wv1[4];
+      w2_frags(0, wv0);
+      __builtin_amdgcn_sched_barrier(0);
+      const bf16x8 hf0 = silu_frag(0);
+      __builtin_amdgcn_sched_barrier(0);
+      w2_frags(1, wv1);
 #pragma unroll
-        for (int ot = 0; ot < 4; ++ot) {
-          const bf16_t* wp = sW2 + (ot * 32 + (lane & 31)) * LDW2 + kbase;
-          u32x4 wv;
-          const u32x2 lo = *reinterpret_cast<const u32x2*>(wp);
-          const u32x2 hi = *reinterpret_cast<const u32x2*>(wp + 8);
-          wv.x = lo.x; wv.y = lo.y; wv.z = hi.x; wv.w = hi.y;
-          out[ot] = mfma32(as_frag(wv), hf, out[ot]);
-        }
-      }
+      for (int ot = 0; ot < 4; ++ot) out[ot] = mfma32(as_frag(wv0[ot]), hf0, out[ot]);
+      const bf16x8 hf1 = silu_frag(1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ot = 0; ot < 4; ++ot) out[ot] = mfma32(as_frag(wv1[ot]), hf1, out[ot]);
     }
     lds_barrier();  // every wave is done with this slab
     if (hs + 1 < n_slabs) {

@@ -138,6 +138,7 @@ __device__ __forceinline__ void mfma_chunk(const bf16x8* xf, const bf16_t* sW, i
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[nt][r] = 0.f;
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
@@ -145,6 +146,16 @@ __device__ __forceinline__ void mfma_chunk(const bf16x8* xf, const bf16_t* sW, i
       const bf16x8 wf = lds_frag(sW, LDX, nt * 32, ks * 16, lane);
       acc[nt] = TFORM ? mfma32(wf, xf[ks], acc[nt]) : mfma32(xf[ks], wf, acc[nt]);
     }
+  // Weight fragments are read four ahead of the MFMAs that use them (left to
+  // itself the compiler reads each one right in front of its MFMA and waits).
+  __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+  for (int i = 0; i < 8 * NT - 4; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+  __builtin_amdgcn_sched_barrier(0);
 }
 
 // T-form accumulators (lane = pixel, 4 consecutive channels per register
