@@ -9,6 +9,9 @@ from .primitives import Transition
 from .diffusion_transformer import (AdaptiveLayerNorm, AdaLNZero, DiffusionTransition, SelfAttention,
                                     DiffusionTransformer, CrossAttention, DiffusionCrossAttTransformer)
 from .pairformer import PairformerBlock, PairformerStack
+from . import atom_layout
+from .atom_cross_attention import AtomCrossAttEncoder, AtomCrossAttDecoder, AtomCrossAttEncoderOutput
+from .diffusion_head import DiffusionHead, DiffusionSampler, FourierEmbeddings
 
 # names used by the reference for the same modules
 XSMMTriangleMultiplication = TriangleMultiplication
@@ -22,9 +25,15 @@ DistributeDiffusionTransformer = DiffusionTransformer
 DistrubuteCrossAttention = CrossAttention
 DistributeDiffusionCrossAttTransformer = DiffusionCrossAttTransformer
 DistributePairformerBlock = PairformerBlock
+DistributeAtomCrossAttEncoder = AtomCrossAttEncoder
+DistributeAtomCrossAttDecoder = AtomCrossAttDecoder
+DistributeDiffusionHead = DiffusionHead
+DistrubuteFourierEmbeddings = FourierEmbeddings
 
 __all__ = [
     "HipModule", "enable_hip", "check_mode", "in_check_mode", "TriangleMultiplication", "GridSelfAttention", "Transition",
     "AdaptiveLayerNorm", "AdaLNZero", "DiffusionTransition", "SelfAttention", "DiffusionTransformer",
     "CrossAttention", "DiffusionCrossAttTransformer", "PairformerBlock", "PairformerStack",
+    "atom_layout", "AtomCrossAttEncoder", "AtomCrossAttDecoder", "AtomCrossAttEncoderOutput", "DiffusionHead",
+    "DiffusionSampler", "FourierEmbeddings",
 ]

@@ -234,14 +234,27 @@ class DiffusionTransformer(HipModule):
                     w_ss=bf16(torch.cat(w_ss, dim=0)), b_ss=f32(torch.cat(b_ss)),
                     w_gate=bf16(torch.cat(w_gate, dim=0)), b_gate=f32(torch.cat(b_gate)))
 
+    def pair_logits(self, pair_cond: torch.Tensor):
+        """The pair logits of every super-block, [num_super_blocks] x [b, h, N, N].
+        They depend on pair_cond only: a caller that evaluates the transformer
+        many times on one pair_cond (the diffusion sampler) computes them once
+        and hands them to `forward(..., pair_logits=...)`."""
+        p = self.packed()
+        pair_cond = pair_cond.contiguous()
+        n_out = self.super_block_size * self.num_head
+        out = []
+        for sb in range(self.num_super_blocks):
+            logits = ops.pair_logits(pair_cond, p["ln_w"], None, p["w_logits"][sb], n_out)
+            out.append(logits.view(self.super_block_size, self.num_head, *logits.shape[1:]))  # (b h) n s -> b h n s
+        return out
+
     def forward(self, act: torch.Tensor, mask: torch.Tensor, single_cond: torch.Tensor,
-                pair_cond: torch.Tensor) -> torch.Tensor:
+                pair_cond: torch.Tensor, pair_logits=None) -> torch.Tensor:
         """act [B, N, c_act] (updated in place, as the reference's `act +=`),
         mask [N], single_cond [N, c_single_cond], pair_cond [N, N, c_pair_cond]."""
         if in_check_mode():
             return check.diffusion_transformer(self, act, mask, single_cond, pair_cond)
         p = self.packed()
-        pair_cond = pair_cond.contiguous()
         if not act.is_contiguous():
             raise ValueError("act must be contiguous (it is updated in place)")
         n_out = self.super_block_size * self.num_head
@@ -254,8 +267,11 @@ class DiffusionTransformer(HipModule):
                               sigmoid=True)
         gate_all = gate_all.view(rows, n_mod, c).permute(1, 0, 2).contiguous()   # [module][row][c]
         for sb in range(self.num_super_blocks):
-            logits = ops.pair_logits(pair_cond, p["ln_w"], None, p["w_logits"][sb], n_out)
-            logits = logits.view(self.super_block_size, self.num_head, *logits.shape[1:])  # (b h) n s -> b h n s
+            if pair_logits is not None:
+                logits = pair_logits[sb]
+            else:
+                logits = ops.pair_logits(pair_cond.contiguous(), p["ln_w"], None, p["w_logits"][sb], n_out)
+                logits = logits.view(self.super_block_size, self.num_head, *logits.shape[1:])  # (b h) n s -> b h n s
             for j in range(self.super_block_size):
                 i = sb * self.super_block_size + j
                 self.self_attention[i].run(act, mask, logits[j], single_cond, residual=True,
@@ -387,14 +403,14 @@ class DiffusionCrossAttTransformer(HipModule):
         keys = flat[..., idx.reshape(-1), :].reshape(lead + tuple(idx.shape) + (c,))
         return (keys * gmask.to(keys.dtype)[..., None]).contiguous()
 
-    def forward(self, queries_act, queries_mask, queries_to_keys, keys_mask, queries_single_cond,
-                keys_single_cond, pair_cond):
-        if in_check_mode():
-            return check.cross_att_transformer(self, queries_act, queries_mask, queries_to_keys, keys_mask,
-                                               queries_single_cond, keys_single_cond, pair_cond)
+    def conditioning(self, queries_single_cond, keys_single_cond, pair_cond):
+        """Everything the blocks take from the conditioning inputs: the pair
+        logits of every block, the adaptive LayerNorm scale | shift of queries
+        and keys and the AdaLN-Zero gates.  None of it depends on queries_act,
+        so a caller that runs the transformer many times on one conditioning
+        (the diffusion sampler) computes it once and passes it as
+        `forward(..., cond=...)`."""
         p = self.packed()
-        if not queries_act.is_contiguous():
-            raise ValueError("queries_act must be contiguous (it is updated in place)")
         pair_act = ops.layer_norm(pair_cond.contiguous(), p["ln_w"])
         logits = ops.linear(pair_act, p["w"], out_dtype=torch.float32)           # [S, Q, K, (b h)]
         s, q, k, _ = logits.shape
@@ -409,6 +425,18 @@ class DiffusionCrossAttTransformer(HipModule):
         ss_k = ss_k.view(rk, self.num_blocks, 2 * c)
         gate = ops.linear(cq.to(torch.bfloat16), p["w_gate"], bias=p["b_gate"], out_dtype=torch.float32, sigmoid=True)
         gate = gate.view(rq, 2 * self.num_blocks, c).permute(1, 0, 2).contiguous()   # [module][row][c]
+        return logits, ss_q, ss_k, gate
+
+    def forward(self, queries_act, queries_mask, queries_to_keys, keys_mask, queries_single_cond,
+                keys_single_cond, pair_cond, cond=None):
+        if in_check_mode():
+            return check.cross_att_transformer(self, queries_act, queries_mask, queries_to_keys, keys_mask,
+                                               queries_single_cond, keys_single_cond, pair_cond)
+        if not queries_act.is_contiguous():
+            raise ValueError("queries_act must be contiguous (it is updated in place)")
+        if cond is None:
+            cond = self.conditioning(queries_single_cond, keys_single_cond, pair_cond)
+        logits, ss_q, ss_k, gate = cond
         for blk in range(self.num_blocks):
             keys_act = self._gather(queries_to_keys, queries_act)
             self.cross_attention[blk].run(queries_act, keys_act, queries_mask, keys_mask, logits[blk],
