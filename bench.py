@@ -114,6 +114,45 @@ def cpu_baseline(n_metric, budget_s=25.0):
     }
 
 
+def diffusion_step(pkg, n, dev, samples=5, iters=20):
+    """One denoising evaluation of the diffusion head (atom cross-attention
+    encoder, 24-block diffusion transformer, decoder) on `samples` samples of an
+    n-token synthetic batch with 24 atom slots per token, bf16 activations,
+    random-init weights; the per-batch conditioning is computed once, as the
+    sampler does, and timed separately."""
+    import torch
+    from oracle import af3_head_oracle as H     # parameter generator only
+    g = torch.Generator().manual_seed(1)
+    head = pkg.nn.DiffusionHead()
+    head.load_state_dict(H.make_diffusion_head_params(g))
+    head = head.to(dev)
+    head.load_hip_params()
+    batch = pkg.nn.atom_layout.synthetic_batch(n, g, n_padding_tokens=n // 10).to(dev)
+    emb = {"single": torch.randn(n, 384, generator=g).to(dev), "pair": torch.randn(n, n, 128, generator=g).to(dev),
+           "target_feat": torch.randn(n, 447, generator=g).to(dev)}
+    sampler = pkg.nn.DiffusionSampler(head, num_samples=samples)
+    _, t_hat, _ = sampler.schedule(dev)
+
+    def setup():
+        sc, pc = head.pre_conditioning(batch, emb, t_hat, True)
+        return sc, pc, head.prepare(batch, emb, pc)
+    setup()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    sc, pc, state = setup()
+    torch.cuda.synchronize()
+    setup_ms = (time.perf_counter() - t0) * 1e3
+    pos = torch.randn(samples, n, 24, 3, generator=g).to(dev) * float(t_hat[100])
+    ms = gpu_time_ms(lambda: head(pos, t_hat[100], batch, emb, sc[100], pc, state=state), iters, warm_ms=40.0)
+    ms_ref = gpu_time_ms(lambda: head(pos, t_hat[100], batch, emb, sc[100], pc), 5)
+    return {"workload": f"one denoising evaluation, {samples} samples, N_token={n}, 24 atom slots per token, "
+                        "24 transformer blocks, 3+3 atom-attention blocks, bf16 activations",
+            "ms_per_evaluation": round(ms, 3),
+            "ms_per_evaluation_conditioning_recomputed": round(ms_ref, 3),
+            "per_batch_setup_ms": round(setup_ms, 1),
+            "sampling_200_steps_s": round((setup_ms + 200 * ms) / 1e3, 3)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -122,6 +161,7 @@ def main():
     ap.add_argument("--n-token", type=int, default=768)
     ap.add_argument("--io", choices=["bf16", "f32"], default="bf16", help="dtype of the residual stream")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-diffusion", action="store_true", help="skip the diffusion-head timing")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain elementwise kernel that reads and writes 256 MiB, three times: the "
                          "reference against which the FETCH_SIZE / WRITE_SIZE counters of a profiler run are scaled")
@@ -212,6 +252,11 @@ def main():
                    for k, v in kernels.items() if k != dom},
     }
 
+    # ---- the diffusion head that calls the diffusion transformer / atom cross-attention (informational) ----
+    diffusion = None
+    if not args.no_diffusion:
+        diffusion = diffusion_step(pkg, n, dev)
+
     if args.calibrate:
         cx = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device=dev)   # 256 MiB in, 256 MiB out
         cy = torch.empty_like(cx)
@@ -234,6 +279,8 @@ def main():
         "tflops_per_op": {k: round(v, 2) for k, v in tflops_per_op.items()},
         "roofline": roofline,
     }
+    if diffusion is not None:
+        out["diffusion_head"] = diffusion
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(n)
     print(json.dumps(out))

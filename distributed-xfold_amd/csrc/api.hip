@@ -302,6 +302,65 @@ int af3_batch_diffusion_cross_attention_forward(
   return launch_flash_attention(f, s);
 }
 
+size_t af3_gathered_cross_attention_workspace_bytes(int64_t batch, int64_t sq, int64_t samples, int64_t n_atoms,
+                                                    int channels) {
+  if (batch <= 0 || sq <= 0 || samples <= 0 || n_atoms <= 0 || channels <= 0) return 0;
+  return align_up((size_t)batch * sq * 2 * channels * sizeof(bf16_t), 256) +
+         align_up((size_t)samples * n_atoms * 2 * channels * sizeof(bf16_t), 256);
+}
+
+int af3_gathered_cross_attention_forward(
+    const uint16_t* q_data, const uint16_t* atom_data, const int32_t* key_rows,
+    const float* pair_logits, const float* mask_q, const float* mask_k, int64_t bias_batches,
+    const uint16_t* w_qg, const uint16_t* w_kv, const float* query_b, int num_head,
+    void* out, int out_dtype, int64_t batch, int64_t sq, int64_t sk, int64_t samples, int64_t n_atoms, int channels,
+    void* workspace, size_t workspace_bytes, af3_stream_t stream) {
+  if (!q_data || !atom_data || !key_rows || !w_qg || !w_kv || !out) return AF3_ERR_BAD_ARG;
+  if (bad_dtype(out_dtype) || batch <= 0 || sq <= 0 || sk <= 0 || samples <= 0 || n_atoms <= 0 || channels <= 0 ||
+      (channels & 7) || num_head <= 0 || channels % num_head)
+    return AF3_ERR_BAD_ARG;
+  if ((mask_q == nullptr) != (mask_k == nullptr)) return AF3_ERR_BAD_ARG;
+  if (bias_batches <= 0 || batch != samples * bias_batches) return AF3_ERR_BAD_ARG;
+  if (batch * sq > 0x7fffffff || samples * n_atoms > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  const int d = channels / num_head;
+  if (d != 24 && d != 32 && d != 48) return AF3_ERR_UNSUPPORTED;
+  Carver ws(workspace, workspace_bytes);
+  bf16_t* qg = ws.take<bf16_t>((size_t)batch * sq * 2 * channels);
+  bf16_t* kv = ws.take<bf16_t>((size_t)samples * n_atoms * 2 * channels);
+  if (!ws.ok) return AF3_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+
+  GemmArgs g;
+  g.A = q_data; g.B = w_qg; g.C = qg;
+  g.M = (int)(batch * sq); g.N = 2 * channels; g.K = channels;
+  g.lda = channels; g.ldb = channels; g.ldc = 2 * channels;
+  g.epi = EPI_SEGMENTED; g.seg_len = channels;
+  g.seg_ops = SEG_BIAS_SCALE | (SEG_SIGMOID << 4);
+  g.alpha = 1.0f / sqrtf((float)d);
+  g.bias = query_b;
+  int rc = launch_gemm_nt(g, s);
+  if (rc) return rc;
+  GemmArgs g2;
+  g2.A = atom_data; g2.B = w_kv; g2.C = kv;
+  g2.M = (int)(samples * n_atoms); g2.N = 2 * channels; g2.K = channels;
+  g2.lda = channels; g2.ldb = channels; g2.ldc = 2 * channels;
+  rc = launch_gemm_nt(g2, s);
+  if (rc) return rc;
+
+  FlashArgs f;
+  f.q = qg; f.g = qg + channels; f.k = kv; f.v = kv + channels;
+  f.q_ss = f.g_ss = f.k_ss = f.v_ss = 2 * channels;
+  f.q_sb = f.g_sb = sq * 2 * channels;
+  f.k_sb = f.v_sb = n_atoms * 2 * channels;   // one K / V table per sample
+  f.key_rows = key_rows;
+  f.out = out; f.out_f32 = out_dtype == AF3_F32; f.o_ss = channels; f.o_sb = sq * channels;
+  f.B = (int)batch; f.H = num_head; f.Sq = (int)sq; f.Sk = (int)sk; f.d = d;
+  f.bias = pair_logits; f.bias_sb = (int64_t)num_head * sq * sk; f.bias_sh = sq * sk; f.bias_sq = sk;
+  f.qpad = mask_q; f.kpad = mask_k; f.qp_sb = sq; f.kp_sb = sk;
+  f.bias_mod = (int)bias_batches;
+  return launch_flash_attention(f, s);
+}
+
 // ------------------------------------------------------------------ pair logits
 int af3_pair_logits_forward(
     const void* pair, int io_dtype, const float* norm_weight, const float* norm_bias,

@@ -64,8 +64,12 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
   }
   const bf16x8 onesf = as_frag(u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
 
-  const bf16_t* kg = a.k + (int64_t)b * a.k_sb + h * d;
-  const bf16_t* vg = a.v + (int64_t)b * a.v_sb + h * d;
+  // With key_rows, K / V are tables of rows shared by bias_mod consecutive batch
+  // entries (one table per sample) and the key rows of this batch entry are
+  // looked up in key_rows; a negative entry is a key whose K and V rows are zero.
+  const int64_t kv_b = a.key_rows ? b / a.bias_mod : b;
+  const bf16_t* kg = a.k + kv_b * a.k_sb + h * d;
+  const bf16_t* vg = a.v + kv_b * a.v_sb + h * d;
   const int dch = d / 8;  // 16-byte chunks per real key row
 
   // Tile loaders (global -> registers -> LDS).  Every load is unconditional,
@@ -78,8 +82,10 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
   constexpr int KCH = KT * (KD / 8);
   constexpr int NLD = (KCH + NT - 1) / NT;
   u32x4 rk[NLD], rv[NLD];
+  bool k_row_ok[NLD], v_row_ok[NLD];
   float rkm = 1.f, rkp = 1.f;  // key mask / key padding flag of key tid (threads 0..63)
   const int bb = a.bias_mod > 0 ? b % a.bias_mod : b;  // batch index of bias / padding masks
+  const int* krows = a.key_rows ? a.key_rows + (int64_t)bb * a.Sk : nullptr;
   const float* kmask = a.key_mask ? a.key_mask + (int64_t)b * a.km_sb : nullptr;
   const float* kpad = a.kpad ? a.kpad + (int64_t)bb * a.kp_sb : nullptr;
   int k0_loaded = 0;
@@ -89,9 +95,13 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
     for (int i = 0; i < NLD; ++i) {
       const int idx = min(tid + i * NT, KCH - 1);
       const int key = min(k0 + idx / (KD / 8), a.Sk - 1), c = idx % (KD / 8);
-      rk[i] = *reinterpret_cast<const u32x4*>(kg + (int64_t)key * a.k_ss + (c < dch ? c : 0) * 8);
+      const int krow = krows ? krows[key] : key;
+      k_row_ok[i] = krow >= 0;
+      rk[i] = *reinterpret_cast<const u32x4*>(kg + (int64_t)max(krow, 0) * a.k_ss + (c < dch ? c : 0) * 8);
       const int vkey = min(k0 + idx % KT, a.Sk - 1), vc = idx / KT;
-      rv[i] = *reinterpret_cast<const u32x4*>(vg + (int64_t)vkey * a.v_ss + (vc < dch ? vc : 0) * 8);
+      const int vrow = krows ? krows[vkey] : vkey;
+      v_row_ok[i] = vrow >= 0;
+      rv[i] = *reinterpret_cast<const u32x4*>(vg + (int64_t)max(vrow, 0) * a.v_ss + (vc < dch ? vc : 0) * 8);
     }
     if (tid < KT) {
       const int key = min(k0 + tid, a.Sk - 1);
@@ -106,10 +116,11 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
       const int idx = tid + i * NT;
       if (idx >= KCH) continue;
       const int key = idx / (KD / 8), c = idx % (KD / 8);
-      *reinterpret_cast<u32x4*>(&sK[buf][key * LDK + c * 8]) = (k0_loaded + key < a.Sk && c < dch) ? rk[i] : z;
+      *reinterpret_cast<u32x4*>(&sK[buf][key * LDK + c * 8]) =
+          (k0_loaded + key < a.Sk && c < dch && k_row_ok[i]) ? rk[i] : z;
       const int vkey = idx % KT, vc = idx / KT;
       if (vc * 8 < DVT * 32) {
-        const bool ok = k0_loaded + vkey < a.Sk && vc < dch;
+        const bool ok = k0_loaded + vkey < a.Sk && vc < dch && v_row_ok[i];
         const uint32_t w4[4] = {rv[i].x, rv[i].y, rv[i].z, rv[i].w};
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -320,6 +331,7 @@ int launch_flash_attention(const FlashArgs& a, hipStream_t stream) {
       ((uintptr_t)a.out & 15))
     return AF3_ERR_BAD_ARG;
   if ((a.qpad == nullptr) != (a.kpad == nullptr)) return AF3_ERR_BAD_ARG;
+  if (a.key_rows && (a.bias_mod <= 0 || a.B % a.bias_mod)) return AF3_ERR_BAD_ARG;
   if (a.d == 48) return launch_nw<3, 2>(a, stream);
   return launch_nw<2, 1>(a, stream);
 }

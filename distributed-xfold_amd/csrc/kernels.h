@@ -122,6 +122,10 @@ struct FlashArgs {
   const float *qpad = nullptr, *kpad = nullptr;  // [B][Sq], [B][Sk]: +1e9 where both are 0
   int64_t qp_sb = 0, kp_sb = 0;
   int bias_mod = 0;  // > 0: bias, qpad and kpad are indexed by batch % bias_mod
+  // Gathered keys: key s of batch entry b is row key_rows[(b % bias_mod) * Sk + s]
+  // of the K / V table of sample b / bias_mod (k_sb / v_sb: table stride); a
+  // negative row is a key with zero K and V.  Null: key s is row s of batch b.
+  const int* key_rows = nullptr;
 };
 int launch_flash_attention(const FlashArgs& a, hipStream_t stream);
 

@@ -30,6 +30,10 @@ SIGNATURES = {
     "af3_batch_diffusion_cross_attention_workspace_bytes": (_sz, [_i64, _i64, _i64, _i]),
     "af3_batch_diffusion_cross_attention_forward": (
         _i, [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i, _vp, _i, _i64, _i64, _i64, _i, _vp, _sz, _vp]),
+    "af3_gathered_cross_attention_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i]),
+    "af3_gathered_cross_attention_forward": (
+        _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i, _vp, _i, _i64, _i64, _i64, _i64, _i64, _i,
+             _vp, _sz, _vp]),
     "af3_pair_logits_forward": (_i, [_vp, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp]),
     "af3_layer_norm_forward": (_i, [_vp, _i, _vp, _i64, _i, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "af3_linear_forward": (

@@ -142,6 +142,7 @@ class AtomCrossAttEncoder(HipModule):
         pair_act = pair_act + _lin(1.0 / (1 + (d * d).sum(-1, keepdim=True)), self.embed_pair_distances)
         return act, pair_act
 
+    @torch.no_grad()
     def conditioning(self, batch, trunk_single_cond, trunk_pair_cond) -> EncoderConditioning:
         """The position-independent part of `forward` (:168-179, 205-311)."""
         p = self.packed()
@@ -182,9 +183,11 @@ class AtomCrossAttEncoder(HipModule):
         q_cond, k_cond = q_cond.contiguous(), k_cond.contiguous()
         tcond = None
         if not in_check_mode():
-            tcond = self.atom_transformer_encoder.conditioning(q_cond, k_cond, pair_act)
+            tcond = self.atom_transformer_encoder.conditioning(q_cond, k_cond, pair_act,
+                                                               keys_are_query_atoms=aca.queries_to_keys)
         return EncoderConditioning(q_mask, q_cond, k_mask, k_cond, pair_act, tcond)
 
+    @torch.no_grad()
     def forward(self, batch, token_atoms_act: Optional[torch.Tensor], trunk_single_cond: Optional[torch.Tensor],
                 trunk_pair_cond: Optional[torch.Tensor], conditioning: Optional[EncoderConditioning] = None,
                 act_dtype: torch.dtype = torch.bfloat16) -> AtomCrossAttEncoderOutput:
@@ -245,14 +248,17 @@ class AtomCrossAttDecoder(HipModule):
         return dict(w_bcast=bf16(self.project_token_features_for_broadcast.weight),
                     ln_w=f32(self.atom_features_layer_norm.weight))
 
-    def conditioning(self, enc):
+    @torch.no_grad()
+    def conditioning(self, enc, queries_to_keys=None):
         """The decoder transformer's conditioning projections for the
-        encoder's (position-independent) conditioning tensors."""
+        encoder's (position-independent) conditioning tensors; `queries_to_keys`
+        (batch.atom_cross_att.queries_to_keys) selects the per-atom key path."""
         if in_check_mode():
             return None
         return self.atom_transformer_decoder.conditioning(enc.queries_single_cond, enc.keys_single_cond,
-                                                          enc.pair_cond)
+                                                          enc.pair_cond, keys_are_query_atoms=queries_to_keys)
 
+    @torch.no_grad()
     def forward(self, batch, token_act: torch.Tensor, enc: AtomCrossAttEncoderOutput,
                 transformer_cond=None) -> torch.Tensor:
         """:355-414 -> position update [(samples), N, A, 3], fp32."""

@@ -166,6 +166,7 @@ class DiffusionHead(HipModule):
         y = F.pad(y, (0, (-x.shape[-1]) % 8)).to(torch.bfloat16)
         return ops.linear(y, w_padded, out_dtype=torch.float32)
 
+    @torch.no_grad()
     def pre_conditioning(self, batch, embeddings, noise_level: torch.Tensor, use_conditioning):
         """:96-169 -> (single_cond [T, N, 384] fp32, pair_cond [N, N, 128] fp32)
         for the noise levels [T] of all steps."""
@@ -201,14 +202,16 @@ class DiffusionHead(HipModule):
             return x + mod(x)
         return mod.run(x, None, residual=True)
 
+    @torch.no_grad()
     def prepare(self, batch, embeddings, trunk_pair_cond: torch.Tensor) -> HeadState:
         """Everything `forward` needs that depends neither on the positions nor
         on the noise level."""
         enc = self.atom_cross_att_encoder.conditioning(batch, embeddings["single"], trunk_pair_cond)
-        dec = self.atom_cross_att_decoder.conditioning(enc)
+        dec = self.atom_cross_att_decoder.conditioning(enc, batch.atom_cross_att.queries_to_keys)
         logits = None if in_check_mode() else self.transformer.pair_logits(trunk_pair_cond)
         return HeadState(enc, dec, logits)
 
+    @torch.no_grad()
     def forward(self, positions_noisy: torch.Tensor, noise_level: torch.Tensor, batch, embeddings,
                 trunk_single_cond: torch.Tensor, trunk_pair_cond: torch.Tensor,
                 state: Optional[HeadState] = None, act_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:

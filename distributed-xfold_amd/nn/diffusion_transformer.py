@@ -332,6 +332,27 @@ class CrossAttention(HipModule):
         return self.adaptive_zero_init.run(avg, single_cond_q, x_q.dtype, residual=x_q if residual else None,
                                            gate=gate)
 
+    def run_gathered(self, x_q, key_rows, mask_q, mask_k, pair_logits, single_cond_q, cond):
+        """`run(..., residual=True)` for keys that are query atoms: key k of
+        subset s is atom key_rows[s, k] of the flattened (subset, query) axis of
+        x_q (negative: a masked slot, whose gathered activation and conditioning
+        are zero, hence K = V = 0).  The keys' adaptive LayerNorm and K / V
+        projection then run once per atom, not once per (subset, key), and no
+        key tensor is gathered: cond = (scale_shift_q, scale_shift_k of the
+        ATOMS [S * Q, 2c], gate)."""
+        p = self.packed()
+        n_sub, n_q, c = x_q.shape[-3:]
+        ss_q, ss_k_atoms, gate = cond
+        xq = self.q_adaptive_layernorm(x_q, single_cond_q, scale_shift=ss_q)
+        xk = self.k_adaptive_layernorm(x_q, single_cond_q, scale_shift=ss_k_atoms)
+        pl = None
+        if pair_logits is not None:
+            pl = pair_logits.reshape(-1, self.num_head, n_q, key_rows.shape[-1]).to(torch.float32).contiguous()
+        avg = ops.gathered_cross_attention(
+            xq.reshape(-1, n_q, c), xk.reshape(-1, n_sub * n_q, c), key_rows, pl, mask_q.reshape(-1, n_q),
+            mask_k.reshape(-1, key_rows.shape[-1]), p["w_qg"], p["w_kv"], p["q_b"], self.num_head)
+        return self.adaptive_zero_init.run(avg.reshape(x_q.shape), single_cond_q, x_q.dtype, residual=x_q, gate=gate)
+
     def forward(self, x_q, x_k, mask_q, mask_k, pair_logits=None, single_cond_q=None, single_cond_k=None):
         """x_q [(B,) S, Q, c], x_k [(B,) S, K, c], masks [(1,) S, Q] / [(1,) S, K],
         pair_logits [(1,) S, H, Q, K], conditioning [(1,) S, Q|K, c]."""
@@ -392,25 +413,43 @@ class DiffusionCrossAttTransformer(HipModule):
                     w_gate=bf16(torch.cat(wg, dim=0)), b_gate=f32(torch.cat(bg)))
 
     @staticmethod
-    def _gather(queries_to_keys, queries_act):
+    def _gather_info(queries_to_keys):
         if hasattr(queries_to_keys, "gather_idxs"):
-            idx, gmask = queries_to_keys.gather_idxs, queries_to_keys.gather_mask
-        else:
-            idx, gmask = queries_to_keys
+            return queries_to_keys.gather_idxs, queries_to_keys.gather_mask
+        return queries_to_keys
+
+    @staticmethod
+    def _gather(queries_to_keys, queries_act):
+        idx, gmask = DiffusionCrossAttTransformer._gather_info(queries_to_keys)
         lead = queries_act.shape[:-3]
         s, q, c = queries_act.shape[-3:]
         flat = queries_act.reshape(lead + (s * q, c))
         keys = flat[..., idx.reshape(-1), :].reshape(lead + tuple(idx.shape) + (c,))
         return (keys * gmask.to(keys.dtype)[..., None]).contiguous()
 
-    def conditioning(self, queries_single_cond, keys_single_cond, pair_cond):
+    def conditioning(self, queries_single_cond, keys_single_cond, pair_cond, keys_are_query_atoms=None):
         """Everything the blocks take from the conditioning inputs: the pair
         logits of every block, the adaptive LayerNorm scale | shift of queries
         and keys and the AdaLN-Zero gates.  None of it depends on queries_act,
         so a caller that runs the transformer many times on one conditioning
         (the diffusion sampler) computes it once and passes it as
-        `forward(..., cond=...)`."""
+        `forward(..., cond=...)`.
+
+        `keys_are_query_atoms`: the `queries_to_keys` gather, given by a caller
+        whose keys_single_cond IS that gather of queries_single_cond (the atom
+        cross-attention encoder and decoder build it so,
+        nn/d_atom_cross_attention.py:205-209).  The key side is then computed per
+        atom (see CrossAttention.run_gathered) instead of per (subset, key)."""
         p = self.packed()
+        key_rows = None
+        if keys_are_query_atoms is not None:
+            idx, gmask = self._gather_info(keys_are_query_atoms)
+            n_atoms = queries_single_cond.shape[-3] * queries_single_cond.shape[-2]
+            if int(idx.min()) < 0 or int(idx.max()) >= n_atoms:
+                raise ValueError("queries_to_keys indexes beyond the query atoms")
+            key_rows = torch.where(gmask.bool(), idx, torch.full_like(idx, -1)).to(torch.int32).contiguous()
+            key_rows._af3_checked_rows = n_atoms
+            keys_single_cond = queries_single_cond          # per atom
         pair_act = ops.layer_norm(pair_cond.contiguous(), p["ln_w"])
         logits = ops.linear(pair_act, p["w"], out_dtype=torch.float32)           # [S, Q, K, (b h)]
         s, q, k, _ = logits.shape
@@ -425,7 +464,7 @@ class DiffusionCrossAttTransformer(HipModule):
         ss_k = ss_k.view(rk, self.num_blocks, 2 * c)
         gate = ops.linear(cq.to(torch.bfloat16), p["w_gate"], bias=p["b_gate"], out_dtype=torch.float32, sigmoid=True)
         gate = gate.view(rq, 2 * self.num_blocks, c).permute(1, 0, 2).contiguous()   # [module][row][c]
-        return logits, ss_q, ss_k, gate
+        return logits, ss_q, ss_k, gate, key_rows
 
     def forward(self, queries_act, queries_mask, queries_to_keys, keys_mask, queries_single_cond,
                 keys_single_cond, pair_cond, cond=None):
@@ -436,12 +475,17 @@ class DiffusionCrossAttTransformer(HipModule):
             raise ValueError("queries_act must be contiguous (it is updated in place)")
         if cond is None:
             cond = self.conditioning(queries_single_cond, keys_single_cond, pair_cond)
-        logits, ss_q, ss_k, gate = cond
+        logits, ss_q, ss_k, gate, key_rows = cond
         for blk in range(self.num_blocks):
-            keys_act = self._gather(queries_to_keys, queries_act)
-            self.cross_attention[blk].run(queries_act, keys_act, queries_mask, keys_mask, logits[blk],
-                                          queries_single_cond, keys_single_cond, residual=True,
-                                          cond=(ss_q[:, 2 * blk], ss_k[:, blk], gate[2 * blk]))
+            if key_rows is not None:
+                self.cross_attention[blk].run_gathered(queries_act, key_rows, queries_mask, keys_mask, logits[blk],
+                                                       queries_single_cond,
+                                                       cond=(ss_q[:, 2 * blk], ss_k[:, blk], gate[2 * blk]))
+            else:
+                keys_act = self._gather(queries_to_keys, queries_act)
+                self.cross_attention[blk].run(queries_act, keys_act, queries_mask, keys_mask, logits[blk],
+                                              queries_single_cond, keys_single_cond, residual=True,
+                                              cond=(ss_q[:, 2 * blk], ss_k[:, blk], gate[2 * blk]))
             self.transition_block[blk].run(queries_act, queries_single_cond, residual=True,
                                            cond=(ss_q[:, 2 * blk + 1], gate[2 * blk + 1]))
         return queries_act

@@ -233,6 +233,49 @@ def batch_diffusion_cross_attention(q_data, m_data, pair_logits, mask_q, mask_k,
     return out
 
 
+def gathered_cross_attention(q_data, atom_data, key_rows, pair_logits, mask_q, mask_k, w_qg, w_kv, query_b,
+                             num_head, out_dtype=torch.bfloat16):
+    """The cross-attention above with the key windows looked up inside the
+    kernel (af3_gathered_cross_attention_forward).  q_data [samples * Bb, Sq, C]
+    bf16; atom_data [samples, n_atoms, C] bf16; key_rows [Bb, Sk] int32 (row of
+    atom_data, negative for a masked slot); pair_logits [Bb, H, Sq, Sk] fp32 or
+    None; masks [Bb, Sq] / [Bb, Sk] or None.  Returns [samples * Bb, Sq, H, C/H]."""
+    lib = _L.load()
+    _gpu(q_data, "q_data", torch.bfloat16)
+    _gpu(atom_data, "atom_data", torch.bfloat16)
+    _gpu(key_rows, "key_rows", torch.int32)
+    b, sq, c = q_data.shape
+    if atom_data.dim() != 3 or atom_data.shape[2] != c:
+        raise ValueError("atom_data: expected [samples, n_atoms, C]")
+    samples, n_atoms = atom_data.shape[:2]
+    bb, sk = key_rows.shape
+    if b != samples * bb:
+        raise ValueError("q_data: batch must be samples * windows")
+    if getattr(key_rows, "_af3_checked_rows", None) != n_atoms:
+        # (one device round trip; the tensor is marked so that it is paid once)
+        if int(key_rows.max()) >= n_atoms:
+            raise ValueError("key_rows: row index beyond atom_data")
+        key_rows._af3_checked_rows = n_atoms
+    if pair_logits is not None:
+        _gpu(pair_logits, "pair_logits", torch.float32, (bb, num_head, sq, sk))
+    mq = mk = None
+    if mask_q is not None:
+        mq = _mask_f32(mask_q, (bb, sq), "mask_q")
+        mk = _mask_f32(mask_k, (bb, sk), "mask_k")
+    _gpu(w_qg, "w_qg", torch.bfloat16, (2 * c, c))
+    _gpu(w_kv, "w_kv", torch.bfloat16, (2 * c, c))
+    if query_b is not None:
+        _gpu(query_b, "query_b", torch.float32, (c,))
+    out = torch.empty((b, sq, num_head, c // num_head), dtype=out_dtype, device=q_data.device)
+    ws = _ws(lib.af3_gathered_cross_attention_workspace_bytes(b, sq, samples, n_atoms, c), q_data.device)
+    rc = lib.af3_gathered_cross_attention_forward(
+        _p(q_data), _p(atom_data), _p(key_rows), _p(pair_logits), _p(mq), _p(mk), bb, _p(w_qg), _p(w_kv),
+        _p(query_b), int(num_head), _p(out), _dt(out), b, sq, sk, samples, n_atoms, c, _p(ws), ws.numel(),
+        _stream(q_data.device))
+    _L.check(rc, "af3_gathered_cross_attention_forward")
+    return out
+
+
 def pair_logits(pair, norm_weight, norm_bias, w_padded, n_out):
     """LayerNorm + projection of the pair tensor to [n_out, N, N] fp32 logits
     (nn/d_pairformer.py:160-162, nn/d_diffusion_transformer.py:299-305)."""

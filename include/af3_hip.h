@@ -162,6 +162,29 @@ int af3_batch_diffusion_cross_attention_forward(
     void* workspace, size_t workspace_bytes, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * The same cross-attention with the key windows gathered inside the kernel.
+ * Replaces the sequence `atom_layout.convert(queries_to_keys, queries_act)`
+ * (nn/d_diffusion_transformer.py:519-523) -> adaptive LayerNorm of the keys ->
+ * batch_diffusion_cross_attention_forward for the case the reference always
+ * has in the atom transformers: every key of a window is one of the query
+ * atoms (or a masked slot).  K and V are then projected once per atom instead
+ * of once per (window, key), a quarter of the rows at 128 keys per 32 queries.
+ * q_data [B,Sq,C] as above with B = samples * bias_batches; atom_data
+ * [samples, n_atoms, C] bf16, the adaptive-LayerNorm-ed key input of every atom;
+ * key_rows [bias_batches, Sk] int32: row of atom_data that key k of window b is,
+ * or negative for a masked slot (K = V = 0, as the reference's zeroed gather
+ * gives).  Everything else as in af3_batch_diffusion_cross_attention_forward.
+ */
+size_t af3_gathered_cross_attention_workspace_bytes(int64_t batch, int64_t sq, int64_t samples, int64_t n_atoms,
+                                                    int channels);
+int af3_gathered_cross_attention_forward(
+    const uint16_t* q_data, const uint16_t* atom_data, const int32_t* key_rows,
+    const float* pair_logits, const float* mask_q, const float* mask_k, int64_t bias_batches,
+    const uint16_t* w_qg, const uint16_t* w_kv, const float* query_b, int num_head,
+    void* out, int out_dtype, int64_t batch, int64_t sq, int64_t sk, int64_t samples, int64_t n_atoms, int channels,
+    void* workspace, size_t workspace_bytes, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Pair-logit projection: out[h][i][j] = (LayerNorm(pair)[i][j] . w[h]).
  * Replaces the eager `single_pair_logits_projection(single_pair_logits_norm(
  * pair)).permute(2,0,1)` of nn/d_pairformer.py:160-162 and the

@@ -1,0 +1,170 @@
+"""Diffusion head on the GPU (HIP kernels through the C ABI) against the CPU
+oracle in float64 (oracle/af3_head_oracle.py), at sizes the oracle finishes in
+seconds, and size-independent properties at 768 tokens x 5 samples.
+
+Tolerances: bf16 path rms error of the position UPDATE (denoised minus the
+skip term) <= 1e-2 of its rms, max <= 8e-2; fp32 check mode 2e-4 / 2e-3."""
+
+import pytest
+import torch
+
+from oracle import af3_head_oracle as H
+from oracle import af3_oracle as O
+
+pytestmark = pytest.mark.gpu
+D = torch.float64
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def compare(name, got, ref, rms_tol, max_tol):
+    got, ref = got.double().cpu(), ref.double().cpu()
+    scale = float((ref ** 2).mean().sqrt())
+    rms = float(((got - ref) ** 2).mean().sqrt()) / scale
+    mx = float((got - ref).abs().max()) / scale
+    print(f"head {name}: rms {rms:.3e} max {mx:.3e} (rms of reference {scale:.3e})", flush=True)
+    assert torch.isfinite(got).all() and scale > 0
+    assert rms <= rms_tol and mx <= max_tol, (name, rms, mx)
+
+
+def case(pkg, n, blocks, seed, samples=2, pad=1, std=0.05):
+    g = gen(seed)
+    batch = pkg.nn.atom_layout.synthetic_batch(n, g, n_padding_tokens=pad, chain_len=5)
+    p = {k: O.round_bf16(v) for k, v in H.make_diffusion_head_params(g, num_blocks=blocks, std=std).items()}
+    emb = {"single": O.round_bf16(torch.randn(n, 384, generator=g)),
+           "pair": O.round_bf16(torch.randn(n, n, 128, generator=g)),
+           "target_feat": O.round_bf16(torch.randn(n, 447, generator=g))}
+    pos = torch.randn(samples, n, 24, 3, generator=g)
+    head = pkg.nn.DiffusionHead(num_blocks=blocks)
+    head.load_state_dict(p)
+    head.to(dev())
+    return g, batch, p, emb, pos, head
+
+
+def on_gpu(emb):
+    return {k: v.to(dev()) for k, v in emb.items()}
+
+
+@pytest.mark.parametrize("n,blocks", [(8, 1), (20, 4)])
+def test_pre_conditioning_and_head_against_oracle(gpu_pkg, n, blocks):
+    g, batch, p, emb, pos, head = case(gpu_pkg, n, blocks, seed=21 + n)
+    pd = O.cast_params(p, D)
+    embd = {k: v.double() for k, v in emb.items()}
+    levels, t_hat, _ = H.sampler_schedule(6)
+    want_sc, want_pc = H.pre_conditioning(batch, embd, t_hat, True, pd)
+    gb, ge = batch.to(dev()), on_gpu(emb)
+    for mode, rms_tol, max_tol in (("check", 2e-4, 2e-3), ("bf16", 1e-2, 8e-2)):
+        with gpu_pkg.nn.check_mode(mode == "check"):
+            sc, pc = head.pre_conditioning(gb, ge, t_hat.float().to(dev()), True)
+            compare(f"single_cond {mode}", sc, want_sc, rms_tol, max_tol)
+            compare(f"pair_cond {mode}", pc, want_pc, rms_tol, max_tol)
+            for step in (0, 3, 5):          # high, middle and low noise
+                t = t_hat[step]
+                noisy = pos.double() * float(t)
+                want = H.diffusion_head(noisy, t, batch, embd, want_sc[step], want_pc, pd, True, blocks)
+                got = head(noisy.float().to(dev()), t.float().to(dev()), gb, ge,
+                           want_sc[step].float().to(dev()), want_pc.float().to(dev()))
+                am = batch.predicted_structure_info.atom_mask.double()[None, ..., None]
+                skip = 256.0 / (float(t) ** 2 + 256.0) * noisy * am
+                compare(f"update, step {step}, {mode}", got.double().cpu() - skip, want - skip, rms_tol, max_tol)
+
+
+def test_state_reuse_is_exact_and_samples_are_independent(gpu_pkg):
+    g, batch, p, emb, pos, head = case(gpu_pkg, 16, 4, seed=31, samples=3)
+    gb, ge = batch.to(dev()), on_gpu(emb)
+    levels, t_hat, _ = H.sampler_schedule(4)
+    sc, pc = head.pre_conditioning(gb, ge, t_hat.float().to(dev()), True)
+    noisy = (pos * float(t_hat[2])).to(dev())
+    state = head.prepare(gb, ge, pc)
+    a = head(noisy, t_hat[2].float().to(dev()), gb, ge, sc[2], pc, state=state)
+    b = head(noisy, t_hat[2].float().to(dev()), gb, ge, sc[2], pc)                  # conditioning recomputed
+    c = head(noisy, t_hat[2].float().to(dev()), gb, ge, sc[2], pc, state=state)    # the state is not consumed
+    assert torch.equal(a, b) and torch.equal(a, c)
+    # a sample's result does not depend on which other samples share the batch
+    one = head(noisy[1:2].contiguous(), t_hat[2].float().to(dev()), gb, ge, sc[2], pc, state=state)
+    assert torch.equal(one[0], a[1])
+
+
+def test_sampler_against_oracle(gpu_pkg):
+    n, blocks, steps, samples = 12, 2, 4, 2
+    g, batch, p, emb, pos, head = case(gpu_pkg, n, blocks, seed=41, samples=samples)
+    pd = O.cast_params(p, D)
+    embd = {k: v.double() for k, v in emb.items()}
+    rots = torch.stack([gpu_pkg.nn.diffusion_head.random_rotation(g, "cpu", D) for _ in range(steps)])
+    transs = torch.randn(steps, 3, generator=g, dtype=D)
+    want = H.sample_diffusion(batch, embd, pd, pos.double(), rots, transs, steps, num_blocks=blocks)
+    gb, ge = batch.to(dev()), on_gpu(emb)
+    sampler = gpu_pkg.nn.DiffusionSampler(head, num_samples=samples, diffusion_steps=steps)
+    for mode, rms_tol, max_tol in (("check", 2e-4, 2e-3), ("bf16", 1e-2, 8e-2)):
+        with gpu_pkg.nn.check_mode(mode == "check"):
+            out = sampler(gb, ge, positions=pos.to(dev()), rotations=rots.float().to(dev()),
+                          translations=transs.float().to(dev()))
+        assert torch.equal(out["mask"].cpu(), batch.predicted_structure_info.atom_mask)
+        compare(f"sampled positions after {steps} steps, {mode}", out["atom_positions"], want, rms_tol, max_tol)
+    # gaussian noise handed in: the oracle takes the same draws
+    noises = torch.randn(steps, samples, n, 24, 3, generator=g, dtype=D)
+    want = H.sample_diffusion(batch, embd, pd, pos.double(), rots, transs, steps, num_blocks=blocks, noises=noises)
+    out = sampler(gb, ge, positions=pos.to(dev()), rotations=rots.float().to(dev()),
+                  translations=transs.float().to(dev()), noises=noises.float().to(dev()))
+    compare("sampled positions, gaussian noise", out["atom_positions"], want, 1e-2, 8e-2)
+
+
+def test_full_size_head_properties(gpu_pkg):
+    """768 tokens x 5 samples x 24 blocks: equal samples stay equal; a sample
+    evaluated alone gives the same result as inside the batch; padding atoms
+    stay at zero; one evaluation against the fp32 check mode."""
+    n, samples = 768, 5
+    g, batch, p, emb, pos, head = case(gpu_pkg, n, 24, seed=51, samples=samples, pad=40, std=0.02)
+    gb, ge = batch.to(dev()), on_gpu(emb)
+    levels, t_hat, _ = H.sampler_schedule(200)
+    t = t_hat[120:121].float().to(dev())
+    sc, pc = head.pre_conditioning(gb, ge, t, True)
+    state = head.prepare(gb, ge, pc)
+    am = gb.predicted_structure_info.atom_mask.bool()
+    noisy = (pos * float(t)).to(dev())
+    noisy[3] = noisy[0]
+    out = head(noisy, t[0], gb, ge, sc[0], pc, state=state)
+    assert torch.isfinite(out).all()
+    assert torch.equal(out[3], out[0])
+    assert torch.equal(out[:, ~am], torch.zeros_like(out[:, ~am]))
+    one = head(noisy[2:3].contiguous(), t[0], gb, ge, sc[0], pc, state=state)
+    assert torch.equal(one[0], out[2])
+    with gpu_pkg.nn.check_mode():
+        sc32, pc32 = head.pre_conditioning(gb, ge, t, True)
+        ref = head(noisy[:1].contiguous(), t[0], gb, ge, sc32[0], pc32)
+    compare("single_cond, bf16 vs fp32 check", sc, sc32, 1e-2, 8e-2)
+    compare("pair_cond, bf16 vs fp32 check", pc, pc32, 1e-2, 8e-2)
+    skip = 256.0 / (float(t) ** 2 + 256.0) * noisy[:1] * am[None, ..., None]
+    compare("update, bf16 vs fp32 check", out[:1] - skip, ref - skip, 2e-2, 2e-1)
+
+
+def test_per_atom_key_path_matches_the_gathered_key_tensor_path(gpu_pkg):
+    """The atom transformer with keys looked up inside the attention kernel
+    (K / V projected once per atom) against the same transformer fed the
+    gathered key tensors, which is the reference's formulation."""
+    g = gen(61)
+    batch = gpu_pkg.nn.atom_layout.synthetic_batch(20, g, n_padding_tokens=3)
+    q2k = batch.atom_cross_att.queries_to_keys.to(dev())
+    s = q2k.gather_idxs.shape[0]
+    p = {k: O.round_bf16(v) for k, v in O.make_cross_att_transformer_params(g, std=0.05).items()}
+    mod = gpu_pkg.nn.DiffusionCrossAttTransformer()
+    mod.load_state_dict(p)
+    mod.to(dev())
+    rb = O.round_bf16
+    qm = batch.atom_cross_att.token_atoms_to_queries.gather_mask.to(dev())
+    act = (rb(torch.randn(3, s, 32, 128, generator=g)).to(dev()) * qm[None, ..., None]).bfloat16()
+    cq = rb(torch.randn(s, 32, 128, generator=g)).to(dev()) * qm[..., None]
+    pc = rb(torch.randn(s, 32, 128, 16, generator=g)).to(dev())
+    ck = gpu_pkg.nn.atom_layout.convert(q2k, cq, (-3, -2)).contiguous()
+    km = gpu_pkg.nn.atom_layout.convert(q2k, qm, (-2, -1))
+    plain = mod(act.clone(), qm, q2k, km, cq, ck, pc)
+    cond = mod.conditioning(cq, ck, pc, keys_are_query_atoms=q2k)
+    fast = mod(act.clone(), qm, q2k, km, cq, ck, pc, cond=cond)
+    live = qm[None, ..., None]
+    compare("per-atom keys vs gathered keys", ((fast - act) * live).float(), ((plain - act) * live).float(), 2e-3, 3e-2)
