@@ -310,7 +310,10 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
 template <int KSTEPS, int DVT>
 int launch_nw(const FlashArgs& a, hipStream_t stream) {
   const int64_t heads = (int64_t)a.H * a.B;
-  const int nw = a.Sq <= 32 ? 1 : (((a.Sq + 127) / 128) * heads < 1024 ? 2 : 4);
+  // Four waves share each staged K / V tile once there are enough 128-query
+  // workgroups to cover the chip; below that, two waves per workgroup spread
+  // the work over twice as many CUs.
+  const int nw = a.Sq <= 32 ? 1 : (((a.Sq + 127) / 128) * heads < 256 ? 2 : 4);
   const int64_t blocks = (int64_t)((a.Sq + nw * 32 - 1) / (nw * 32)) * heads;
   if (blocks <= 0 || blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
   if (nw == 1) hipLaunchKernelGGL((flash_kernel<KSTEPS, DVT, 1>), dim3((unsigned)blocks), dim3(64), 0, stream, a);
