@@ -103,7 +103,12 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
   // and set kt & 1 (just stored) takes slab kt + 2
   auto stage = [&](int kt, auto par_c) {
     constexpr int par = decltype(par_c)::value;
-    if (kt + 2 < nk) gload(par, (kt + 2) * BK);
+    // Requested on every iteration, also past the last slab (a clamped
+    // re-read that is never stored): a load under a condition leaves the
+    // compiler unable to count the loads in flight, and it then waits for all
+    // of them, the slab just requested included, before the LDS stores below.
+    gload(par, (kt + 2) * BK);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       bf16x8 fa[2], fb[2];
@@ -116,6 +121,15 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(fa[i], fb[j], acc[i][j]);
     }
+    // fragment reads four ahead of the MFMAs that use them
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    __builtin_amdgcn_sched_barrier(0);
     if (kt + 1 < nk) sstore(par ^ 1, par ^ 1);
     lds_barrier();
   };
