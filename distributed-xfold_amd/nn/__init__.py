@@ -9,6 +9,7 @@ from .primitives import Transition
 from .diffusion_transformer import (AdaptiveLayerNorm, AdaLNZero, DiffusionTransition, SelfAttention,
                                     DiffusionTransformer, CrossAttention, DiffusionCrossAttTransformer)
 from .pairformer import PairformerBlock, PairformerStack
+from .evoformer import OuterProductMean, MSAAttention, EvoformerBlock
 from . import atom_layout
 from .atom_cross_attention import AtomCrossAttEncoder, AtomCrossAttDecoder, AtomCrossAttEncoderOutput
 from .diffusion_head import DiffusionHead, DiffusionSampler, FourierEmbeddings
@@ -25,6 +26,9 @@ DistributeDiffusionTransformer = DiffusionTransformer
 DistrubuteCrossAttention = CrossAttention
 DistributeDiffusionCrossAttTransformer = DiffusionCrossAttTransformer
 DistributePairformerBlock = PairformerBlock
+DistributeOuterProductMean = OuterProductMean
+DistributeMSAAttention = MSAAttention
+DistributeEvoformerBlock = EvoformerBlock
 DistributeAtomCrossAttEncoder = AtomCrossAttEncoder
 DistributeAtomCrossAttDecoder = AtomCrossAttDecoder
 DistributeDiffusionHead = DiffusionHead
@@ -34,6 +38,7 @@ __all__ = [
     "HipModule", "enable_hip", "check_mode", "in_check_mode", "TriangleMultiplication", "GridSelfAttention", "Transition",
     "AdaptiveLayerNorm", "AdaLNZero", "DiffusionTransition", "SelfAttention", "DiffusionTransformer",
     "CrossAttention", "DiffusionCrossAttTransformer", "PairformerBlock", "PairformerStack",
+    "OuterProductMean", "MSAAttention", "EvoformerBlock",
     "atom_layout", "AtomCrossAttEncoder", "AtomCrossAttDecoder", "AtomCrossAttEncoderOutput", "DiffusionHead",
     "DiffusionSampler", "FourierEmbeddings",
 ]
