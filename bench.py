@@ -153,6 +153,30 @@ def diffusion_step(pkg, n, dev, samples=5, iters=20):
             "sampling_200_steps_s": round((setup_ms + 200 * ms) / 1e3, 3)}
 
 
+def evoformer_block_ms(pkg, n, dev, rows=1024, iters=10):
+    """One Evoformer (MSA) block: outer-product mean, MSA pair-weighted
+    averaging, MSA transition and the five pair operators, bf16 streams."""
+    import torch
+    from oracle import af3_msa_oracle as M      # parameter generator only
+    g = torch.Generator().manual_seed(2)
+    blk = pkg.nn.EvoformerBlock()
+    blk.load_state_dict(M.make_evoformer_block_params(g))
+    blk = blk.to(dev)
+    blk.load_hip_params()
+    msa = torch.randn(rows, n, 64, generator=g).to(dev).bfloat16()
+    pair = torch.randn(n, n, 128, generator=g).to(dev).bfloat16()
+    seq = (torch.arange(n) < int(0.9 * n)).float().to(dev)
+    mm = seq[None, :].expand(rows, n).contiguous()
+    pm = (seq[:, None] * seq[None, :]).contiguous()
+    ms = gpu_time_ms(lambda: blk(msa, pair, mm, pm), iters, warm_ms=40.0)
+    ms_opm = gpu_time_ms(lambda: blk.outer_product_mean.run(msa, mm, residual=pair), iters)
+    ms_att = gpu_time_ms(lambda: blk.msa_attention1.run(msa, mm, pair, residual=True), iters)
+    flops_opm = 2.0 * (32 * n) ** 2 * rows + 2.0 * n * n * 1024 * 128
+    return {"workload": f"one Evoformer block, {rows} MSA rows x {n} tokens, c_msa=64, c_pair=128, bf16",
+            "ms_per_block": round(ms, 3), "outer_product_mean_ms": round(ms_opm, 3),
+            "outer_product_mean_tflops": round(flops_opm / ms_opm / 1e9, 1), "msa_attention_ms": round(ms_att, 3)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -161,7 +185,7 @@ def main():
     ap.add_argument("--n-token", type=int, default=768)
     ap.add_argument("--io", choices=["bf16", "f32"], default="bf16", help="dtype of the residual stream")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-diffusion", action="store_true", help="skip the diffusion-head timing")
+    ap.add_argument("--no-diffusion", action="store_true", help="skip the diffusion-head and Evoformer-block timings")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain elementwise kernel that reads and writes 256 MiB, three times: the "
                          "reference against which the FETCH_SIZE / WRITE_SIZE counters of a profiler run are scaled")
@@ -256,6 +280,7 @@ def main():
     diffusion = None
     if not args.no_diffusion:
         diffusion = diffusion_step(pkg, n, dev)
+    evo = None if args.no_diffusion else evoformer_block_ms(pkg, n, dev)
 
     if args.calibrate:
         cx = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device=dev)   # 256 MiB in, 256 MiB out
@@ -281,6 +306,8 @@ def main():
     }
     if diffusion is not None:
         out["diffusion_head"] = diffusion
+    if evo is not None:
+        out["evoformer_block"] = evo
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(n)
     print(json.dumps(out))

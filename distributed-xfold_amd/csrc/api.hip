@@ -393,9 +393,16 @@ int af3_linear_forward(
     int64_t m, int n, int k, int mode, float alpha, int sigmoid,
     const float* gate, int64_t gate_rows, const void* residual, int res_dtype, af3_stream_t stream) {
   if (!x || !w || !y || bad_dtype(y_dtype) || m <= 0 || m > 0x7fffffff || n <= 0 || k <= 0) return AF3_ERR_BAD_ARG;
-  if (mode != AF3_LINEAR_PLAIN && mode != AF3_LINEAR_SWIGLU && mode != AF3_LINEAR_GATE_RES) return AF3_ERR_BAD_ARG;
+  if (mode != AF3_LINEAR_PLAIN && mode != AF3_LINEAR_SWIGLU && mode != AF3_LINEAR_GATE_RES &&
+      mode != AF3_LINEAR_REGROUP32)
+    return AF3_ERR_BAD_ARG;
   if (residual && bad_dtype(res_dtype)) return AF3_ERR_BAD_ARG;
   GemmArgs g;
+  if (mode == AF3_LINEAR_REGROUP32) {
+    if ((m & 31) || (n & 31) || gate || residual) return AF3_ERR_BAD_ARG;
+    g.regroup32 = 1;
+    mode = AF3_LINEAR_PLAIN;
+  }
   g.A = x; g.B = w; g.C = y;
   g.M = (int)m; g.N = n; g.K = k;
   g.lda = k; g.ldb = k;

@@ -235,7 +235,9 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
         if (g.act_sigmoid) v[e] = sigmoidf_(v[e]);
       }
     }
-    const int64_t off = (int64_t)bz * g.sC + (int64_t)m * g.ldc + n;
+    const int64_t off = g.regroup32
+                            ? ((((int64_t)(m >> 5) * (g.N >> 5) + (n >> 5)) * 32 + (m & 31)) * 32 + (n & 31))
+                            : (int64_t)bz * g.sC + (int64_t)m * g.ldc + n;
     if (OUT_F32) {
       float* dst = reinterpret_cast<float*>(g.C) + off;
       if (full) {
@@ -265,6 +267,7 @@ int launch_gemm_nt(const GemmArgs& g_in, hipStream_t stream) {
   if (g.epi == EPI_SWIGLU && ((g.N & 63) || g.out_f32)) return AF3_ERR_BAD_ARG;
   if (g.epi == EPI_SEGMENTED && (g.seg_len <= 0 || (g.seg_len & 7))) return AF3_ERR_BAD_ARG;
   if (g.gate && g.gate_rows <= 0) return AF3_ERR_BAD_ARG;
+  if (g.regroup32 && (g.epi != EPI_PLAIN || g.batch != 1 || (g.M & 31) || (g.N & 31))) return AF3_ERR_BAD_ARG;
   // 16/32-byte stores need aligned rows; otherwise the epilogue stores element-wise
   const int esz = g.out_f32 ? 4 : 2;
   g.vec_ok = ((uintptr_t)g.C % 16 == 0) && ((g.ldc * esz) % 16 == 0) && ((g.sC * esz) % 16 == 0);

@@ -26,6 +26,10 @@ struct GemmArgs {
   const bf16_t* res_bf16 = nullptr;
   int64_t ld_res = 0, sRes = 0;
   int vec_ok = 0, res_vec_ok = 0;  // set by launch_gemm_nt: rows aligned for 16-byte stores / loads
+  // regroup32 (PLAIN, batch 1, M and N multiples of 32): element (m, n) is stored
+  // at [(m / 32, n / 32)][(m % 32, n % 32)], i.e. C is [(M/32)(N/32)][1024]:
+  // the outer products of 32-channel rows, one contiguous 1024-vector per pair.
+  int regroup32 = 0;
 };
 int launch_gemm_nt(const GemmArgs& g, hipStream_t stream);
 // contract.hip: the same product, plain bf16 output, 256x256 tiles (large M, N)

@@ -8,10 +8,11 @@ Both MSA operators are products over long axes and run on the bf16 MFMA
 kernels:
   * outer-product mean: out[b, d, :] = W^T vec(sum_a L[a, b, :] (x) R[a, d, :]).
     The sum over the MSA rows is one product [(b, c), a] x [(d, e), a]^T per
-    block of 128 tokens b (a 200 MB bf16 slab at 768 tokens, which stays in the
-    256 MB last-level cache for the regrouping to [(b, d), (c, e)] and the
-    second product with W [(c, e), f]); the [N, N, 32, 32] tensor the
-    reference's einsum materialises (1.2 GB) never exists as a whole.
+    block of 128 tokens b, whose epilogue stores element ((b, c), (d, e)) at
+    [(b, d)][(c, e)], the layout the second product with W [(c, e), f] reads
+    (a 200 MB bf16 slab at 768 tokens, inside the 256 MB last-level cache); the
+    [N, N, 32, 32] tensor the reference's einsum materialises (1.2 GB) never
+    exists as a whole and nothing is permuted.
   * pair-weighted averaging: per head, softmax(pair logits) [q, k] times the
     head's values of all MSA rows [(row, channel), k]^T.
 """
@@ -74,8 +75,11 @@ class OuterProductMean(HipModule):
         out = residual if residual is not None else torch.empty((n, n, cf), dtype=torch.float32, device=msa.device)
         for b0 in range(0, n, block):
             b1 = min(n, b0 + block)
-            outer = ops.linear(lt[b0 * co:b1 * co], rt)                                    # [(b, c), (d, e)]
-            outer = outer.view(b1 - b0, co, n, co).permute(0, 2, 1, 3).reshape((b1 - b0) * n, co * co)
+            if co == 32:
+                outer = ops.linear(lt[b0 * co:b1 * co], rt, mode=ops._L.LINEAR_REGROUP32)  # [(b, d), (c, e)]
+            else:
+                outer = ops.linear(lt[b0 * co:b1 * co], rt)                                # [(b, c), (d, e)]
+                outer = outer.view(b1 - b0, co, n, co).permute(0, 2, 1, 3).reshape((b1 - b0) * n, co * co)
             act = ops.linear(outer, p["w_out"], bias=p["b_out"], out_dtype=torch.float32).view(b1 - b0, n, cf)
             act = act / (self.epsilon + norm[b0:b1, :, None])
             if residual is not None:

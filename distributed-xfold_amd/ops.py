@@ -339,6 +339,10 @@ def linear(x, w, bias=None, out_dtype=torch.bfloat16, mode=_L.LINEAR_PLAIN, alph
         _gpu(bias, "bias", torch.float32, (n,))
     n_out = n // 2 if mode == _L.LINEAR_SWIGLU else n
     shape = tuple(x.shape[:-1]) + (n_out,)
+    if mode == _L.LINEAR_REGROUP32:
+        if m % 32 or n % 32:
+            raise ValueError("regrouped store: rows of x and of w must be multiples of 32")
+        shape = ((m // 32) * (n // 32), 1024)
     if out is None:
         out = torch.empty(shape, dtype=out_dtype, device=x.device)
     else:

@@ -223,10 +223,16 @@ int af3_layer_norm_forward(
  *        the linear half
  *  mode AF3_LINEAR_GATE_RES: y = residual + gate[m % gate_rows] * (x W^T + bias)
  *        (gate fp32 [gate_rows,N] or NULL; residual in res_dtype or NULL)
+ *  mode AF3_LINEAR_REGROUP32: PLAIN, with element (m, n) stored at
+ *        y[(m/32, n/32)][(m%32, n%32)], y [(M/32)*(N/32), 1024] (M, N multiples
+ *        of 32).  With x = [(token b, channel c), msa row] and w = [(token d,
+ *        channel e), msa row] this is the outer-product sum of
+ *        nn/d_primitives.py:63-64, laid out for the contraction with output_w.
  */
 #define AF3_LINEAR_PLAIN 0
 #define AF3_LINEAR_SWIGLU 2
 #define AF3_LINEAR_GATE_RES 3
+#define AF3_LINEAR_REGROUP32 4
 int af3_linear_forward(
     const uint16_t* x, const uint16_t* w, const float* bias,
     void* y, int y_dtype, int64_t m, int n, int k,
