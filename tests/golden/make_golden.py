@@ -70,7 +70,65 @@ def expected(n, seed):
     return {k: v.float().numpy() for k, v in out.items()}
 
 
+def head_inputs(n=8, seed=300, blocks=1, samples=2):
+    """Inputs of the diffusion-head case; the feature batch comes from the
+    product package's synthetic layout builder (pure PyTorch, no kernels)."""
+    from oracle import af3_head_oracle as H
+    import __graft_entry__ as ge
+    al = ge.load_package().nn.atom_layout
+    g = torch.Generator().manual_seed(seed)
+    rb = O.round_bf16
+    batch = al.synthetic_batch(n, g, n_padding_tokens=1, chain_len=3)
+    params = {k: rb(v) for k, v in H.make_diffusion_head_params(g, num_blocks=blocks, std=0.05).items()}
+    emb = {"single": rb(torch.randn(n, 384, generator=g)), "pair": rb(torch.randn(n, n, 128, generator=g)),
+           "target_feat": rb(torch.randn(n, 447, generator=g))}
+    pos = torch.randn(samples, n, 24, 3, generator=g)
+    return batch, params, emb, pos
+
+
+def head_expected(n=8, seed=300, blocks=1):
+    from oracle import af3_head_oracle as H
+    batch, params, emb, pos = head_inputs(n, seed, blocks)
+    p = O.cast_params(params, D)
+    embd = {k: v.double() for k, v in emb.items()}
+    _, t_hat, _ = H.sampler_schedule(6)
+    sc, pc = H.pre_conditioning(batch, embd, t_hat, True, p)
+    out = {"single_cond": sc, "pair_cond": pc}
+    for step in (1, 4):
+        out[f"denoised_step{step}"] = H.diffusion_head(pos.double() * float(t_hat[step]), t_hat[step], batch, embd,
+                                                       sc[step], pc, p, True, blocks)
+    return {k: v.float().numpy() for k, v in out.items()}
+
+
+def evoformer_inputs(rows=7, n=12, seed=400):
+    from oracle import af3_msa_oracle as M
+    g = torch.Generator().manual_seed(seed)
+    rb = O.round_bf16
+    params = {k: rb(v) for k, v in M.make_evoformer_block_params(g, std=0.05).items()}
+    msa = rb(torch.randn(rows, n, 64, generator=g))
+    pair = rb(torch.randn(n, n, 128, generator=g))
+    mm = (torch.rand(rows, n, generator=g) > 0.2).float()
+    mm[0] = 1
+    mm[:, n - 1] = 0
+    seq = mm.max(dim=0).values
+    pm = seq[:, None] * seq[None, :]
+    return params, msa, pair, mm, pm
+
+
+def evoformer_expected(rows=7, n=12, seed=400):
+    from oracle import af3_msa_oracle as M
+    params, msa, pair, mm, pm = evoformer_inputs(rows, n, seed)
+    m, z = M.evoformer_block(msa.double(), pair.double(), mm.double(), pm.double(), O.cast_params(params, D))
+    return {"msa": m.float().numpy(), "pair": z.float().numpy()}
+
+
 def main():
+    path = os.path.join(HERE, "diffusion_head_n8.npz")
+    np.savez_compressed(path, **head_expected())
+    print(path, os.path.getsize(path) // 1024, "KiB")
+    path = os.path.join(HERE, "evoformer_n12.npz")
+    np.savez_compressed(path, **evoformer_expected())
+    print(path, os.path.getsize(path) // 1024, "KiB")
     for n in SIZES:
         path = os.path.join(HERE, f"pairformer_n{n}.npz")
         np.savez_compressed(path, **expected(n, seed=100 + n))

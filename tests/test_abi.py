@@ -77,6 +77,52 @@ def test_null_and_bad_arguments_are_rejected_without_a_gpu(pkg):
                                                    None, 0, 8, None, 0, None) == -1
 
 
+def test_gathered_cross_attention_and_regrouped_store_reject_bad_arguments(pkg):
+    lib = pkg.lib.load()
+    one = 1 << 20     # a non-null dummy address: every check below fails before it is touched
+    args = dict(q=one, atoms=one, rows=one, pl=None, mq=None, mk=None, bb=4, wqg=one, wkv=one, qb=None, h=4,
+                out=one, dt=0, batch=8, sq=32, sk=128, samples=2, n_atoms=128, c=128, ws=one, wsb=1 << 30, st=None)
+
+    def call(**kw):
+        a = dict(args, **kw)
+        return lib.af3_gathered_cross_attention_forward(
+            a["q"], a["atoms"], a["rows"], a["pl"], a["mq"], a["mk"], a["bb"], a["wqg"], a["wkv"], a["qb"], a["h"],
+            a["out"], a["dt"], a["batch"], a["sq"], a["sk"], a["samples"], a["n_atoms"], a["c"], a["ws"], a["wsb"],
+            a["st"])
+    assert call(rows=None) == -1                       # key_rows is required
+    assert call(batch=9) == -1                         # batch must be samples * bias_batches
+    assert call(mq=one) == -1                          # masks come in pairs
+    assert call(c=100) == -1                           # channels: multiple of 8 and of the head count
+    assert call(h=8) != 0                              # head dim 16 is not supported
+    assert call(wsb=16) == -2                          # workspace too small
+    assert lib.af3_gathered_cross_attention_workspace_bytes(8, 32, 2, 128, 128) >= (8 * 32 + 2 * 128) * 256 * 2
+    # regrouped store: rows of both operands in multiples of 32, no gate / residual
+    assert lib.af3_linear_forward(one, one, None, one, 0, 48, 64, 8, 4, 1.0, 0, None, 0, None, 0, None) == -1
+    assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 4, 1.0, 0, one, 1, None, 0, None) == -1
+    assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 5, 1.0, 0, None, 0, None, 0, None) == -1
+
+
+def test_new_modules_share_the_reference_parameter_names(pkg):
+    from oracle import af3_head_oracle as H
+    from oracle import af3_msa_oracle as M
+    g = torch.Generator().manual_seed(0)
+    pairs = [
+        (pkg.nn.DiffusionHead(num_blocks=4), H.make_diffusion_head_params(g, num_blocks=4)),
+        (pkg.nn.AtomCrossAttDecoder(), H.make_decoder_params(g)),
+        (pkg.nn.AtomCrossAttEncoder(), H.make_encoder_params(g, 384, False, False, False)),
+        (pkg.nn.EvoformerBlock(), M.make_evoformer_block_params(g)),
+    ]
+    for mod, params in pairs:
+        assert sorted(mod.state_dict()) == sorted(params)
+        for k, v in mod.state_dict().items():
+            assert v.shape == params[k].shape, k
+    mesh = object()
+    assert pkg.nn.DistributeDiffusionHead(mesh, use_batch_infer=True).use_batch_infer is True
+    assert pkg.nn.DistributeEvoformerBlock(mesh, c_msa=64, c_pair=128).c_msa == 64
+    assert pkg.nn.DistributeAtomCrossAttDecoder(mesh, use_batch_infer=True).use_batch_infer is True
+    assert pkg.nn.DistributeOuterProductMean(mesh, c_msa=64, num_output_channel=128).num_outer_channel == 32
+
+
 def test_cpu_tensors_raise(pkg):
     with pytest.raises(ValueError):
         pkg.ops.layer_norm(torch.randn(4, 128))
