@@ -186,6 +186,8 @@ def main():
     ap.add_argument("--io", choices=["bf16", "f32"], default="bf16", help="dtype of the residual stream")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-diffusion", action="store_true", help="skip the diffusion-head and Evoformer-block timings")
+    ap.add_argument("--only", choices=["diffusion-head", "evoformer-block"],
+                    help="run that leg alone and print its object (for profiler runs)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain elementwise kernel that reads and writes 256 MiB, three times: the "
                          "reference against which the FETCH_SIZE / WRITE_SIZE counters of a profiler run are scaled")
@@ -203,6 +205,10 @@ def main():
 
     dev = torch.device("cuda:0")
     n = args.n_token
+    if args.only:
+        leg = diffusion_step(pkg, n, dev) if args.only == "diffusion-head" else evoformer_block_ms(pkg, n, dev)
+        print(json.dumps({args.only: leg}))
+        return
     io = torch.bfloat16 if args.io == "bf16" else torch.float32
     g = torch.Generator().manual_seed(0)
     blk = pkg.nn.PairformerBlock()
