@@ -177,6 +177,25 @@ def evoformer_block_ms(pkg, n, dev, rows=1024, iters=10):
             "outer_product_mean_tflops": round(flops_opm / ms_opm / 1e9, 1), "msa_attention_ms": round(ms_att, 3)}
 
 
+def trunk_recycle_ms(pkg, n, dev, rows=1024, iters=3):
+    """One recycling pass of the Evoformer trunk: input embeddings, 4 Evoformer
+    (MSA) blocks, 48 Pairformer blocks (no template embedding), bf16 streams."""
+    import torch
+    from oracle import af3_trunk_oracle as T     # parameter generator only
+    g = torch.Generator().manual_seed(3)
+    mod = pkg.nn.Evoformer()
+    mod.load_state_dict(T.make_evoformer_params(g))
+    mod = mod.to(dev)
+    mod.load_hip_params()
+    batch = pkg.nn.atom_layout.synthetic_trunk_batch(n, rows, g, n_padding_tokens=n // 10).to(dev)
+    tf = torch.randn(n, 447, generator=g).to(dev)
+    prev = {"pair": torch.randn(n, n, 128, generator=g).to(dev), "single": torch.randn(n, 384, generator=g).to(dev)}
+    ms = gpu_time_ms(lambda: mod(batch, prev, tf), iters, warmup=1)
+    return {"workload": f"one recycling pass of the trunk: embeddings + 4 Evoformer blocks ({rows} MSA rows) + 48 "
+                        f"Pairformer blocks, N_token={n}, bf16",
+            "ms_per_recycle": round(ms, 2)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -186,7 +205,7 @@ def main():
     ap.add_argument("--io", choices=["bf16", "f32"], default="bf16", help="dtype of the residual stream")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-diffusion", action="store_true", help="skip the diffusion-head and Evoformer-block timings")
-    ap.add_argument("--only", choices=["diffusion-head", "evoformer-block"],
+    ap.add_argument("--only", choices=["diffusion-head", "evoformer-block", "trunk-recycle"],
                     help="run that leg alone and print its object (for profiler runs)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain elementwise kernel that reads and writes 256 MiB, three times: the "
@@ -206,7 +225,8 @@ def main():
     dev = torch.device("cuda:0")
     n = args.n_token
     if args.only:
-        leg = diffusion_step(pkg, n, dev) if args.only == "diffusion-head" else evoformer_block_ms(pkg, n, dev)
+        leg = {"diffusion-head": diffusion_step, "evoformer-block": evoformer_block_ms,
+               "trunk-recycle": trunk_recycle_ms}[args.only](pkg, n, dev)
         print(json.dumps({args.only: leg}))
         return
     io = torch.bfloat16 if args.io == "bf16" else torch.float32

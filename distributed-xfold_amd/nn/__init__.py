@@ -10,6 +10,7 @@ from .diffusion_transformer import (AdaptiveLayerNorm, AdaLNZero, DiffusionTrans
                                     DiffusionTransformer, CrossAttention, DiffusionCrossAttTransformer)
 from .pairformer import PairformerBlock, PairformerStack
 from .evoformer import OuterProductMean, MSAAttention, EvoformerBlock
+from .trunk import Evoformer
 from . import atom_layout
 from .atom_cross_attention import AtomCrossAttEncoder, AtomCrossAttDecoder, AtomCrossAttEncoderOutput
 from .diffusion_head import DiffusionHead, DiffusionSampler, FourierEmbeddings
@@ -29,6 +30,7 @@ DistributePairformerBlock = PairformerBlock
 DistributeOuterProductMean = OuterProductMean
 DistributeMSAAttention = MSAAttention
 DistributeEvoformerBlock = EvoformerBlock
+DistributeEvoformer = Evoformer
 DistributeAtomCrossAttEncoder = AtomCrossAttEncoder
 DistributeAtomCrossAttDecoder = AtomCrossAttDecoder
 DistributeDiffusionHead = DiffusionHead
@@ -38,7 +40,7 @@ __all__ = [
     "HipModule", "enable_hip", "check_mode", "in_check_mode", "TriangleMultiplication", "GridSelfAttention", "Transition",
     "AdaptiveLayerNorm", "AdaLNZero", "DiffusionTransition", "SelfAttention", "DiffusionTransformer",
     "CrossAttention", "DiffusionCrossAttTransformer", "PairformerBlock", "PairformerStack",
-    "OuterProductMean", "MSAAttention", "EvoformerBlock",
+    "OuterProductMean", "MSAAttention", "EvoformerBlock", "Evoformer",
     "atom_layout", "AtomCrossAttEncoder", "AtomCrossAttDecoder", "AtomCrossAttEncoderOutput", "DiffusionHead",
     "DiffusionSampler", "FourierEmbeddings",
 ]

@@ -173,3 +173,50 @@ def synthetic_batch(n_token: int, gen: Optional[torch.Generator] = None, atoms_p
         ref_space_uid=idx[:, None].expand(shp).contiguous(),
     )
     return Batch(tf, rs, PredictedStructureInfo(atom_mask.float()), atom_cross_att_layout(atom_mask))
+
+
+@dataclass
+class PolymerLigandBondInfo:
+    tokens_to_polymer_ligand_bonds: GatherInfo     # gather_idxs / gather_mask [bonds, 2]
+
+
+@dataclass
+class LigandLigandBondInfo:
+    tokens_to_ligand_ligand_bonds: GatherInfo      # gather_idxs / gather_mask [bonds, 2]
+
+
+@dataclass
+class TrunkBatch:
+    """What the Evoformer trunk reads (d_alphafold3.py:67-191), with the MSA
+    already featurised: msa_feat [rows, N, 34], msa_mask [rows, N]."""
+    token_features: TokenFeatures
+    polymer_ligand_bond_info: PolymerLigandBondInfo
+    ligand_ligand_bond_info: LigandLigandBondInfo
+    msa_feat: torch.Tensor
+    msa_mask: torch.Tensor
+
+    to = Batch.to
+
+
+def synthetic_trunk_batch(n_token: int, msa_rows: int, gen: Optional[torch.Generator] = None,
+                          n_padding_tokens: int = 0, chain_len: int = 97, n_bonds: int = 6) -> TrunkBatch:
+    """A random trunk batch: the token features of `synthetic_batch`, a few
+    bonds between random live tokens (one of each kind with a masked end) and
+    random MSA features with a 0/1 mask whose first row covers every live token."""
+    g = gen
+    live = n_token - n_padding_tokens
+    idx = torch.arange(n_token)
+    chain = idx // chain_len
+    tf = TokenFeatures(mask=(idx < live).float(), token_index=idx.clone(), residue_index=idx % chain_len,
+                       asym_id=chain + 1, entity_id=chain % 3 + 1, sym_id=chain // 3 + 1)
+
+    def bonds():
+        gi = torch.randint(0, live, (n_bonds, 2), generator=g)
+        gm = torch.ones(n_bonds, 2, dtype=torch.bool)
+        gm[-1, 1] = False
+        return GatherInfo(gi, gm, (n_token,))
+    seq = tf.mask
+    mm = (torch.rand(msa_rows, n_token, generator=g) > 0.2).float() * seq[None, :]
+    mm[0] = seq
+    feat = torch.randn(msa_rows, n_token, 34, generator=g) * mm[..., None]
+    return TrunkBatch(tf, PolymerLigandBondInfo(bonds()), LigandLigandBondInfo(bonds()), feat, mm)
