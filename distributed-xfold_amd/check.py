@@ -64,16 +64,17 @@ def triangle_multiplication(mod, pair, mask):
     x = _ln(pair, mod.left_norm_input)
     proj = _lin(x, mod.projection)
     gate = _lin(x, mod.gate)
-    a = torch.empty((128, n, n), dtype=torch.float32, device=pair.device)
+    c = pair.shape[-1]
+    a = torch.empty((c, n, n), dtype=torch.float32, device=pair.device)
     b = torch.empty_like(a)
     maskf = None if mask is None else mask.to(torch.float32).contiguous()
     incoming = 0 if mod._outgoing else 1
-    ops.ck_elementwise(SPLIT, proj, gate, maskf, a, b, n, 0, incoming)
+    ops.ck_elementwise(SPLIT, proj, gate, maskf, a, b, n, c, incoming)
     # outgoing: t[c] = a[c] b[c]^T ; incoming (operands stored transposed): t[c] = b'[c] a'[c]^T
     lhs, rhs = (a, b) if mod._outgoing else (b, a)
-    t = ops.ck_gemm(lhs, rhs, m=n, n=n, k=n, batch=128, lda=n, ldb=n, sa=n * n, sb=n * n)
-    tp = torch.empty((n, n, 128), dtype=torch.float32, device=pair.device)
-    ops.ck_elementwise(CHAN_TO_PIX, t, None, None, tp, None, n, 128, 0)
+    t = ops.ck_gemm(lhs, rhs, m=n, n=n, k=n, batch=c, lda=n, ldb=n, sa=n * n, sb=n * n)
+    tp = torch.empty((n, n, c), dtype=torch.float32, device=pair.device)
+    ops.ck_elementwise(CHAN_TO_PIX, t, None, None, tp, None, n, c, 0)
     y = _ln(tp, mod.center_norm)
     out_gate = _lin(x, mod.gating_linear, sigmoid=True)
     return _lin(y, mod.output_projection, mul=out_gate)
@@ -86,7 +87,7 @@ def grid_self_attention(mod, pair, mask):
     nb = _lin(x, mod.pair_bias_projection)                    # [q, k, h]
     if mod.transpose:
         x = _transpose_pix(x)
-    d = 128 // h
+    d = pair.shape[-1] // h
     q = _lin(x, mod.q_projection, alpha=d ** -0.5)
     k = _lin(x, mod.k_projection)
     v = _lin(x, mod.v_projection)

@@ -206,7 +206,7 @@ size_t af3_batch_diffusion_self_attention_workspace_bytes(int64_t batch, int64_t
 }
 
 int af3_batch_diffusion_self_attention_forward(
-    const uint16_t* q_data, const float* key_mask, const float* nonbatched_bias,
+    const uint16_t* q_data, const float* key_mask, int64_t mask_batches, const float* nonbatched_bias,
     const uint16_t* w_qkvg, const float* query_b, int num_head,
     void* out, int out_dtype, int64_t batch, int64_t seq, int channels,
     void* workspace, size_t workspace_bytes, af3_stream_t stream) {
@@ -215,8 +215,9 @@ int af3_batch_diffusion_self_attention_forward(
       channels % num_head)
     return AF3_ERR_BAD_ARG;
   if (batch * seq > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  if (key_mask && mask_batches != 1 && mask_batches != batch) return AF3_ERR_BAD_ARG;
   const int d = channels / num_head;
-  if (d != 24 && d != 32 && d != 48) return AF3_ERR_UNSUPPORTED;
+  if (d != 16 && d != 24 && d != 32 && d != 48) return AF3_ERR_UNSUPPORTED;
   Carver ws(workspace, workspace_bytes);
   bf16_t* qkvg = ws.take<bf16_t>((size_t)batch * seq * 4 * channels);
   if (!ws.ok) return AF3_ERR_WORKSPACE;
@@ -240,8 +241,22 @@ int af3_batch_diffusion_self_attention_forward(
   f.out = out; f.out_f32 = out_dtype == AF3_F32; f.o_ss = channels; f.o_sb = seq * channels;
   f.B = (int)batch; f.H = num_head; f.Sq = f.Sk = (int)seq; f.d = d;
   f.bias = nonbatched_bias; f.bias_sb = 0; f.bias_sh = seq * seq; f.bias_sq = seq;
-  f.key_mask = key_mask; f.km_sb = 0;
+  f.key_mask = key_mask; f.km_sb = mask_batches == batch && batch > 1 ? seq : 0;
   return launch_flash_attention(f, s);
+}
+
+// ------------------------------------------------------------ batched NT product
+int af3_batched_nt_product_forward(
+    const uint16_t* a, const uint16_t* b, uint16_t* c, int64_t batch, int64_t m, int64_t n, int64_t k,
+    af3_stream_t stream) {
+  if (!a || !b || !c || batch <= 0 || m <= 0 || n <= 0 || k <= 0 || (k & 7)) return AF3_ERR_BAD_ARG;
+  if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff || batch > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  GemmArgs g;
+  g.A = a; g.B = b; g.C = c;
+  g.M = (int)m; g.N = (int)n; g.K = (int)k; g.batch = (int)batch;
+  g.lda = g.ldb = k; g.ldc = n;
+  g.sA = m * k; g.sB = n * k; g.sC = m * n;
+  return launch_gemm_nt(g, static_cast<hipStream_t>(stream));
 }
 
 // --------------------------------------------------- windowed (atom) cross-attention

@@ -326,7 +326,7 @@ int launch_nw(const FlashArgs& a, hipStream_t stream) {
 
 int launch_flash_attention(const FlashArgs& a, hipStream_t stream) {
   if (a.B <= 0 || a.H <= 0 || a.Sq <= 0 || a.Sk <= 0 || !a.q || !a.k || !a.v || !a.out) return AF3_ERR_BAD_ARG;
-  if (a.d != 24 && a.d != 32 && a.d != 48) return AF3_ERR_UNSUPPORTED;
+  if (a.d != 16 && a.d != 24 && a.d != 32 && a.d != 48) return AF3_ERR_UNSUPPORTED;
   const int64_t strides[] = {a.q_sb, a.q_ss, a.k_sb, a.k_ss, a.v_sb, a.v_ss, a.g_sb, a.g_ss, a.o_sb, a.o_ss};
   for (int64_t s : strides)
     if (s & 7) return AF3_ERR_BAD_ARG;
@@ -336,5 +336,6 @@ int launch_flash_attention(const FlashArgs& a, hipStream_t stream) {
   if ((a.qpad == nullptr) != (a.kpad == nullptr)) return AF3_ERR_BAD_ARG;
   if (a.key_rows && (a.bias_mod <= 0 || a.B % a.bias_mod)) return AF3_ERR_BAD_ARG;
   if (a.d == 48) return launch_nw<3, 2>(a, stream);
+  if (a.d == 16) return launch_nw<1, 1>(a, stream);
   return launch_nw<2, 1>(a, stream);
 }

@@ -99,11 +99,11 @@ __global__ __launch_bounds__(256) void ck_ln_kernel(CkNormArgs a) {
 // triangle multiplication: v = proj * mask * sigmoid(gate); even channels -> a, odd -> b,
 // written channel-major; incoming stores them transposed (a'[c][j][k] = a[k][j][c]).
 __global__ void ck_trimul_split_kernel(const float* proj, const float* gate, const float* mask, float* a, float* b,
-                                       int N, int incoming) {
-  const int64_t total = (int64_t)N * N * 256;
+                                       int N, int C2, int incoming) {
+  const int64_t total = (int64_t)N * N * C2;
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
-    const int ch2 = (int)(idx % 256);
-    const int64_t pix = idx / 256;
+    const int ch2 = (int)(idx % C2);
+    const int64_t pix = idx / C2;
     const int r = (int)(pix / N), c = (int)(pix % N);
     const float m = mask ? mask[pix] : 1.f;
     const float v = proj[idx] * m / (1.0f + expf(-gate[idx]));
@@ -224,7 +224,10 @@ int launch_ck_elementwise(int op, const float* x0, const float* x1, const float*
   switch (op) {
     case CK_TRIMUL_SPLIT:
       if (!x1 || !y1 || n0 > 8192) return AF3_ERR_BAD_ARG;
-      hipLaunchKernelGGL(ck_trimul_split_kernel, dim3(grid_for(n0 * n0 * 256)), dim3(256), 0, s, x0, x1, x2, y0, y1, (int)n0, flag);
+      // n1: pair channels (0 = 128); proj / gate hold twice as many
+      if (n1 < 0 || n1 > 4096) return AF3_ERR_BAD_ARG;
+      hipLaunchKernelGGL(ck_trimul_split_kernel, dim3(grid_for(n0 * n0 * 2 * (n1 ? n1 : 128))), dim3(256), 0, s, x0, x1, x2,
+                         y0, y1, (int)n0, (int)(2 * (n1 ? n1 : 128)), flag);
       break;
     case CK_CHAN_TO_PIX:
       if (n0 > 8192 || n1 <= 0) return AF3_ERR_BAD_ARG;

@@ -18,8 +18,9 @@ class GridSelfAttention(HipModule):
         args = drop_mesh(args)
         vals = list(args) + [c_pair, num_head, transpose][len(args):]
         c_pair, num_head, transpose = vals
-        if c_pair != 128 or c_pair // num_head != 32:
-            raise ValueError("the HIP triangle attention is built for c_pair = 128 and head dim 32")
+        if c_pair % num_head or c_pair // num_head not in (16, 24, 32, 48):
+            raise ValueError("head dim must be 16, 24, 32 or 48")
+        self.fused = c_pair == 128 and c_pair // num_head == 32
         self.c_pair, self.num_head, self.transpose = c_pair, num_head, transpose
         self.qkv_dim = c_pair // num_head
         self.act_norm = nn.LayerNorm(c_pair)
@@ -31,6 +32,12 @@ class GridSelfAttention(HipModule):
         self.output_projection = nn.Linear(c_pair, c_pair, bias=False)
 
     def _pack(self):
+        if not self.fused:
+            return dict(
+                w_qkvg=bf16(torch.cat([self.q_projection.weight, self.k_projection.weight,
+                                       self.v_projection.weight, self.gating_query.weight], dim=0)),
+                w_out=bf16(self.output_projection.weight), w_bias=bf16(self.pair_bias_projection.weight),
+                ln_w=f32(self.act_norm.weight), ln_b=f32(self.act_norm.bias))
         return dict(
             w_qkvg=bf16(torch.stack([self.q_projection.weight, self.k_projection.weight,
                                      self.v_projection.weight, self.gating_query.weight])),
@@ -39,7 +46,32 @@ class GridSelfAttention(HipModule):
             ln_w=f32(self.act_norm.weight), ln_b=f32(self.act_norm.bias),
         )
 
+    def _run_other_width(self, pair, mask, residual: bool):
+        """Pair widths other than 128 (the 64-channel blocks of the template
+        embedding): LayerNorm, the pair-bias projection, the pair-biased gated
+        attention over the rows (or columns) with one key mask per row, and the
+        output projection as separate launches of the general kernels."""
+        p = self.packed()
+        n, c, h = pair.shape[0], self.c_pair, self.num_head
+        x = ops.layer_norm(pair, p["ln_w"], p["ln_b"])                                       # [q, k, c]
+        bias = ops.linear(x, p["w_bias"], out_dtype=torch.float32).permute(2, 0, 1).contiguous()   # [h, q, k]
+        if self.transpose:
+            # bias and key mask are taken before the activations are transposed (nn/d_attention.py:60-65)
+            x = x.transpose(0, 1).contiguous()
+        o = ops.batch_diffusion_self_attention(x, mask.to(torch.float32).contiguous(), bias, p["w_qkvg"], None,
+                                               h)                                              # [b, s, h, d]
+        if not self.transpose:
+            return ops.linear(o.view(n, n, c), p["w_out"], out_dtype=pair.dtype, mode=ops._L.LINEAR_GATE_RES,
+                              residual=pair if residual else None, out=pair if residual else None)
+        upd = ops.linear(o.view(n, n, c), p["w_out"], out_dtype=pair.dtype).transpose(0, 1)
+        if residual:
+            pair += upd
+            return pair
+        return upd.contiguous()
+
     def run(self, pair, mask, residual: bool):
+        if not self.fused:
+            return self._run_other_width(pair, mask, residual)
         p = self.packed()
         return ops.grid_self_attn(pair, mask, self.transpose, p["ln_w"], p["ln_b"], p["w_bias"], None,
                                   p["w_qkvg"], p["w_out"], self.num_head, residual=residual)

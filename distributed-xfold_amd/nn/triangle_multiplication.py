@@ -21,8 +21,8 @@ class TriangleMultiplication(HipModule):
             c_pair = args[0]
         if len(args) > 1:
             _outgoing = args[1]
-        if c_pair != 128:
-            raise ValueError("the HIP triangle multiplication is built for c_pair = 128")
+        if c_pair % 8:
+            raise ValueError("c_pair must be a multiple of 8")
         self.c_pair = c_pair
         self.left_norm_input = nn.LayerNorm(c_pair)
         self.projection = nn.Linear(c_pair, 2 * c_pair, bias=False)
@@ -36,6 +36,12 @@ class TriangleMultiplication(HipModule):
         self.equation = "cik,cjk->cij" if _outgoing else "ckj,cki->cij"
 
     def _pack(self):
+        if self.c_pair != 128:
+            return dict(
+                w_proj=bf16(self.projection.weight), w_gate=bf16(self.gate.weight),
+                w_out=bf16(self.output_projection.weight), w_gl=bf16(self.gating_linear.weight),
+                ln_in_w=f32(self.left_norm_input.weight), ln_in_b=f32(self.left_norm_input.bias),
+                ln_c_w=f32(self.center_norm.weight), ln_c_b=f32(self.center_norm.bias))
         # operand a of channel c is output row 2c of projection/gate, operand b row
         # 2c+1 (d_triangle_multiplication.py:162-165; de-interleave as :128-129),
         # regrouped into four [64 projection rows | 64 gate rows] chunks.
@@ -53,7 +59,35 @@ class TriangleMultiplication(HipModule):
             ln_c_w=f32(self.center_norm.weight), ln_c_b=f32(self.center_norm.bias),
         )
 
+    def _run_other_width(self, pair: torch.Tensor, mask, residual: bool):
+        """Pair widths other than 128 (the 64-channel blocks of the template
+        embedding, nn/d_template.py:198-201): the same steps as separate
+        launches — LayerNorm, projections and the per-channel contraction on the
+        MFMA kernels, the gating products and layout changes as elementwise passes."""
+        p = self.packed()
+        n, c = pair.shape[0], self.c_pair
+        x = ops.layer_norm(pair, p["ln_in_w"], p["ln_in_b"])
+        proj = ops.linear(x, p["w_proj"], out_dtype=torch.float32)
+        gate = ops.linear(x, p["w_gate"], out_dtype=torch.float32, sigmoid=True)
+        pg = proj * gate * mask.to(torch.float32)[..., None]                      # [i, k, 2c]
+        # operand a of channel ch is row 2 ch, operand b row 2 ch + 1 (:162-165); channel-major, k last
+        if self._outgoing:       # out[i, j] = sum_k a[i, k] b[j, k]
+            lhs, rhs = pg[..., 0::2].permute(2, 0, 1), pg[..., 1::2].permute(2, 0, 1)
+        else:                    # out[i, j] = sum_k b[k, i] a[k, j]
+            lhs, rhs = pg[..., 1::2].permute(2, 1, 0), pg[..., 0::2].permute(2, 1, 0)
+        pad = (0, (-n) % 8)
+        lhs = torch.nn.functional.pad(lhs.to(torch.bfloat16), pad).contiguous()
+        rhs = torch.nn.functional.pad(rhs.to(torch.bfloat16), pad).contiguous()
+        t = ops.batched_nt_product(lhs, rhs).permute(1, 2, 0).contiguous()        # [i, j, c]
+        y = ops.layer_norm(t, p["ln_c_w"], p["ln_c_b"])
+        out_gate = ops.linear(x, p["w_gl"], out_dtype=torch.float32, sigmoid=True)
+        return ops.linear(y, p["w_out"], out_dtype=pair.dtype, mode=ops._L.LINEAR_GATE_RES,
+                          gate=out_gate.view(n * n, c), residual=pair if residual else None,
+                          out=pair if residual else None)
+
     def run(self, pair: torch.Tensor, mask, residual: bool):
+        if self.c_pair != 128:
+            return self._run_other_width(pair, mask, residual)
         p = self.packed()
         return ops.triangle_multiplication(
             pair, mask, 0 if self._outgoing else 1, p["ln_in_w"], p["ln_in_b"], p["w_proj_gate"],

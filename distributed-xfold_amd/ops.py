@@ -171,13 +171,19 @@ def transition128(act, layernorm_weight, layernorm_bias, w1_packed, w2, residual
 def batch_diffusion_self_attention(q_data, key_mask, nonbatched_bias, w_qkvg, query_b, num_head,
                                    out_dtype=torch.bfloat16):
     """batch_diffusion_self_attention_forward (csrc/Alpha_Attention.cpp:72-92).
-    q_data [B, S, C] bf16 (already normalised); returns [B, S, H, C/H]."""
+    q_data [B, S, C] bf16 (already normalised); key_mask [S] (shared) or [B, S];
+    returns [B, S, H, C/H]."""
     lib = _L.load()
     _gpu(q_data, "q_data", torch.bfloat16)
     if q_data.dim() != 3:
         raise ValueError("q_data: expected [B, S, C]")
     b, s, c = q_data.shape
-    km = _mask_f32(key_mask, (s,), "key_mask")
+    mask_batches = 1
+    if key_mask is not None and key_mask.dim() == 2:
+        mask_batches = b
+        km = _mask_f32(key_mask, (b, s), "key_mask")
+    else:
+        km = _mask_f32(key_mask, (s,), "key_mask")
     if nonbatched_bias is not None:
         _gpu(nonbatched_bias, "nonbatched_bias", torch.float32, (num_head, s, s))
     _gpu(w_qkvg, "w_qkvg", torch.bfloat16, (4 * c, c))
@@ -187,7 +193,7 @@ def batch_diffusion_self_attention(q_data, key_mask, nonbatched_bias, w_qkvg, qu
     nbytes = lib.af3_batch_diffusion_self_attention_workspace_bytes(b, s, c)
     ws = _ws(nbytes, q_data.device)
     rc = lib.af3_batch_diffusion_self_attention_forward(
-        _p(q_data), _p(km), _p(nonbatched_bias), _p(w_qkvg), _p(query_b), int(num_head), _p(out),
+        _p(q_data), _p(km), mask_batches, _p(nonbatched_bias), _p(w_qkvg), _p(query_b), int(num_head), _p(out),
         _dt(out), b, s, c, _p(ws), ws.numel(), _stream(q_data.device))
     _L.check(rc, "af3_batch_diffusion_self_attention_forward")
     return out
@@ -273,6 +279,26 @@ def gathered_cross_attention(q_data, atom_data, key_rows, pair_logits, mask_q, m
         _p(query_b), int(num_head), _p(out), _dt(out), b, sq, sk, samples, n_atoms, c, _p(ws), ws.numel(),
         _stream(q_data.device))
     _L.check(rc, "af3_gathered_cross_attention_forward")
+    return out
+
+
+def batched_nt_product(a, b, out=None):
+    """out[i] = a[i] @ b[i].T for a [batch, m, k], b [batch, n, k] bf16 (af3_batched_nt_product_forward)."""
+    lib = _L.load()
+    _gpu(a, "a", torch.bfloat16)
+    _gpu(b, "b", torch.bfloat16)
+    if a.dim() != 3 or b.dim() != 3 or a.shape[0] != b.shape[0] or a.shape[2] != b.shape[2]:
+        raise ValueError("expected a [batch, m, k] and b [batch, n, k]")
+    batch, m, k = a.shape
+    n = b.shape[1]
+    if k % 8:
+        raise ValueError("k must be a multiple of 8 (pad with zero columns)")
+    if out is None:
+        out = torch.empty((batch, m, n), dtype=torch.bfloat16, device=a.device)
+    else:
+        _gpu(out, "out", torch.bfloat16, (batch, m, n))
+    rc = lib.af3_batched_nt_product_forward(_p(a), _p(b), _p(out), batch, m, n, k, _stream(a.device))
+    _L.check(rc, "af3_batched_nt_product_forward")
     return out
 
 

@@ -124,15 +124,17 @@ int af3_transition_forward(
  *   csrc/batch_diffusion_self_attention{,_bf16}.h), used for the Pairformer
  *   single attention and the diffusion transformer
  *   (nn/d_diffusion_transformer.py:197-218).
- * q_data [B,S,C] bf16, already (adaptive-)LayerNorm-ed; key_mask [S] fp32 0/1
- * (masked keys replaced by -1e9) or NULL; nonbatched_bias [H,S,S] fp32 shared
- * by the batch, or NULL.  w_qkvg [4C][C] bf16 = q, k, v, gating_query rows as
- * stored by nn.Linear; query_b [C] fp32.  head_dim = C/H in {24, 32, 48}.
+ * q_data [B,S,C] bf16, already (adaptive-)LayerNorm-ed; key_mask fp32 0/1
+ * (masked keys replaced by -1e9) or NULL: [S] shared by the batch
+ * (mask_batches = 1) or [B,S], one per batch entry as the reference operator's
+ * bias [B,1,1,S] is (mask_batches = B); nonbatched_bias [H,S,S] fp32 shared by
+ * the batch, or NULL.  w_qkvg [4C][C] bf16 = q, k, v, gating_query rows as
+ * stored by nn.Linear; query_b [C] fp32 or NULL.  head_dim = C/H in {16, 24, 32, 48}.
  * out [B,S,H,head_dim] (= [B,S,C]) in out_dtype: sigmoid(gate) * softmax(..) v.
  */
 size_t af3_batch_diffusion_self_attention_workspace_bytes(int64_t batch, int64_t seq, int channels);
 int af3_batch_diffusion_self_attention_forward(
-    const uint16_t* q_data, const float* key_mask, const float* nonbatched_bias,
+    const uint16_t* q_data, const float* key_mask, int64_t mask_batches, const float* nonbatched_bias,
     const uint16_t* w_qkvg, const float* query_b, int num_head,
     void* out, int out_dtype, int64_t batch, int64_t seq, int channels,
     void* workspace, size_t workspace_bytes, af3_stream_t stream);
@@ -183,6 +185,18 @@ int af3_gathered_cross_attention_forward(
     const uint16_t* w_qg, const uint16_t* w_kv, const float* query_b, int num_head,
     void* out, int out_dtype, int64_t batch, int64_t sq, int64_t sk, int64_t samples, int64_t n_atoms, int channels,
     void* workspace, size_t workspace_bytes, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Batched product c[i] = a[i] b[i]^T, a [batch][m][k], b [batch][n][k],
+ * c [batch][m][n], all bf16 and contiguous, k a multiple of 8.  The triangle
+ * contraction `cik,cjk->cij` of nn/d_triangle_multiplication.py:118-124 for a
+ * pair width other than 128 (the 64-channel Pairformer blocks of the template
+ * embedding, nn/d_template.py:198-201); the 128-channel path has its own kernel
+ * inside af3_triangle_multiplication_forward.
+ */
+int af3_batched_nt_product_forward(
+    const uint16_t* a, const uint16_t* b, uint16_t* c, int64_t batch, int64_t m, int64_t n, int64_t k,
+    af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
  * Pair-logit projection: out[h][i][j] = (LayerNorm(pair)[i][j] . w[h]).
@@ -283,8 +297,8 @@ int af3_grid_attention_core_forward(
  *   B(b,n,k) = b[b*sb + n*ldb + k*kb] (so either operand may be read transposed).
  * af3_check_layer_norm_f32: the fp32 twin of af3_layer_norm_forward.
  * af3_check_elementwise_f32: op 0 triangle-multiplication gating and a/b split
- *   (x0 proj [N*N,256], x1 gate, x2 mask or NULL -> y0 a, y1 b channel-major
- *   [128][N][N]; flag 1 = incoming, stored transposed), op 1 channel-major
+ *   (x0 proj [N*N,2c], x1 gate, x2 mask or NULL -> y0 a, y1 b channel-major
+ *   [c][N][N], c = n1 or 128 if n1 is 0; flag 1 = incoming, stored transposed), op 1 channel-major
  *   [n1][N][N] -> [N][N][n1], op 2 out[j][i][:] = in[i][j][:] with n1 channels,
  *   op 3 SwiGLU y0[m][f] = silu(x0[m][f]) * x0[m][n1 + f] for n0 rows,
  *   op 4 y0 = x0 * x1 (flag 0) or x0 + x1 (flag 1) over n0 elements.
