@@ -168,3 +168,26 @@ def test_per_atom_key_path_matches_the_gathered_key_tensor_path(gpu_pkg):
     fast = mod(act.clone(), qm, q2k, km, cq, ck, pc, cond=cond)
     live = qm[None, ..., None]
     compare("per-atom keys vs gathered keys", ((fast - act) * live).float(), ((plain - act) * live).float(), 2e-3, 3e-2)
+
+
+def test_encoder_without_positions_and_trunk_conditioning(gpu_pkg):
+    """The encoder as the trunk's input embedder uses it (d_alphafold3.py:303-308:
+    no atom positions, no trunk conditioning, 384 token channels, no sample axis)."""
+    g = gen(71)
+    n = 12
+    batch = gpu_pkg.nn.atom_layout.synthetic_batch(n, g, n_padding_tokens=2, chain_len=5)
+    p = {k: O.round_bf16(v) for k, v in H.make_encoder_params(g, 384, False, False, False, std=0.05).items()}
+    want = H.atom_cross_att_encoder(batch, None, None, None, O.cast_params(p, D), batched=False)
+    enc = gpu_pkg.nn.AtomCrossAttEncoder()
+    enc.load_state_dict(p)
+    enc.to(dev())
+    gb = batch.to(dev())
+    for mode, rms_tol, max_tol in (("check", 2e-4, 2e-3), ("bf16", 1e-2, 8e-2)):
+        with gpu_pkg.nn.check_mode(mode == "check"):
+            got = enc(batch=gb, token_atoms_act=None, trunk_single_cond=None, trunk_pair_cond=None)
+        assert got.token_act.shape == (n, 384)
+        compare(f"token_act {mode}", got.token_act, want.token_act, rms_tol, max_tol)
+        compare(f"pair_cond {mode}", got.pair_cond, want.pair_cond, 1e-5, 1e-4)
+        live = want.queries_mask[..., None]
+        compare(f"skip connection {mode}", got.skip_connection.float().cpu() * live, want.skip_connection * live,
+                rms_tol, max_tol)
