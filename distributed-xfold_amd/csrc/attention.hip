@@ -37,6 +37,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t sK[2][KT * LDK];
   __shared__ __attribute__((aligned(16))) bf16_t sVt[2][DVT * 32 * LDV];
   __shared__ __attribute__((aligned(16))) int sCode[2][KT];
+  __shared__ int sAnyCode[2];  // whether any key of the staged tile carries a code
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hh = lane >> 5, j = lane & 31;
@@ -129,8 +130,12 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
         }
       }
     }
-    if (tid < KT)
-      sCode[buf][tid] = (k0_loaded + tid >= a.Sk ? KEY_BEYOND : 0) | (rkm == 0.f ? KEY_MASKED : 0) | (rkp == 0.f ? KEY_PAD : 0);
+    if (tid < KT) {  // wave 0, all of it (KT = 64)
+      const int code = (k0_loaded + tid >= a.Sk ? KEY_BEYOND : 0) | (rkm == 0.f ? KEY_MASKED : 0) | (rkp == 0.f ? KEY_PAD : 0);
+      sCode[buf][tid] = code;
+      const bool any = __any(code != 0);
+      if (tid == 0) sAnyCode[buf] = any ? 1 : 0;
+    }
   };
   // V^T rows that no chunk covers (head dim padding) must read as zero
   for (int idx = tid; idx < 2 * DVT * 32 * LDV; idx += NT) (&sVt[0][0])[idx] = 0;
@@ -141,7 +146,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
   for (int t = 0; t < DVT; ++t)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
-  float m_run = NEG_INF, l_run = 0.f;  // running maximum in base-2 units
+  float m_run = NEG_INF, l_run = 0.f;  // running maximum in natural units
 
   // Pair bias (fp32, one row per query): the 8 quads of a 64-key tile are
   // fetched one tile ahead, unconditionally, from addresses clamped into the
@@ -203,33 +208,45 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
       }
     gload((kt + 1) * KT);
     gload_bias((kt + 1) * KT);
-    // masks from the per-key codes, logits to base 2
+    // Masks from the per-key codes; most tiles carry none (a workgroup-uniform
+    // test skips the block).  The logits stay in natural units: the maximum
+    // does not care, and exp2 takes fma(s, log2 e, -m log2 e).  (For a row
+    // whose keys are all masked every s equals m = -1e9 and the fma leaves the
+    // rounding error of m log2 e, at most 2^6 in magnitude and the same for
+    // every key: the weights stay uniform.)
+    if (__builtin_amdgcn_readfirstlane(sAnyCode[buf])) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int* cp = &sCode[buf][u * 32 + 8 * g + 4 * hh];
-        const int code[4] = {cp[0], cp[1], cp[2], cp[3]};
+        for (int g = 0; g < 4; ++g) {
+          const int* cp = &sCode[buf][u * 32 + 8 * g + 4 * hh];
+          const int code[4] = {cp[0], cp[1], cp[2], cp[3]};
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float v = s[u][4 * g + e];
-          if (code[e] & KEY_MASKED) v = -1e9f;
-          if (q_is_pad && (code[e] & KEY_PAD)) v += 1e9f;
-          v *= LOG2E;
-          if (code[e] & KEY_BEYOND) v = NEG_INF;
-          s[u][4 * g + e] = v;
+          for (int e = 0; e < 4; ++e) {
+            float v = s[u][4 * g + e];
+            if (code[e] & KEY_MASKED) v = -1e9f;
+            if (q_is_pad && (code[e] & KEY_PAD)) v += 1e9f;
+            if (code[e] & KEY_BEYOND) v = NEG_INF;
+            s[u][4 * g + e] = v;
+          }
         }
-      }
-    float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
+    }
+    // maximum of the lane's 32 logits as a tree of three-input maxima
+    float t3[11];
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int g = (u == 0 ? 1 : 0); g < 4; ++g)
-        mx = fmaxf(mx, fmaxf(fmaxf(s[u][4 * g], s[u][4 * g + 1]), fmaxf(s[u][4 * g + 2], s[u][4 * g + 3])));
+    for (int i = 0; i < 10; ++i) {
+      const int e = 3 * i;
+      t3[i] = fmaxf(fmaxf(s[e >> 4][e & 15], s[(e + 1) >> 4][(e + 1) & 15]), s[(e + 2) >> 4][(e + 2) & 15]);
+    }
+    t3[10] = fmaxf(s[1][14], s[1][15]);
+    const float t9a = fmaxf(fmaxf(t3[0], t3[1]), t3[2]), t9b = fmaxf(fmaxf(t3[3], t3[4]), t3[5]);
+    const float t9c = fmaxf(fmaxf(t3[6], t3[7]), t3[8]), t9d = fmaxf(t3[9], t3[10]);
+    float mx = fmaxf(fmaxf(fmaxf(t9a, t9b), t9c), t9d);
     mx = fmaxf(mx, half_swap(xaddr, mx));
     const float m_new = fmaxf(m_run, mx);
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first tile (m_run = -inf, m_new finite)
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);  // 0 on the first tile (m_run = -inf, m_new finite)
     m_run = m_new;
+    const float m2 = m_new * LOG2E;
     bf16x8 pf[2][2];
 #pragma unroll
     for (int u = 0; u < 2; ++u)
@@ -237,7 +254,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
       for (int half = 0; half < 2; ++half) {
         float pv[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(s[u][8 * half + e] - m_new);
+        for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[u][8 * half + e], LOG2E, -m2));
         pf[u][half] = as_frag(pack8(pv));
       }
     // row sums of the ROUNDED probabilities on the matrix unit (ones * P), so
