@@ -409,7 +409,7 @@ int af3_linear_forward(
     const float* gate, int64_t gate_rows, const void* residual, int res_dtype, af3_stream_t stream) {
   if (!x || !w || !y || bad_dtype(y_dtype) || m <= 0 || m > 0x7fffffff || n <= 0 || k <= 0) return AF3_ERR_BAD_ARG;
   if (mode != AF3_LINEAR_PLAIN && mode != AF3_LINEAR_SWIGLU && mode != AF3_LINEAR_GATE_RES &&
-      mode != AF3_LINEAR_REGROUP32)
+      mode != AF3_LINEAR_REGROUP32 && mode != AF3_LINEAR_ROWGATE_RES)
     return AF3_ERR_BAD_ARG;
   if (residual && bad_dtype(res_dtype)) return AF3_ERR_BAD_ARG;
   GemmArgs g;
@@ -417,6 +417,11 @@ int af3_linear_forward(
     if ((m & 31) || (n & 31) || gate || residual) return AF3_ERR_BAD_ARG;
     g.regroup32 = 1;
     mode = AF3_LINEAR_PLAIN;
+  }
+  if (mode == AF3_LINEAR_ROWGATE_RES) {
+    if (!gate || gate_rows <= 0) return AF3_ERR_BAD_ARG;
+    g.gate_per_row = 1;
+    mode = AF3_LINEAR_GATE_RES;
   }
   g.A = x; g.B = w; g.C = y;
   g.M = (int)m; g.N = n; g.K = k;

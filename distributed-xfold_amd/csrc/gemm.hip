@@ -212,7 +212,11 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
       float gt[8], rs[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) { gt[e] = 1.f; rs[e] = 0.f; }
-      if (g.gate) {
+      if (g.gate && g.gate_per_row) {
+        const float f = g.gate[m % g.gate_rows];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) gt[e] = f;
+      } else if (g.gate) {
         const float* gp = g.gate + (int64_t)(m % g.gate_rows) * g.ld_gate + n;
 #pragma unroll
         for (int e = 0; e < 8; ++e) if (e < nv) gt[e] = gp[e];

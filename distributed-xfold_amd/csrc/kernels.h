@@ -21,6 +21,7 @@ struct GemmArgs {
   int seg_len = 0, seg_ops = 0; // SEGMENTED: op of column segment s in bits [4s, 4s+4)
   const float* gate = nullptr;  // GATE_RES: multiply by gate[m % gate_rows][n]
   int gate_rows = 0;
+  int gate_per_row = 0;         // GATE_RES: gate is one factor per row, gate[m % gate_rows]
   int64_t ld_gate = 0;
   const float* res_f32 = nullptr;   // GATE_RES: residual added last (either dtype)
   const bf16_t* res_bf16 = nullptr;

@@ -9,7 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libaf3hip.so")
 
 AF3_BF16, AF3_F32 = 0, 1
-LINEAR_PLAIN, LINEAR_SWIGLU, LINEAR_GATE_RES, LINEAR_REGROUP32 = 0, 2, 3, 4
+LINEAR_PLAIN, LINEAR_SWIGLU, LINEAR_GATE_RES, LINEAR_REGROUP32, LINEAR_ROWGATE_RES = 0, 2, 3, 4, 5
 
 _vp, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 

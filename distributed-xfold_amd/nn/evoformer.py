@@ -71,8 +71,8 @@ class OuterProductMean(HipModule):
         lr = ops.linear(x, p["w_lr"]) * m[..., None].to(torch.bfloat16)            # [a, N, 2 co]
         lt = _pad_last(lr[..., :co].permute(1, 2, 0).reshape(n * co, a)).contiguous()      # [(b, c), a]
         rt = _pad_last(lr[..., co:].permute(1, 2, 0).reshape(n * co, a)).contiguous()      # [(d, e), a]
-        norm = m.t() @ m                                                                   # [b, d]
-        out = residual if residual is not None else torch.empty((n, n, cf), dtype=torch.float32, device=msa.device)
+        inv_norm = (1.0 / (self.epsilon + m.t() @ m)).contiguous()                         # [b, d]
+        out = residual if residual is not None else torch.zeros((n, n, cf), dtype=torch.float32, device=msa.device)
         for b0 in range(0, n, block):
             b1 = min(n, b0 + block)
             if co == 32:
@@ -80,12 +80,10 @@ class OuterProductMean(HipModule):
             else:
                 outer = ops.linear(lt[b0 * co:b1 * co], rt)                                # [(b, c), (d, e)]
                 outer = outer.view(b1 - b0, co, n, co).permute(0, 2, 1, 3).reshape((b1 - b0) * n, co * co)
-            act = ops.linear(outer, p["w_out"], bias=p["b_out"], out_dtype=torch.float32).view(b1 - b0, n, cf)
-            act = act / (self.epsilon + norm[b0:b1, :, None])
-            if residual is not None:
-                out[b0:b1] += act.to(out.dtype)
-            else:
-                out[b0:b1] = act
+            # (outer W + b) / (eps + coverage), added to the pair rows, in the product's epilogue
+            rows = out[b0:b1].view(-1, cf)
+            ops.linear(outer, p["w_out"], bias=p["b_out"], out_dtype=out.dtype, mode=ops._L.LINEAR_ROWGATE_RES,
+                       gate=inv_norm[b0:b1], residual=rows, out=rows)
         return out
 
     def forward(self, msa: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:

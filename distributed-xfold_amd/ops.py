@@ -374,7 +374,12 @@ def linear(x, w, bias=None, out_dtype=torch.bfloat16, mode=_L.LINEAR_PLAIN, alph
     else:
         _gpu(out, "out", None, shape)
     gate_rows = 0
-    if gate is not None:
+    if gate is not None and mode == _L.LINEAR_ROWGATE_RES:
+        _gpu(gate, "gate", torch.float32)
+        gate_rows = gate.numel()
+        if m % gate_rows:
+            raise ValueError("rows must be a multiple of the gate rows")
+    elif gate is not None:
         _gpu(gate, "gate", torch.float32)
         if gate.shape[-1] != n:
             raise ValueError("gate: last dimension must equal the output width")

@@ -242,11 +242,15 @@ int af3_layer_norm_forward(
  *        of 32).  With x = [(token b, channel c), msa row] and w = [(token d,
  *        channel e), msa row] this is the outer-product sum of
  *        nn/d_primitives.py:63-64, laid out for the contraction with output_w.
+ *  mode AF3_LINEAR_ROWGATE_RES: GATE_RES with one factor per row,
+ *        y = residual + gate[m % gate_rows] * (x W^T + bias), gate fp32 [gate_rows]
+ *        (the division by the coverage count of nn/d_primitives.py:69-70)
  */
 #define AF3_LINEAR_PLAIN 0
 #define AF3_LINEAR_SWIGLU 2
 #define AF3_LINEAR_GATE_RES 3
 #define AF3_LINEAR_REGROUP32 4
+#define AF3_LINEAR_ROWGATE_RES 5
 int af3_linear_forward(
     const uint16_t* x, const uint16_t* w, const float* bias,
     void* y, int y_dtype, int64_t m, int n, int k,

@@ -99,7 +99,8 @@ def test_gathered_cross_attention_and_regrouped_store_reject_bad_arguments(pkg):
     # regrouped store: rows of both operands in multiples of 32, no gate / residual
     assert lib.af3_linear_forward(one, one, None, one, 0, 48, 64, 8, 4, 1.0, 0, None, 0, None, 0, None) == -1
     assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 4, 1.0, 0, one, 1, None, 0, None) == -1
-    assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 5, 1.0, 0, None, 0, None, 0, None) == -1
+    assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 5, 1.0, 0, None, 0, None, 0, None) == -1   # row gate missing
+    assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 6, 1.0, 0, None, 0, None, 0, None) == -1   # unknown mode
 
 
 def test_new_modules_share_the_reference_parameter_names(pkg):
