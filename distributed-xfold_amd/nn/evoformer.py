@@ -129,9 +129,7 @@ class MSAAttention(HipModule):
         v = ops.linear(x, p["w_v"])                                                               # [a, k, (h d)]
         gate = ops.linear(x, p["w_g"], sigmoid=True)
         vt = _pad_last(v.view(a, n, h, d).permute(2, 0, 3, 1).reshape(h, a * d, n)).contiguous()  # [h, (row, d), k]
-        avg = torch.empty((h, n, a * d), dtype=torch.bfloat16, device=msa.device)
-        for i in range(h):
-            ops.linear(w[i], vt[i], out=avg[i])                                                   # [q, (row, d)]
+        avg = ops.batched_nt_product(w, vt)                                                       # [h, q, (row, d)]
         avg = avg.view(h, n, a, d).permute(2, 1, 0, 3).reshape(a, n, c) * gate
         if residual:
             return ops.linear(avg, p["w_o"], out_dtype=msa.dtype, mode=ops._L.LINEAR_GATE_RES, residual=msa, out=msa)
