@@ -245,6 +245,11 @@ int af3_batch_diffusion_self_attention_forward(
   return launch_flash_attention(f, s);
 }
 
+// -------------------------------------------------------------------- transpose
+int af3_transpose_bf16_forward(const uint16_t* in, uint16_t* out, int64_t rows, int64_t cols, af3_stream_t stream) {
+  return launch_transpose(in, out, rows, cols, static_cast<hipStream_t>(stream));
+}
+
 // ------------------------------------------------------------ batched NT product
 int af3_batched_nt_product_forward(
     const uint16_t* a, const uint16_t* b, uint16_t* c, int64_t batch, int64_t m, int64_t n, int64_t k,

@@ -54,6 +54,8 @@ struct RowNormArgs {
   int param_vec = 0, cond_vec = 0;  // set by launch_row_norm: arrays aligned for 16-byte loads
 };
 int launch_row_norm(const RowNormArgs& a, hipStream_t stream);
+// out[c][r] = in[r][c], bf16, rows and cols multiples of 8
+int launch_transpose(const bf16_t* in, bf16_t* out, int64_t rows, int64_t cols, hipStream_t stream);
 
 // -------------------------------------------------------------- pair_tile.hip
 // Residual-stream tensors (`pair`, `out`, `x`) are bf16 or fp32 (io_f32).

@@ -152,3 +152,48 @@ int launch_row_norm(const RowNormArgs& a_in, hipStream_t stream) {
   else hipLaunchKernelGGL(ln_rows_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, a);
   return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }
+
+// ------------------------------------------------------------------ transpose
+// out[c][r] = in[r][c] for a bf16 matrix, 64 x 64 tiles through LDS: 16-byte
+// loads along the input rows, 16-byte stores along the output rows.  (The dense
+// kernels want the summation index innermost in both operands; the MSA
+// operators sum over MSA rows or tokens, which the activations carry as outer
+// indices.)
+namespace {
+constexpr int TT = 64, TLD = TT + 2;  // 33 dwords per row: the column reads of a wave spread over the banks
+
+__global__ __launch_bounds__(256) void transpose_kernel(const bf16_t* in, bf16_t* out, int64_t rows, int64_t cols) {
+  __shared__ bf16_t tile[TT * TLD];
+  const int tid = threadIdx.x;
+  const int64_t tiles_c = (cols + TT - 1) / TT;
+  const int64_t r0 = (blockIdx.x / tiles_c) * TT, c0 = (blockIdx.x % tiles_c) * TT;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int idx = tid + 256 * i, r = idx >> 3, ch = (idx & 7) * 8;
+    u32x4 v = {0, 0, 0, 0};
+    if (r0 + r < rows && c0 + ch < cols) v = *reinterpret_cast<const u32x4*>(in + (r0 + r) * cols + c0 + ch);
+    uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[r * TLD + ch]);  // rows are 4-byte aligned only
+    dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int idx = tid + 256 * i, c = idx >> 3, rh = (idx & 7) * 8;
+    if (c0 + c >= cols || r0 + rh >= rows) continue;
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      w[e] = (uint32_t)tile[(rh + 2 * e) * TLD + c] | ((uint32_t)tile[(rh + 2 * e + 1) * TLD + c] << 16);
+    *reinterpret_cast<u32x4*>(out + (c0 + c) * rows + r0 + rh) = u32x4{w[0], w[1], w[2], w[3]};
+  }
+}
+}  // namespace
+
+int launch_transpose(const bf16_t* in, bf16_t* out, int64_t rows, int64_t cols, hipStream_t stream) {
+  if (!in || !out || rows <= 0 || cols <= 0 || (rows & 7) || (cols & 7)) return AF3_ERR_BAD_ARG;
+  if (((uintptr_t)in & 15) || ((uintptr_t)out & 15)) return AF3_ERR_BAD_ARG;
+  const int64_t blocks = ((rows + TT - 1) / TT) * ((cols + TT - 1) / TT);
+  if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, in, out, rows, cols);
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}

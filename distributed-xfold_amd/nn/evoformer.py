@@ -15,6 +15,10 @@ kernels:
     exists as a whole and nothing is permuted.
   * pair-weighted averaging: per head, softmax(pair logits) [q, k] times the
     head's values of all MSA rows [(row, channel), k]^T.
+Both sum over an index (MSA rows, tokens) that the activations [rows, N, c]
+carry as an outer one, while the dense kernels want it innermost: the operands
+are produced transposed (projection weights as the left operand) or run through
+the bf16 transpose kernel, not through strided copies.
 """
 
 from __future__ import annotations
@@ -57,7 +61,7 @@ class OuterProductMean(HipModule):
     def _pack(self):
         co = self.num_outer_channel
         return dict(ln_w=f32(self.layer_norm_input.weight), ln_b=f32(self.layer_norm_input.bias),
-                    w_lr=bf16(torch.cat([self.left_projection.weight, self.right_projection.weight], dim=0)),
+                    w_l=bf16(self.left_projection.weight), w_r=bf16(self.right_projection.weight),
                     w_out=bf16(self.output_w.detach().reshape(co * co, -1).t()), b_out=f32(self.output_b))
 
     @torch.no_grad()
@@ -68,9 +72,14 @@ class OuterProductMean(HipModule):
         co, cf = self.num_outer_channel, self.num_output_channel
         m = mask.float()
         x = ops.layer_norm(msa.contiguous(), p["ln_w"], p["ln_b"])
-        lr = ops.linear(x, p["w_lr"]) * m[..., None].to(torch.bfloat16)            # [a, N, 2 co]
-        lt = _pad_last(lr[..., :co].permute(1, 2, 0).reshape(n * co, a)).contiguous()      # [(b, c), a]
-        rt = _pad_last(lr[..., co:].permute(1, 2, 0).reshape(n * co, a)).contiguous()      # [(d, e), a]
+        mb = m[..., None].to(torch.bfloat16)
+
+        def projected(w):        # [(token, channel), MSA row]: the summation index innermost
+            y = ops.linear(x, w) * mb                                                       # [a, N, co]
+            if a % 8 == 0 and (n * co) % 8 == 0:
+                return ops.transpose2d(y.view(a, n * co))
+            return _pad_last(y.permute(1, 2, 0).reshape(n * co, a)).contiguous()
+        lt, rt = projected(p["w_l"]), projected(p["w_r"])
         inv_norm = (1.0 / (self.epsilon + m.t() @ m)).contiguous()                         # [b, d]
         out = residual if residual is not None else torch.zeros((n, n, cf), dtype=torch.float32, device=msa.device)
         for b0 in range(0, n, block):
@@ -126,11 +135,22 @@ class MSAAttention(HipModule):
         logits = ops.pair_logits(pair.contiguous(), p["pn_w"], p["pn_b"], p["w_logits"], h)     # [h, q, k] fp32
         logits += 1e9 * (msa_mask.float().max(dim=0).values - 1.0)
         w = _pad_last(torch.softmax(logits, dim=-1).to(torch.bfloat16)).contiguous()              # [h, q, k]
-        v = ops.linear(x, p["w_v"])                                                               # [a, k, (h d)]
-        gate = ops.linear(x, p["w_g"], sigmoid=True)
-        vt = _pad_last(v.view(a, n, h, d).permute(2, 0, 3, 1).reshape(h, a * d, n)).contiguous()  # [h, (row, d), k]
-        avg = ops.batched_nt_product(w, vt)                                                       # [h, q, (row, d)]
-        avg = avg.view(h, n, a, d).permute(2, 1, 0, 3).reshape(a, n, c) * gate
+        if n % 8 == 0 and (a * n) % 8 == 0 and c % 8 == 0:
+            # Everything with the tokens innermost: the value and gate projections are taken
+            # transposed (weights as the left operand), [(h, d), (row, k)], which is per head the
+            # k-contiguous right operand of the averaging product; its result [(h, d), (row, q)]
+            # has the same layout, takes the gate there and is transposed once for the output projection.
+            x2 = x.view(a * n, c)
+            v_t = ops.linear(p["w_v"], x2)                                                        # [(h d), (row, k)]
+            gate_t = ops.linear(p["w_g"], x2, sigmoid=True)
+            avg_t = ops.batched_nt_product(v_t.view(h, d * a, n), w)                              # [h, (d, row), q]
+            avg = ops.transpose2d(avg_t.view(c, a * n) * gate_t).view(a, n, c)
+        else:
+            v = ops.linear(x, p["w_v"])                                                           # [a, k, (h d)]
+            gate = ops.linear(x, p["w_g"], sigmoid=True)
+            vt = _pad_last(v.view(a, n, h, d).permute(2, 0, 3, 1).reshape(h, a * d, n)).contiguous()
+            avg = ops.batched_nt_product(w, vt)                                                   # [h, q, (row, d)]
+            avg = avg.view(h, n, a, d).permute(2, 1, 0, 3).reshape(a, n, c) * gate
         if residual:
             return ops.linear(avg, p["w_o"], out_dtype=msa.dtype, mode=ops._L.LINEAR_GATE_RES, residual=msa, out=msa)
         return ops.linear(avg, p["w_o"], out_dtype=msa.dtype)

@@ -282,6 +282,19 @@ def gathered_cross_attention(q_data, atom_data, key_rows, pair_logits, mask_q, m
     return out
 
 
+def transpose2d(x):
+    """out[c, r] = x[r, c] for a contiguous bf16 GPU matrix (af3_transpose_bf16_forward);
+    both sizes multiples of 8."""
+    lib = _L.load()
+    _gpu(x, "x", torch.bfloat16)
+    if x.dim() != 2 or x.shape[0] % 8 or x.shape[1] % 8:
+        raise ValueError("expected a 2-D tensor with both sizes multiples of 8")
+    out = torch.empty((x.shape[1], x.shape[0]), dtype=torch.bfloat16, device=x.device)
+    rc = lib.af3_transpose_bf16_forward(_p(x), _p(out), x.shape[0], x.shape[1], _stream(x.device))
+    _L.check(rc, "af3_transpose_bf16_forward")
+    return out
+
+
 def batched_nt_product(a, b, out=None):
     """out[i] = a[i] @ b[i].T for a [batch, m, k], b [batch, n, k] bf16 (af3_batched_nt_product_forward)."""
     lib = _L.load()

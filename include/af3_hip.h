@@ -199,6 +199,15 @@ int af3_batched_nt_product_forward(
     af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * out[c][r] = in[r][c] for a contiguous bf16 matrix [rows][cols], rows and cols
+ * multiples of 8.  The MSA operators sum over MSA rows (outer-product mean,
+ * nn/d_primitives.py:63) or tokens (pair-weighted averaging, nn/d_attention.py:
+ * 137), which their activations [rows, N, c] carry as outer indices; the dense
+ * kernels want the summation index innermost in both operands.
+ */
+int af3_transpose_bf16_forward(const uint16_t* in, uint16_t* out, int64_t rows, int64_t cols, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Pair-logit projection: out[h][i][j] = (LayerNorm(pair)[i][j] . w[h]).
  * Replaces the eager `single_pair_logits_projection(single_pair_logits_norm(
  * pair)).permute(2,0,1)` of nn/d_pairformer.py:160-162 and the

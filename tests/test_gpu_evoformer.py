@@ -51,7 +51,7 @@ def inputs(a, n, seed, std=0.05):
 MODES = (("check", 2e-4, 2e-3), ("bf16", 1e-2, 8e-2))
 
 
-@pytest.mark.parametrize("a,n", [(5, 12), (37, 45)])
+@pytest.mark.parametrize("a,n", [(5, 12), (37, 45), (16, 24)])   # the last one takes the transposed-operand paths
 def test_msa_operators_against_oracle(gpu_pkg, a, n):
     g, p, msa, pair, mm, pm = inputs(a, n, 70 + n)
     pd = O.cast_params(p, D)
@@ -74,7 +74,7 @@ def test_msa_operators_against_oracle(gpu_pkg, a, n):
             compare(f"msa attention {mode}", att(t(msa), t(mm), t(pair)), want_att, rms_tol, max_tol)
 
 
-@pytest.mark.parametrize("a,n", [(6, 17), (20, 40)])
+@pytest.mark.parametrize("a,n", [(6, 17), (20, 40), (8, 16)])
 def test_evoformer_block_against_oracle(gpu_pkg, a, n):
     g, p, msa, pair, mm, pm = inputs(a, n, 80 + n)
     pd = O.cast_params(p, D)
@@ -113,3 +113,12 @@ def test_full_size_block_against_check_mode(gpu_pkg):
     compare("msa attention, bf16 vs fp32 check", blk.msa_attention1(t(msa), t(mm), t(pair)), want_att, 1e-2, 8e-2)
     got_msa, got_pair = blk(t(msa).clone(), t(pair).clone(), t(mm), t(pm))
     assert torch.isfinite(got_msa).all() and torch.isfinite(got_pair).all()
+
+
+@pytest.mark.parametrize("rows,cols", [(8, 8), (72, 200), (64, 4096), (1000, 24)])
+def test_transpose_is_exact(gpu_pkg, rows, cols):
+    x = torch.randn(rows, cols, generator=gen(rows + cols)).bfloat16().to(dev())
+    y = gpu_pkg.ops.transpose2d(x)
+    assert y.shape == (cols, rows) and torch.equal(y, x.t().contiguous())
+    with pytest.raises(ValueError):
+        gpu_pkg.ops.transpose2d(x[:, :cols - 1].contiguous() if cols > 8 else x[:7].contiguous())
