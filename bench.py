@@ -59,6 +59,23 @@ def flops_attention_core(n):  # QK^T and PV for N rows x 4 heads x d=32
     return 512.0 * n ** 3
 
 
+def random_init_(module, gen, std=0.02):
+    """Random-init weights for timing: every matrix and bias N(0, std), every
+    LayerNorm weight (and the other 1-D `weight` vectors) 1 + N(0, std).  Only
+    bench.py's cpu_baseline leg touches the CPU oracle; the timed modules get
+    their parameters here."""
+    import torch
+    with torch.no_grad():
+        for name, p in module.named_parameters():
+            noise = torch.randn(p.shape, generator=gen) * std
+            if p.dim() == 1 and name.endswith("weight"):
+                noise += 1.0
+            p.copy_(noise)
+    if hasattr(module, "invalidate"):
+        module.invalidate()
+    return module
+
+
 def gpu_time_ms(fn, iters, warmup=2, warm_ms=0.0):
     """Average duration of fn() in ms, timed with HIP events on torch's current
     stream (the stream handed to the C ABI).  `warm_ms`: keep launching untimed
@@ -121,11 +138,8 @@ def diffusion_step(pkg, n, dev, samples=5, iters=20):
     random-init weights; the per-batch conditioning is computed once, as the
     sampler does, and timed separately."""
     import torch
-    from oracle import af3_head_oracle as H     # parameter generator only
     g = torch.Generator().manual_seed(1)
-    head = pkg.nn.DiffusionHead()
-    head.load_state_dict(H.make_diffusion_head_params(g))
-    head = head.to(dev)
+    head = random_init_(pkg.nn.DiffusionHead(), g).to(dev)
     head.load_hip_params()
     batch = pkg.nn.atom_layout.synthetic_batch(n, g, n_padding_tokens=n // 10).to(dev)
     emb = {"single": torch.randn(n, 384, generator=g).to(dev), "pair": torch.randn(n, n, 128, generator=g).to(dev),
@@ -157,11 +171,8 @@ def evoformer_block_ms(pkg, n, dev, rows=1024, iters=10):
     """One Evoformer (MSA) block: outer-product mean, MSA pair-weighted
     averaging, MSA transition and the five pair operators, bf16 streams."""
     import torch
-    from oracle import af3_msa_oracle as M      # parameter generator only
     g = torch.Generator().manual_seed(2)
-    blk = pkg.nn.EvoformerBlock()
-    blk.load_state_dict(M.make_evoformer_block_params(g))
-    blk = blk.to(dev)
+    blk = random_init_(pkg.nn.EvoformerBlock(), g).to(dev)
     blk.load_hip_params()
     msa = torch.randn(rows, n, 64, generator=g).to(dev).bfloat16()
     pair = torch.randn(n, n, 128, generator=g).to(dev).bfloat16()
@@ -181,11 +192,8 @@ def trunk_recycle_ms(pkg, n, dev, rows=1024, iters=3):
     """One recycling pass of the Evoformer trunk: input embeddings, 4 Evoformer
     (MSA) blocks, 48 Pairformer blocks (no template embedding), bf16 streams."""
     import torch
-    from oracle import af3_trunk_oracle as T     # parameter generator only
     g = torch.Generator().manual_seed(3)
-    mod = pkg.nn.Evoformer()
-    mod.load_state_dict(T.make_evoformer_params(g))
-    mod = mod.to(dev)
+    mod = random_init_(pkg.nn.Evoformer(), g).to(dev)
     mod.load_hip_params()
     batch = pkg.nn.atom_layout.synthetic_trunk_batch(n, rows, g, n_padding_tokens=n // 10).to(dev)
     tf = torch.randn(n, 447, generator=g).to(dev)
@@ -220,7 +228,6 @@ def main():
     import __graft_entry__ as ge
     pkg = ge.load_package()
     pkg.lib.load()                       # raises if the HIP library is missing
-    from oracle import af3_oracle as O   # parameter generator + CPU baseline only
 
     dev = torch.device("cuda:0")
     n = args.n_token
@@ -231,9 +238,7 @@ def main():
         return
     io = torch.bfloat16 if args.io == "bf16" else torch.float32
     g = torch.Generator().manual_seed(0)
-    blk = pkg.nn.PairformerBlock()
-    blk.load_state_dict(O.make_pairformer_block_params(g))
-    blk = blk.to(dev)
+    blk = random_init_(pkg.nn.PairformerBlock(), g).to(dev)
     blk.load_hip_params()
     pair = torch.randn(n, n, 128, generator=g).to(dev).to(io)
     single = torch.randn(n, 384, generator=g).to(dev).to(io)
