@@ -19,12 +19,17 @@ struct Tile {
   __device__ __forceinline__ bool valid(int p) const { return r0 + p < N; }
 };
 
-__device__ __forceinline__ Tile make_tile(int N, bool column_mode) {
+// `reverse`: walk the tiles from the last to the first.  A kernel that reads
+// what the previous kernel has just written (and whose output the next kernel
+// starts reading from the other end) finds the most recently written part
+// still in the last-level cache when it starts there.
+__device__ __forceinline__ Tile make_tile(int N, bool column_mode, bool reverse = false) {
   const int tiles_r = (N + TM - 1) / TM;
   Tile t;
   t.N = N;
-  t.o = blockIdx.x / tiles_r;
-  t.r0 = (blockIdx.x % tiles_r) * TM;
+  const unsigned bid = reverse ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
+  t.o = bid / tiles_r;
+  t.r0 = (bid % tiles_r) * TM;
   t.so = column_mode ? 1 : N;
   t.sr = column_mode ? N : 1;
   return t;
