@@ -229,15 +229,18 @@ __global__ __launch_bounds__(256, 3) void triattn_flash_kernel(TriAttnArgs a) {
   const int xaddr = half_swap_addr();
   const int N = a.N;
   const int QT = (N + QW - 1) / QW;
-  // XCD-aware remap: physical id -> (xcd, slot) -> logical id; logical order is
-  // (head, row, query tile) with the query tile fastest.
-  const int total = H * N * QT;
-  const int per_xcd = (total + 7) / 8;
-  const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (logical >= total) return;
-  const int qt = logical % QT;
-  const int b = (logical / QT) % N;
-  const int h = logical / (QT * N);
+  // Workgroup ids are dealt round-robin to the 8 XCDs.  The query tiles of one
+  // (row, head) share its K / V and run back to back on one XCD (id = slot * 8 +
+  // xcd, query tile fastest within the XCD's slots); the (row, head) pairs
+  // themselves are dealt to the XCDs in turn, rows ascending, so that the whole
+  // chip moves through the rows together, starting with the ones the
+  // projection kernel wrote last.
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int qt = slot % QT;
+  const int pair_idx = (slot / QT) * 8 + xcd;
+  if (pair_idx >= H * N) return;
+  const int b = pair_idx / H;
+  const int h = pair_idx % H;
   const int q0 = qt * QW;
   const int qw = q0 + wave * 32 + j;
   const int qi = min(qw, N - 1);
@@ -521,8 +524,7 @@ int launch_triattn_flash(const TriAttnArgs& a, hipStream_t stream) {
   if (!a.q || !a.k || !a.vt || !a.g || !a.og || a.N <= 0) return AF3_ERR_BAD_ARG;
   if (a.ldn < a.N || (a.ldn & 7)) return AF3_ERR_BAD_ARG;
   if (!al16(a.q) || !al16(a.k) || !al16(a.vt) || !al16(a.g) || !al16(a.og) || !al16(a.bias)) return AF3_ERR_BAD_ARG;
-  const int64_t total = (int64_t)((a.N + QW - 1) / QW) * H * a.N;
-  const int64_t blocks = (total + 7) / 8 * 8;
+  const int64_t blocks = ((int64_t)H * a.N + 7) / 8 * 8 * ((a.N + QW - 1) / QW);
   if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
   if (a.bias) hipLaunchKernelGGL(triattn_flash_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
   else hipLaunchKernelGGL(triattn_flash_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
