@@ -261,7 +261,7 @@ int af3_batched_nt_product_forward(
   g.M = (int)m; g.N = (int)n; g.K = (int)k; g.batch = (int)batch;
   g.lda = g.ldb = k; g.ldc = n;
   g.sA = m * k; g.sB = n * k; g.sC = m * n;
-  return launch_gemm_nt(g, static_cast<hipStream_t>(stream));
+  return contraction(g, static_cast<hipStream_t>(stream));
 }
 
 // --------------------------------------------------- windowed (atom) cross-attention

@@ -1,5 +1,8 @@
 // Triangle contraction on bf16 MFMA:  T[c][i][j] = sum_k A[c][i][k] * B[c][j][k]
-// for a batch of channels c, bf16 in and out, fp32 accumulation.
+// for a batch of channels c, bf16 in and out, fp32 accumulation.  The same
+// kernel, with a per-column or SwiGLU epilogue, takes the large dense
+// projections (x W^T with thousands of rows and columns) of the diffusion
+// transformer and the outer-product mean.
 //
 // Both operands are k-contiguous (the natural fragment order of
 // v_mfma_f32_32x32x16_bf16).  The tile is as large as the register file
@@ -67,6 +70,15 @@ __device__ __forceinline__ void wait_loads_but() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x70);
 }
 
+// MODE 0: plain bf16 product (the triangle contraction).
+// MODE 1: per-column epilogue of the dense projections, (acc + bias) * alpha
+//         and / or a sigmoid, uniform over the tile or chosen per segment of
+//         seg_len columns, and optionally the 32x32-regrouped output order.
+// MODE 2: SwiGLU, weight rows packed in blocks of 64 (32 "a" rows, then the 32
+//         matching "b" rows): output column 32 p + x = silu(a) * b of block p.
+enum { BIG_PLAIN = 0, BIG_COLUMN_OPS = 1, BIG_SWIGLU = 2 };
+
+template <int MODE>
 __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   // Four arrays, not one: the compiler then knows that a load in flight to one
   // buffer cannot alias a fragment read from another and does not make the
@@ -245,26 +257,81 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
   bf16_t* sE = reinterpret_cast<bf16_t*>(buf(wave));
+  // Values are finished four at a time on their way from the accumulators to
+  // LDS, so that few of them are live at once.
+  constexpr int JSTEP = MODE == BIG_SWIGLU ? 2 : 1;  // SwiGLU: tiles (0,1) and (2,3) give 32 output columns each
 #pragma unroll
-  for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-    for (int it = 0; it < 4; ++it)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        u32x2 v;
-        v.x = pack2bf(acc[jt][it][4 * q], acc[jt][it][4 * q + 1]);
-        v.y = pack2bf(acc[jt][it][4 * q + 2], acc[jt][it][4 * q + 3]);
-        *reinterpret_cast<u32x2*>(sE + (32 * it + l31) * LDE + 32 * jt + 8 * q + 4 * hh) = v;
+  for (int jt = 0; jt < 4; jt += JSTEP) {
+    // column ops: a 32-column block never straddles segments (seg_len % 32 == 0)
+    bool affine = false, sig = false;
+    float alpha = 1.f;
+    const int nb = n0 + wn + 32 * jt;
+    if constexpr (MODE == BIG_COLUMN_OPS) {
+      int op = SEG_BIAS_SCALE;
+      sig = g.act_sigmoid != 0;
+      if (g.epi == EPI_SEGMENTED) {
+        op = (g.seg_ops >> (4 * (min(nb, g.N - 1) / g.seg_len))) & 15;
+        sig = op == SEG_SIGMOID;
       }
-  bf16_t* C = reinterpret_cast<bf16_t*>(g.C) + (int64_t)bz * g.sC;
-  const int c16 = lane & 15, rsub = lane >> 4;  // 16 chunks of 8 columns per row, 4 rows per instruction
-  const int col = n0 + wn + c16 * 8;
+      affine = op == SEG_BIAS_SCALE;
+      if (affine) alpha = g.alpha;
+    }
 #pragma unroll
-  for (int s = 0; s < 32; ++s) {
-    const int r = 4 * s + rsub;
-    const int row = m0 + wm + r;
-    const u32x4 v = *reinterpret_cast<const u32x4*>(sE + r * LDE + c16 * 8);
-    if (row < g.M && col < g.ldc) *reinterpret_cast<u32x4*>(C + (int64_t)row * g.ldc + col) = v;
+    for (int q = 0; q < 4; ++q) {
+      float bb[4] = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (MODE == BIG_COLUMN_OPS) {
+        if (affine && g.bias) {
+          const f32x4 b = *reinterpret_cast<const f32x4*>(g.bias + min(nb + 8 * q + 4 * hh, g.N - 4));
+          bb[0] = b.x; bb[1] = b.y; bb[2] = b.z; bb[3] = b.w;
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float v = acc[jt][it][4 * q + e];
+          if constexpr (MODE == BIG_COLUMN_OPS) {
+            v = (v + bb[e]) * alpha;
+            if (sig) v = sigmoidf_(v);
+          }
+          if constexpr (MODE == BIG_SWIGLU) v = v * sigmoidf_(v) * acc[jt + 1][it][4 * q + e];
+          o[e] = v;
+        }
+        u32x2 v2;
+        v2.x = pack2bf(o[0], o[1]);
+        v2.y = pack2bf(o[2], o[3]);
+        *reinterpret_cast<u32x2*>(sE + (32 * it + l31) * LDE + 32 * (jt / JSTEP) + 8 * q + 4 * hh) = v2;
+      }
+    }
+  }
+  bf16_t* C = reinterpret_cast<bf16_t*>(g.C) + (int64_t)bz * g.sC;
+  if constexpr (MODE == BIG_SWIGLU) {
+    const int c8 = lane & 7, rsub = lane >> 3;  // 8 chunks of 8 output columns per row, 8 rows per instruction
+    const int col = (n0 + wn) / 2 + c8 * 8;
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+      const int r = 8 * s + rsub;
+      const int row = m0 + wm + r;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(sE + r * LDE + c8 * 8);
+      if (row < g.M && col < g.N / 2) *reinterpret_cast<u32x4*>(C + (int64_t)row * g.ldc + col) = v;
+    }
+  } else {
+    const int c16 = lane & 15, rsub = lane >> 4;  // 16 chunks of 8 columns per row, 4 rows per instruction
+    const int col = n0 + wn + c16 * 8;
+    const int col_end = MODE == BIG_PLAIN ? g.ldc : g.N;
+#pragma unroll
+    for (int s = 0; s < 32; ++s) {
+      const int r = 4 * s + rsub;
+      const int row = m0 + wm + r;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(sE + r * LDE + c16 * 8);
+      if (row < g.M && col < col_end) {
+        int64_t off = (int64_t)row * g.ldc + col;
+        if (MODE == BIG_COLUMN_OPS && g.regroup32)
+          off = (((int64_t)(row >> 5) * (g.N >> 5) + (col >> 5)) * 32 + (row & 31)) * 32 + (col & 31);
+        *reinterpret_cast<u32x4*>(C + off) = v;
+      }
+    }
   }
 }
 
@@ -272,21 +339,49 @@ bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 }  // namespace
 
-// Plain bf16 batched NT product with the large tile; false if the operands do
-// not meet its layout assumptions (the caller then takes the general GEMM).
-bool contract_supported(const GemmArgs& g) {
-  return g.epi == EPI_PLAIN && !g.out_f32 && !g.bias && !g.act_sigmoid && g.alpha == 1.f && g.M > 0 && g.N > 0 &&
-         g.K > 0 && g.batch > 0 && (g.lda & 7) == 0 && (g.ldb & 7) == 0 && (g.ldc & 7) == 0 && (g.K & 7) == 0 &&
-         g.K <= g.lda && g.K <= g.ldb && g.ldc >= ((g.N + 7) & ~7) && (g.sA & 7) == 0 && (g.sB & 7) == 0 &&
+// Layout assumptions the large tile shares over its modes.
+static bool big_tile_layout_ok(const GemmArgs& g) {
+  return !g.out_f32 && g.M > 0 && g.N > 0 && g.K > 0 && g.batch > 0 && (g.lda & 7) == 0 && (g.ldb & 7) == 0 &&
+         (g.ldc & 7) == 0 && (g.K & 7) == 0 && g.K <= g.lda && g.K <= g.ldb && (g.sA & 7) == 0 && (g.sB & 7) == 0 &&
          (g.sC & 7) == 0 && al16(g.A) && al16(g.B) && al16(g.C) &&
          (int64_t)g.M * g.lda < (1ll << 30) && (int64_t)g.N * g.ldb < (1ll << 30);
 }
 
-int launch_contract(const GemmArgs& g, hipStream_t stream) {
-  if (!g.A || !g.B || !g.C || !contract_supported(g)) return AF3_ERR_BAD_ARG;
+// Plain bf16 batched NT product with the large tile; false if the operands do
+// not meet its layout assumptions (the caller then takes the general GEMM).
+bool contract_supported(const GemmArgs& g) {
+  return g.epi == EPI_PLAIN && !g.bias && !g.act_sigmoid && g.alpha == 1.f && !g.regroup32 && !g.gate &&
+         big_tile_layout_ok(g) && g.ldc >= ((g.N + 7) & ~7);
+}
+
+// Which large-tile instance can take this product with its epilogue: -1 = none.
+int big_tile_mode(const GemmArgs& g) {
+  if (!big_tile_layout_ok(g) || g.gate || g.res_f32 || g.res_bf16) return -1;
+  if (g.epi == EPI_SWIGLU) return (g.N & 63) == 0 && g.ldc >= g.N / 2 && !g.regroup32 ? BIG_SWIGLU : -1;
+  if (g.N & 7) return -1;
+  if (!g.regroup32 && g.ldc < g.N) return -1;
+  if (g.bias && !al16(g.bias)) return -1;
+  if (g.epi == EPI_SEGMENTED) return g.seg_len > 0 && (g.seg_len & 31) == 0 && !g.regroup32 ? BIG_COLUMN_OPS : -1;
+  if (g.epi != EPI_PLAIN) return -1;
+  if (g.regroup32) return g.batch == 1 && (g.M & 31) == 0 && (g.N & 31) == 0 ? BIG_COLUMN_OPS : -1;
+  return (g.bias || g.act_sigmoid || g.alpha != 1.f) ? BIG_COLUMN_OPS : BIG_PLAIN;
+}
+
+int launch_big_tile(const GemmArgs& g, int mode, hipStream_t stream) {
+  if (!g.A || !g.B || !g.C) return AF3_ERR_BAD_ARG;
+  if (mode != big_tile_mode(g) && !(mode == BIG_PLAIN && contract_supported(g))) return AF3_ERR_BAD_ARG;
+  if (mode < BIG_PLAIN || mode > BIG_SWIGLU) return AF3_ERR_BAD_ARG;
   const int64_t total = (int64_t)((g.M + CM - 1) / CM) * ((g.N + CN - 1) / CN) * g.batch;
   const int64_t blocks = (total + 7) / 8 * 8;
   if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
-  hipLaunchKernelGGL(contract_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, g);
+  const dim3 grid((unsigned)blocks), block(256);
+  if (mode == BIG_PLAIN) hipLaunchKernelGGL(contract_kernel<BIG_PLAIN>, grid, block, 0, stream, g);
+  else if (mode == BIG_COLUMN_OPS) hipLaunchKernelGGL(contract_kernel<BIG_COLUMN_OPS>, grid, block, 0, stream, g);
+  else hipLaunchKernelGGL(contract_kernel<BIG_SWIGLU>, grid, block, 0, stream, g);
   return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+int launch_contract(const GemmArgs& g, hipStream_t stream) {
+  if (!g.A || !g.B || !g.C || !contract_supported(g)) return AF3_ERR_BAD_ARG;
+  return launch_big_tile(g, BIG_PLAIN, stream);
 }

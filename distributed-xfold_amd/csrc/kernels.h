@@ -36,6 +36,11 @@ int launch_gemm_nt(const GemmArgs& g, hipStream_t stream);
 // contract.hip: the same product, plain bf16 output, 256x256 tiles (large M, N)
 bool contract_supported(const GemmArgs& g);
 int launch_contract(const GemmArgs& g, hipStream_t stream);
+// the 256x256 tile with the epilogues of the dense projections (bias / scale /
+// sigmoid per column segment, SwiGLU, regrouped output): big_tile_mode names the
+// kernel instance that can take `g`, or -1
+int big_tile_mode(const GemmArgs& g);
+int launch_big_tile(const GemmArgs& g, int mode, hipStream_t stream);
 
 // ---------------------------------------------------------------- rowops.hip
 // y = LN(x) [* weight + bias] ; then, if scale: y = sigmoid(scale[r]) * y + shift[r]

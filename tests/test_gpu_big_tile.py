@@ -1,0 +1,112 @@
+"""GPU parity of the dense projections at sizes that take the 256x256-tile
+kernel (at least 160 such tiles): plain / bias / scale / sigmoid, SwiGLU, the
+regrouped store and the segmented q-k-v-gate projection of the diffusion
+self-attention, against float64 products of the same bf16 operands.  Ragged
+M (not a multiple of 256), N (a partial last tile) and K (not a multiple of
+the 32-deep slab) are part of every case."""
+
+import pytest
+import torch
+
+from oracle import af3_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def within_bf16_ulp(name, got, want, ulps=1.01, atol=1e-4):
+    got, want = got.detach().double().cpu(), want.double()
+    bad = (got - want).abs() > ulps * 2.0 ** -8 * want.abs() + atol
+    assert not bad.any(), f"{name}: {int(bad.sum())} elements beyond {ulps} bf16 ulp"
+
+
+@pytest.mark.parametrize("m,n,k", [(3850, 2824, 200), (4096, 2560, 768)])
+def test_linear_bias_scale_sigmoid(gpu_pkg, m, n, k):
+    print(f"test_linear_bias_scale_sigmoid m={m} n={n} k={k}", flush=True)
+    g = gen(m + n + k)
+    x, w = O.round_bf16(torch.randn(m, k, generator=g)), O.round_bf16(torch.randn(n, k, generator=g) * 0.1)
+    b = torch.randn(n, generator=g)
+    xd, wd = x.to(dev()).bfloat16(), w.to(dev()).bfloat16()
+    y = x.double() @ w.double().T
+    got = gpu_pkg.ops.linear(xd, wd)
+    within_bf16_ulp("plain", got, y)
+    got = gpu_pkg.ops.linear(xd, wd, bias=b.to(dev()), alpha=0.5)
+    within_bf16_ulp("bias, scale", got, (y + b.double()) * 0.5)
+    got = gpu_pkg.ops.linear(xd, wd, sigmoid=True)
+    within_bf16_ulp("sigmoid", got, torch.sigmoid(y))
+    # the same products from the 128x128-tile kernel (fp32 output is not a large-tile case)
+    ref = gpu_pkg.ops.linear(xd, wd, bias=b.to(dev()), alpha=0.5, out_dtype=torch.float32)
+    got = gpu_pkg.ops.linear(xd, wd, bias=b.to(dev()), alpha=0.5)
+    assert torch.equal(got, ref.bfloat16()) or float((got.float() - ref).abs().max()) <= 2.0 ** -7 * float(ref.abs().max())
+
+
+def test_linear_swiglu(gpu_pkg):
+    print("test_linear_swiglu (large tile)", flush=True)
+    from distributed_xfold_amd.nn.base import pack_swiglu
+    g = gen(11)
+    m, k, hidden = 3850, 264, 1440            # N = 2880 = 11.25 tiles of 256
+    x = O.round_bf16(torch.randn(m, k, generator=g))
+    w1 = O.round_bf16(torch.randn(2 * hidden, k, generator=g) * 0.1)
+    h = gpu_pkg.ops.linear(x.to(dev()).bfloat16(), pack_swiglu(w1, 32).to(dev()).bfloat16(),
+                           mode=gpu_pkg.lib.LINEAR_SWIGLU)
+    y = x.double() @ w1.double().T
+    within_bf16_ulp("swiglu", h, torch.nn.functional.silu(y[:, :hidden]) * y[:, hidden:])
+
+
+def test_linear_regrouped_store(gpu_pkg):
+    print("test_linear_regrouped_store (large tile)", flush=True)
+    g = gen(12)
+    m, n, k = 3872, 2720, 136
+    x, w = O.round_bf16(torch.randn(m, k, generator=g)), O.round_bf16(torch.randn(n, k, generator=g) * 0.1)
+    got = gpu_pkg.ops.linear(x.to(dev()).bfloat16(), w.to(dev()).bfloat16(), mode=gpu_pkg.lib.LINEAR_REGROUP32)
+    y = x.double() @ w.double().T
+    want = y.reshape(m // 32, 32, n // 32, 32).permute(0, 2, 1, 3).reshape(-1, 1024)
+    assert got.shape == want.shape
+    within_bf16_ulp("regroup32", got, want)
+
+
+def test_self_attention_projection_segments(gpu_pkg):
+    """Five samples of 768 tokens send the q-k-v-gate projection (scaled and
+    biased queries, plain keys and values, sigmoid gates) to the large tile; one
+    sample alone goes through the 128x128-tile kernel.  Attention treats the
+    samples independently, so the two must agree to the rounding of the bf16
+    intermediates."""
+    print("test_self_attention_projection_segments", flush=True)
+    g = gen(13)
+    b, s, c, h = 5, 768, 768, 16
+    x = torch.randn(b, s, c, generator=g).to(dev()).bfloat16()
+    w = (torch.randn(4 * c, c, generator=g) * 0.05).to(dev()).bfloat16()
+    qb = torch.randn(c, generator=g).to(dev())
+    mask = (torch.arange(s) < 700).float().to(dev())
+    logits = torch.randn(h, s, s, generator=g).to(dev())
+    full = gpu_pkg.ops.batch_diffusion_self_attention(x, mask, logits, w, qb, h, out_dtype=torch.float32)
+    for i in (0, 4):
+        one = gpu_pkg.ops.batch_diffusion_self_attention(x[i:i + 1].contiguous(), mask, logits, w, qb, h,
+                                                         out_dtype=torch.float32)
+        d = (full[i] - one[0]).double()
+        rms = float(one.double().pow(2).mean().sqrt())
+        e_max, e_rms = float(d.abs().max()) / rms, float(d.pow(2).mean().sqrt()) / rms
+        print(f"  sample {i}: large tile vs 128 tile max {e_max:.3e} rms {e_rms:.3e}", flush=True)
+        assert e_rms < 3e-3 and e_max < 5e-2
+    # and against the float64 formula on the first sample, with the projections
+    # rounded to bf16 where the kernel stores them
+    xd, wd = x[0].double().cpu(), w.double().cpu()
+
+    def r(t):
+        return O.round_bf16(t.float()).double()
+    q = r((xd @ wd[:c].T + qb.double().cpu()) / (c // h) ** 0.5).reshape(s, h, -1)
+    k = r(xd @ wd[c:2 * c].T).reshape(s, h, -1)
+    v = r(xd @ wd[2 * c:3 * c].T).reshape(s, h, -1)
+    gate = r(torch.sigmoid(xd @ wd[3 * c:].T)).reshape(s, h, -1)
+    lg = torch.einsum("qhd,khd->hqk", q, k) + logits.double().cpu() + (mask.double().cpu() - 1.0) * 1e9
+    want = torch.einsum("hqk,khd->qhd", torch.softmax(lg, -1), v) * gate
+    e = O.rel_err(full[0].cpu(), want)
+    print(f"  vs float64: rel err {e:.3e}", flush=True)
+    assert e < 2e-2
