@@ -142,6 +142,34 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
   // ------------------------------------------------------------- epilogue
   // accumulators (lane = column, registers = rows) -> fp32 tile in LDS, then
   // each thread finishes 8 consecutive columns of a row with 16/32-byte stores
+  const int cc = (tid & 15) * 8, r0 = tid >> 4;
+  // Gate and residual of the thread's eight output chunks are requested here,
+  // all at once and ahead of the staging: asked for one chunk at a time between
+  // the stores (which may alias the residual, so the compiler keeps the order)
+  // they would be eight memory round trips in a row at the end of a workgroup
+  // that, in the small products, has nothing else to hide them behind.
+  const bool gr_ahead = g.epi == EPI_GATE_RES && g.vec_ok && n0 + cc + 8 <= g.N && !g.res_f32 &&
+                        (!g.gate || g.gate_per_row || g.gate_vec_ok) && (!g.res_bf16 || g.res_vec_ok);
+  f32x4 gate_lo[8], gate_hi[8];
+  u32x4 res_pk[8];
+  float gate_row[8];
+  if (gr_ahead) {
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int m = min(m0 + it * 16 + r0, g.M - 1), n = n0 + cc;
+      gate_row[it] = 1.f;
+      gate_lo[it] = gate_hi[it] = f32x4{1.f, 1.f, 1.f, 1.f};
+      res_pk[it] = u32x4{0, 0, 0, 0};
+      if (g.gate && g.gate_per_row) gate_row[it] = g.gate[m % g.gate_rows];
+      else if (g.gate) {
+        const float* gp = g.gate + (int64_t)(m % g.gate_rows) * g.ld_gate + n;
+        gate_lo[it] = *reinterpret_cast<const f32x4*>(gp);
+        gate_hi[it] = *reinterpret_cast<const f32x4*>(gp + 4);
+      }
+      if (g.res_bf16)
+        res_pk[it] = *reinterpret_cast<const u32x4*>(g.res_bf16 + (int64_t)bz * g.sRes + (int64_t)m * g.ld_res + n);
+    }
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -151,7 +179,6 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
         sC[(wm + 32 * i + acc_row(r, lane)) * LDC_S + wn + 32 * j + (lane & 31)] = acc[i][j][r];
   lds_barrier();
 
-  const int cc = (tid & 15) * 8, r0 = tid >> 4;
   if (g.epi == EPI_SWIGLU) {
     // weight rows are packed in blocks of 64: 32 "a" rows then the 32 matching
     // "b" rows; output has N/2 columns.  Threads with cc < 64 produce 8 outputs each.
@@ -208,6 +235,14 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
         if (op == SEG_BIAS_SCALE) v[e] = (v[e] + bias[e]) * g.alpha;
         else if (op == SEG_SIGMOID) v[e] = sigmoidf_(v[e]);
       }
+    } else if (gr_ahead) {
+      const f32x4 gl = gate_lo[it], gh = gate_hi[it];
+      const float gt[8] = {gl.x * gate_row[it], gl.y * gate_row[it], gl.z * gate_row[it], gl.w * gate_row[it],
+                           gh.x * gate_row[it], gh.y * gate_row[it], gh.z * gate_row[it], gh.w * gate_row[it]};
+      float rs[8];
+      unpack8(res_pk[it], rs);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = (v[e] + bias[e]) * gt[e] + rs[e];
     } else if (g.epi == EPI_GATE_RES) {
       const int64_t roff = (int64_t)bz * g.sRes + (int64_t)m * g.ld_res + n;
       float gt[8], rs[8];
@@ -288,6 +323,7 @@ int launch_gemm_nt(const GemmArgs& g_in, hipStream_t stream) {
   // 16/32-byte stores need aligned rows; otherwise the epilogue stores element-wise
   const int esz = g.out_f32 ? 4 : 2;
   g.vec_ok = ((uintptr_t)g.C % 16 == 0) && ((g.ldc * esz) % 16 == 0) && ((g.sC * esz) % 16 == 0);
+  g.gate_vec_ok = g.gate && !g.gate_per_row && ((uintptr_t)g.gate % 16 == 0) && (g.ld_gate % 4 == 0);
   g.res_vec_ok = g.res_bf16 && ((uintptr_t)g.res_bf16 % 16 == 0) && (g.ld_res % 8 == 0) && (g.sRes % 8 == 0);
   const int64_t total = (int64_t)((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN) * g.batch;
   const int64_t blocks = (total + 7) / 8 * 8;

@@ -26,7 +26,7 @@ struct GemmArgs {
   const float* res_f32 = nullptr;   // GATE_RES: residual added last (either dtype)
   const bf16_t* res_bf16 = nullptr;
   int64_t ld_res = 0, sRes = 0;
-  int vec_ok = 0, res_vec_ok = 0;  // set by launch_gemm_nt: rows aligned for 16-byte stores / loads
+  int vec_ok = 0, res_vec_ok = 0, gate_vec_ok = 0;  // set by launch_gemm_nt: rows aligned for 16-byte stores / loads
   // regroup32 (PLAIN, batch 1, M and N multiples of 32): element (m, n) is stored
   // at [(m / 32, n / 32)][(m % 32, n % 32)], i.e. C is [(M/32)(N/32)][1024]:
   // the outer products of 32-channel rows, one contiguous 1024-vector per pair.
