@@ -207,10 +207,11 @@ size_t af3_batch_diffusion_self_attention_workspace_bytes(int64_t batch, int64_t
 
 int af3_batch_diffusion_self_attention_forward(
     const uint16_t* q_data, const float* key_mask, int64_t mask_batches, const float* nonbatched_bias,
-    const uint16_t* w_qkvg, const float* query_b, int num_head,
+    int bias_quad_major, const uint16_t* w_qkvg, const float* query_b, int num_head,
     void* out, int out_dtype, int64_t batch, int64_t seq, int channels,
     void* workspace, size_t workspace_bytes, af3_stream_t stream) {
   if (!q_data || !w_qkvg || !out) return AF3_ERR_BAD_ARG;
+  if (bias_quad_major != 0 && (bias_quad_major != 1 || (seq & 3))) return AF3_ERR_BAD_ARG;
   if (bad_dtype(out_dtype) || batch <= 0 || seq <= 0 || channels <= 0 || (channels & 7) || num_head <= 0 ||
       channels % num_head)
     return AF3_ERR_BAD_ARG;
@@ -241,6 +242,7 @@ int af3_batch_diffusion_self_attention_forward(
   f.out = out; f.out_f32 = out_dtype == AF3_F32; f.o_ss = channels; f.o_sb = seq * channels;
   f.B = (int)batch; f.H = num_head; f.Sq = f.Sk = (int)seq; f.d = d;
   f.bias = nonbatched_bias; f.bias_sb = 0; f.bias_sh = seq * seq; f.bias_sq = seq;
+  if (bias_quad_major) { f.bias_sq = 4; f.bias_squad = seq * 4; }
   f.key_mask = key_mask; f.km_sb = mask_batches == batch && batch > 1 ? seq : 0;
   return launch_flash_attention(f, s);
 }

@@ -154,7 +154,10 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
   const float* bias_row = a.bias ? a.bias + (int64_t)bb * a.bias_sb + (int64_t)h * a.bias_sh + (int64_t)qi * a.bias_sq : nullptr;
   const bool q_is_pad = a.qpad ? (a.qpad[(int64_t)bb * a.qp_sb + qi] == 0.f) : false;
   const bool bias_vec = a.bias && a.Sk >= 4 && ((a.bias_sq & 3) == 0) && ((a.bias_sb & 3) == 0) &&
-                        ((a.bias_sh & 3) == 0) && (((uintptr_t)a.bias & 15) == 0);
+                        ((a.bias_sh & 3) == 0) && ((a.bias_squad & 3) == 0) && (((uintptr_t)a.bias & 15) == 0);
+  // key k of the row: at k (row-major) or, with quads of four keys as the outer
+  // index, at (k / 4) * bias_squad + k % 4
+  const int64_t quad_step = a.bias_squad ? a.bias_squad : 4;
   const int last_quad = (a.Sk - 1) & ~3;
   f32x4 rbias[2][4];
 #pragma unroll
@@ -167,7 +170,8 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
     for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int g = 0; g < 4; ++g)
-        rbias[u][g] = *reinterpret_cast<const f32x4*>(bias_row + min(k0 + u * 32 + 8 * g + 4 * hh, last_quad));
+        rbias[u][g] = *reinterpret_cast<const f32x4*>(
+            bias_row + (int64_t)(min(k0 + u * 32 + 8 * g + 4 * hh, last_quad) >> 2) * quad_step);
   };
 
   const int nkt = (a.Sk + KT - 1) / KT;
@@ -202,7 +206,8 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int key = k0 + u * 32 + 8 * g + 4 * hh + e;
-            s[u][4 * g + e] += bias_row[min(key, a.Sk - 1)];
+            const int kc = min(key, a.Sk - 1);
+            s[u][4 * g + e] += bias_row[(int64_t)(kc >> 2) * quad_step + (kc & 3)];
           }
         }
       }
@@ -352,6 +357,7 @@ int launch_flash_attention(const FlashArgs& a, hipStream_t stream) {
     return AF3_ERR_BAD_ARG;
   if ((a.qpad == nullptr) != (a.kpad == nullptr)) return AF3_ERR_BAD_ARG;
   if (a.key_rows && (a.bias_mod <= 0 || a.B % a.bias_mod)) return AF3_ERR_BAD_ARG;
+  if (a.bias_squad && (a.bias_sq != 4 || (a.bias_squad & 3))) return AF3_ERR_BAD_ARG;
   if (a.d == 48) return launch_nw<3, 2>(a, stream);
   if (a.d == 16) return launch_nw<1, 1>(a, stream);
   return launch_nw<2, 1>(a, stream);

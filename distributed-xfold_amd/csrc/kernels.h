@@ -129,6 +129,11 @@ struct FlashArgs {
   int B = 0, H = 0, Sq = 0, Sk = 0, d = 0;
   const float* bias = nullptr;  // [.][H][Sq][Sk], key stride 1
   int64_t bias_sb = 0, bias_sh = 0, bias_sq = 0;
+  // bias_squad != 0: quads of four keys are the outer index, [.][H][Sk/4][Sq][4]:
+  // key k of query q at q * bias_sq + (k / 4) * bias_squad + k % 4 with bias_sq = 4.
+  // The lanes of a wave hold 32 consecutive queries, so a load of one quad per
+  // lane is then one contiguous 512-byte run instead of 32 pieces of 16 bytes.
+  int64_t bias_squad = 0;
   const float* key_mask = nullptr;  // [B][Sk] (km_sb may be 0): 0 -> logit replaced by -1e9
   int64_t km_sb = 0;
   const float *qpad = nullptr, *kpad = nullptr;  // [B][Sq], [B][Sk]: +1e9 where both are 0

@@ -235,7 +235,9 @@ class DiffusionTransformer(HipModule):
                     w_gate=bf16(torch.cat(w_gate, dim=0)), b_gate=f32(torch.cat(b_gate)))
 
     def pair_logits(self, pair_cond: torch.Tensor):
-        """The pair logits of every super-block, [num_super_blocks] x [b, h, N, N].
+        """The pair logits of every super-block, [num_super_blocks] x [b, h, N, N]
+        (stored as [b, h, N/4, N, 4], the order the attention kernel reads best,
+        when N is a multiple of 4).
         They depend on pair_cond only: a caller that evaluates the transformer
         many times on one pair_cond (the diffusion sampler) computes them once
         and hands them to `forward(..., pair_logits=...)`."""
@@ -245,7 +247,10 @@ class DiffusionTransformer(HipModule):
         out = []
         for sb in range(self.num_super_blocks):
             logits = ops.pair_logits(pair_cond, p["ln_w"], None, p["w_logits"][sb], n_out)
-            out.append(logits.view(self.super_block_size, self.num_head, *logits.shape[1:]))  # (b h) n s -> b h n s
+            logits = logits.view(self.super_block_size, self.num_head, *logits.shape[1:])     # (b h) n s -> b h n s
+            if logits.shape[-1] % 4 == 0:
+                logits = ops.quad_major_bias(logits)     # computed once, read by every evaluation
+            out.append(logits)
         return out
 
     def forward(self, act: torch.Tensor, mask: torch.Tensor, single_cond: torch.Tensor,

@@ -172,6 +172,7 @@ def batch_diffusion_self_attention(q_data, key_mask, nonbatched_bias, w_qkvg, qu
                                    out_dtype=torch.bfloat16):
     """batch_diffusion_self_attention_forward (csrc/Alpha_Attention.cpp:72-92).
     q_data [B, S, C] bf16 (already normalised); key_mask [S] (shared) or [B, S];
+    nonbatched_bias [H, S, S] fp32, or [H, S/4, S, 4] as `quad_major_bias` makes it;
     returns [B, S, H, C/H]."""
     lib = _L.load()
     _gpu(q_data, "q_data", torch.bfloat16)
@@ -184,7 +185,11 @@ def batch_diffusion_self_attention(q_data, key_mask, nonbatched_bias, w_qkvg, qu
         km = _mask_f32(key_mask, (b, s), "key_mask")
     else:
         km = _mask_f32(key_mask, (s,), "key_mask")
-    if nonbatched_bias is not None:
+    quad_major = 0
+    if nonbatched_bias is not None and nonbatched_bias.dim() == 4:
+        quad_major = 1
+        _gpu(nonbatched_bias, "nonbatched_bias", torch.float32, (num_head, s // 4, s, 4))
+    elif nonbatched_bias is not None:
         _gpu(nonbatched_bias, "nonbatched_bias", torch.float32, (num_head, s, s))
     _gpu(w_qkvg, "w_qkvg", torch.bfloat16, (4 * c, c))
     if query_b is not None:
@@ -193,10 +198,22 @@ def batch_diffusion_self_attention(q_data, key_mask, nonbatched_bias, w_qkvg, qu
     nbytes = lib.af3_batch_diffusion_self_attention_workspace_bytes(b, s, c)
     ws = _ws(nbytes, q_data.device)
     rc = lib.af3_batch_diffusion_self_attention_forward(
-        _p(q_data), _p(km), mask_batches, _p(nonbatched_bias), _p(w_qkvg), _p(query_b), int(num_head), _p(out),
+        _p(q_data), _p(km), mask_batches, _p(nonbatched_bias), quad_major, _p(w_qkvg), _p(query_b), int(num_head), _p(out),
         _dt(out), b, s, c, _p(ws), ws.numel(), _stream(q_data.device))
     _L.check(rc, "af3_batch_diffusion_self_attention_forward")
     return out
+
+
+def quad_major_bias(bias):
+    """[..., Sq, Sk] -> [..., Sk/4, Sq, 4]: the pair-bias order in which the
+    attention kernel's loads are contiguous (Sk a multiple of 4).  One strided
+    copy: for a bias that is computed once and used by many attention calls."""
+    sq, sk = bias.shape[-2:]
+    if sk % 4:
+        raise ValueError("quad-major bias needs a key count that is a multiple of 4")
+    lead = tuple(bias.shape[:-2])
+    k = len(lead)
+    return bias.reshape(lead + (sq, sk // 4, 4)).permute(*range(k), k + 1, k, k + 2).contiguous()
 
 
 def batch_diffusion_cross_attention(q_data, m_data, pair_logits, mask_q, mask_k, w_qg, w_kv, query_b,

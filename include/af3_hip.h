@@ -128,14 +128,18 @@ int af3_transition_forward(
  * (masked keys replaced by -1e9) or NULL: [S] shared by the batch
  * (mask_batches = 1) or [B,S], one per batch entry as the reference operator's
  * bias [B,1,1,S] is (mask_batches = B); nonbatched_bias [H,S,S] fp32 shared by
- * the batch, or NULL.  w_qkvg [4C][C] bf16 = q, k, v, gating_query rows as
+ * the batch, or NULL; with bias_quad_major = 1 (S a multiple of 4) it is given
+ * as [H,S/4,S,4], element (h, q, k) at ((h * S/4 + k/4) * S + q) * 4 + k%4: the
+ * kernel's lanes hold consecutive queries, so this order makes its bias loads
+ * contiguous (worth it for a bias that is computed once and used many times).
+ * w_qkvg [4C][C] bf16 = q, k, v, gating_query rows as
  * stored by nn.Linear; query_b [C] fp32 or NULL.  head_dim = C/H in {16, 24, 32, 48}.
  * out [B,S,H,head_dim] (= [B,S,C]) in out_dtype: sigmoid(gate) * softmax(..) v.
  */
 size_t af3_batch_diffusion_self_attention_workspace_bytes(int64_t batch, int64_t seq, int channels);
 int af3_batch_diffusion_self_attention_forward(
     const uint16_t* q_data, const float* key_mask, int64_t mask_batches, const float* nonbatched_bias,
-    const uint16_t* w_qkvg, const float* query_b, int num_head,
+    int bias_quad_major, const uint16_t* w_qkvg, const float* query_b, int num_head,
     void* out, int out_dtype, int64_t batch, int64_t seq, int channels,
     void* workspace, size_t workspace_bytes, af3_stream_t stream);
 

@@ -103,6 +103,25 @@ def test_gathered_cross_attention_and_regrouped_store_reject_bad_arguments(pkg):
     assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 6, 1.0, 0, None, 0, None, 0, None) == -1   # unknown mode
 
 
+def test_quad_major_bias_layout_and_its_argument_check(pkg):
+    """[H, Sq, Sk] -> [H, Sk/4, Sq, 4]: element (h, q, k) at ((h * Sk/4 + k/4) * Sq + q) * 4 + k%4."""
+    bias = torch.arange(2 * 6 * 8, dtype=torch.float32).reshape(2, 6, 8)
+    qm = pkg.ops.quad_major_bias(bias)
+    assert qm.shape == (2, 2, 6, 4) and qm.is_contiguous()
+    flat = qm.reshape(-1)
+    for h, q, k in ((0, 0, 0), (1, 5, 7), (0, 3, 4), (1, 2, 1)):
+        assert flat[((h * 2 + k // 4) * 6 + q) * 4 + k % 4] == bias[h, q, k]
+    with pytest.raises(ValueError):
+        pkg.ops.quad_major_bias(torch.zeros(2, 6, 6))
+    lib = pkg.lib.load()
+    one = 1 << 20
+    # quad-major bias with a sequence length that is not a multiple of 4, or an unknown layout flag
+    assert lib.af3_batch_diffusion_self_attention_forward(one, None, 1, one, 1, one, None, 4, one, 0, 1, 30, 128,
+                                                          one, 1 << 30, None) == -1
+    assert lib.af3_batch_diffusion_self_attention_forward(one, None, 1, one, 2, one, None, 4, one, 0, 1, 32, 128,
+                                                          one, 1 << 30, None) == -1
+
+
 def test_new_modules_share_the_reference_parameter_names(pkg):
     from oracle import af3_head_oracle as H
     from oracle import af3_msa_oracle as M

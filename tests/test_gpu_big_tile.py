@@ -110,3 +110,19 @@ def test_self_attention_projection_segments(gpu_pkg):
     e = O.rel_err(full[0].cpu(), want)
     print(f"  vs float64: rel err {e:.3e}", flush=True)
     assert e < 2e-2
+
+
+@pytest.mark.parametrize("b,s,c,h", [(5, 768, 768, 16), (2, 100, 128, 4), (1, 36, 64, 4)])
+def test_quad_major_bias_is_bit_identical(gpu_pkg, b, s, c, h):
+    """The pair bias given with quads of four keys as the outer index changes
+    which addresses the attention kernel loads, not what it computes."""
+    print(f"test_quad_major_bias_is_bit_identical b={b} s={s} c={c} h={h}", flush=True)
+    g = gen(s)
+    x = torch.randn(b, s, c, generator=g).to(dev()).bfloat16()
+    w = (torch.randn(4 * c, c, generator=g) * 0.05).to(dev()).bfloat16()
+    mask = (torch.arange(s) < s - 3).float().to(dev())
+    logits = torch.randn(h, s, s, generator=g).to(dev())
+    want = gpu_pkg.ops.batch_diffusion_self_attention(x, mask, logits, w, None, h, out_dtype=torch.float32)
+    got = gpu_pkg.ops.batch_diffusion_self_attention(x, mask, gpu_pkg.ops.quad_major_bias(logits), w, None, h,
+                                                     out_dtype=torch.float32)
+    assert torch.equal(got, want)
