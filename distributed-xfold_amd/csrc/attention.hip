@@ -137,9 +137,13 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
       if (tid == 0) sAnyCode[buf] = any ? 1 : 0;
     }
   };
-  // V^T rows that no chunk covers (head dim padding) must read as zero
-  for (int idx = tid; idx < 2 * DVT * 32 * LDV; idx += NT) (&sVt[0][0])[idx] = 0;
-  lds_barrier();
+  // V^T rows that no chunk covers (head dim padding: rows KD .. 32 DVT - 1 of
+  // either buffer) must read as zero
+  if constexpr (KD < DVT * 32) {
+    constexpr int PAD_WORDS = (DVT * 32 - KD) * LDV / 2;
+    for (int idx = tid; idx < 2 * PAD_WORDS; idx += NT)
+      reinterpret_cast<uint32_t*>(&sVt[idx / PAD_WORDS][KD * LDV])[idx % PAD_WORDS] = 0u;
+  }  // (no tile store touches these rows; the barrier after the first tile's stores orders them too)
 
   f32x16 o[DVT];
 #pragma unroll
