@@ -30,7 +30,10 @@ constexpr float LOG2E = 1.4426950408889634f;
 constexpr int KEY_MASKED = 1, KEY_PAD = 2, KEY_BEYOND = 4;
 
 template <int KSTEPS, int DVT, int NW>
-__global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
+// at least two waves per SIMD: the register allocator then keeps everything in
+// the 256 architectural VGPRs instead of parking loop state in accumulation
+// registers, which would leave a single wave per SIMD
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) void flash_kernel(FlashArgs a) {
   constexpr int KD = KSTEPS * 16;  // padded q/k head dim
   constexpr int LDK = KD + 8;      // sK row stride (bf16)
   constexpr int NT = NW * 64;
@@ -90,17 +93,28 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
   const float* kmask = a.key_mask ? a.key_mask + (int64_t)b * a.km_sb : nullptr;
   const float* kpad = a.kpad ? a.kpad + (int64_t)bb * a.kp_sb : nullptr;
   int k0_loaded = 0;
+  // Rows of the K / V chunks this thread moves.  With key_rows they are looked
+  // up one tile before the chunks themselves are requested, so that a tile
+  // costs one memory round trip, not two in a row.
+  int krow_i[NLD], vrow_i[NLD];
+  auto gidx = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int idx = min(tid + i * NT, KCH - 1);
+      const int key = min(k0 + idx / (KD / 8), a.Sk - 1), vkey = min(k0 + idx % KT, a.Sk - 1);
+      krow_i[i] = krows ? krows[key] : key;
+      vrow_i[i] = krows ? krows[vkey] : vkey;
+    }
+  };
   auto gload = [&](int k0) {
     k0_loaded = k0;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int idx = min(tid + i * NT, KCH - 1);
-      const int key = min(k0 + idx / (KD / 8), a.Sk - 1), c = idx % (KD / 8);
-      const int krow = krows ? krows[key] : key;
+      const int c = idx % (KD / 8), vc = idx / KT;
+      const int krow = krow_i[i], vrow = vrow_i[i];
       k_row_ok[i] = krow >= 0;
       rk[i] = *reinterpret_cast<const u32x4*>(kg + (int64_t)max(krow, 0) * a.k_ss + (c < dch ? c : 0) * 8);
-      const int vkey = min(k0 + idx % KT, a.Sk - 1), vc = idx / KT;
-      const int vrow = krows ? krows[vkey] : vkey;
       v_row_ok[i] = vrow >= 0;
       rv[i] = *reinterpret_cast<const u32x4*>(vg + (int64_t)max(vrow, 0) * a.v_ss + (vc < dch ? vc : 0) * 8);
     }
@@ -179,14 +193,29 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
   };
 
   const int nkt = (a.Sk + KT - 1) / KT;
+  gidx(0);
   gload(0);
+  gidx(KT);
   gload_bias(0);
+  // the output gate of the lane's query: asked for now, used after the last tile
+  u32x2 gate_w[DVT][4];
+#pragma unroll
+  for (int t = 0; t < DVT; ++t)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int dd = 32 * t + 8 * g + 4 * hh;
+      gate_w[t][g] = u32x2{0x3F803F80u, 0x3F803F80u};
+      if (a.g) gate_w[t][g] = *reinterpret_cast<const u32x2*>(a.g + (int64_t)b * a.g_sb + (int64_t)qi * a.g_ss + h * d + (dd < d ? dd : 0));
+    }
   sstore(0);
   lds_barrier();
 
   for (int kt = 0; kt < nkt; ++kt) {
     const int buf = kt & 1;
     const int k0 = kt * KT;
+    // next tile's K / V chunks (their rows are known) and the rows of the one after
+    gload((kt + 1) * KT);
+    gidx((kt + 2) * KT);
     // both 32-key halves through the matrix unit first (two independent chains);
     // s[u][4g + e] = logit(query j, key k0 + 32u + 8g + 4hh + e)
     f32x16 s[2];
@@ -198,7 +227,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
       for (int ks = 0; ks < KSTEPS; ++ks)
         s[u] = mfma32(lds_frag(sK[buf], LDK, u * 32, ks * 16, lane), qf[ks], s[u]);
     }
-    // bias, then the next tile's loads into the registers just freed
+    // bias, then the next tile's bias into the registers just freed
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -215,7 +244,6 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
           }
         }
       }
-    gload((kt + 1) * KT);
     gload_bias((kt + 1) * KT);
     // Masks from the per-key codes; most tiles carry none (a workgroup-uniform
     // test skips the block).  The logits stay in natural units: the maximum
@@ -313,8 +341,8 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashArgs a) {
       float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = o[t][4 * g + e] * inv;
-      if (a.g) {
-        const u32x2 gw = *reinterpret_cast<const u32x2*>(a.g + (int64_t)b * a.g_sb + (int64_t)qi * a.g_ss + h * d + dd);
+      {
+        const u32x2 gw = gate_w[t][g];   // ones without a gate
         v[0] *= bflo(gw.x); v[1] *= bfhi(gw.x); v[2] *= bflo(gw.y); v[3] *= bfhi(gw.y);
       }
       const int64_t off = (int64_t)b * a.o_sb + (int64_t)qi * a.o_ss + h * d + dd;
