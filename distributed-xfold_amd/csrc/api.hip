@@ -252,6 +252,14 @@ int af3_transpose_bf16_forward(const uint16_t* in, uint16_t* out, int64_t rows, 
   return launch_transpose(in, out, rows, cols, static_cast<hipStream_t>(stream));
 }
 
+// ------------------------------------------------ atoms -> tokens aggregation
+int af3_gathered_relu_mean_forward(const uint16_t* src, const int32_t* idx, const float* count, float* out,
+                                   int64_t batch, int64_t n_src, int64_t n_out, int slots, int channels,
+                                   af3_stream_t stream) {
+  return launch_gathered_relu_mean(src, idx, count, out, batch, n_src, n_out, slots, channels,
+                                   static_cast<hipStream_t>(stream));
+}
+
 // ------------------------------------------------------------ batched NT product
 int af3_batched_nt_product_forward(
     const uint16_t* a, const uint16_t* b, uint16_t* c, int64_t batch, int64_t m, int64_t n, int64_t k,

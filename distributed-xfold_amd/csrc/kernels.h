@@ -60,6 +60,9 @@ struct RowNormArgs {
 };
 int launch_row_norm(const RowNormArgs& a, hipStream_t stream);
 // out[c][r] = in[r][c], bf16, rows and cols multiples of 8
+// out[b][t][:] = sum over slots a, idx[t][a] >= 0, of relu(src[b][idx[t][a]][:]) / count[t]  (fp32 out, <= 32 slots)
+int launch_gathered_relu_mean(const bf16_t* src, const int* idx, const float* count, float* out, int64_t batch,
+                              int64_t n_src, int64_t n_out, int slots, int channels, hipStream_t stream);
 int launch_transpose(const bf16_t* in, bf16_t* out, int64_t rows, int64_t cols, hipStream_t stream);
 
 // -------------------------------------------------------------- pair_tile.hip

@@ -187,7 +187,66 @@ __global__ __launch_bounds__(256) void transpose_kernel(const bf16_t* in, bf16_t
     *reinterpret_cast<u32x4*>(out + (c0 + c) * rows + r0 + rh) = u32x4{w[0], w[1], w[2], w[3]};
   }
 }
+// out[b][t][c] = (sum over slots a with idx[t][a] >= 0 of relu(src[b][idx[t][a]][c])) / count[t].
+// One thread per (b, t, 8 channels): the rows of all slots are requested
+// before any is used.
+template <int SLOTS_MAX>
+__global__ __launch_bounds__(256) void gathered_relu_mean_kernel(const bf16_t* __restrict__ src,
+                                                                  const int* __restrict__ idx,
+                                                                  const float* __restrict__ count,
+                                                                  float* __restrict__ out, int64_t batch,
+                                                                  int64_t n_src, int64_t n_out, int slots, int C) {
+  const int cch = C >> 3;
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (item >= batch * n_out * cch) return;
+  const int c8 = (int)(item % cch);
+  const int64_t t = (item / cch) % n_out, b = item / ((int64_t)cch * n_out);
+  const int* rows = idx + t * slots;
+  const bf16_t* base = src + b * n_src * C + c8 * 8;
+  u32x4 v[SLOTS_MAX];
+  bool live[SLOTS_MAX];
+#pragma unroll
+  for (int a = 0; a < SLOTS_MAX; ++a) {
+    const int r = a < slots ? rows[a] : -1;
+    live[a] = r >= 0;
+    v[a] = *reinterpret_cast<const u32x4*>(base + (int64_t)(r >= 0 ? r : 0) * C);
+  }
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll
+  for (int a = 0; a < SLOTS_MAX; ++a) {
+    float f[8];
+    unpack8(v[a], f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += live[a] ? fmaxf(f[e], 0.f) : 0.f;
+  }
+  const float d = count[t];
+  float* dst = out + (b * n_out + t) * C + c8 * 8;
+  *reinterpret_cast<f32x4*>(dst) = f32x4{acc[0] / d, acc[1] / d, acc[2] / d, acc[3] / d};
+  *reinterpret_cast<f32x4*>(dst + 4) = f32x4{acc[4] / d, acc[5] / d, acc[6] / d, acc[7] / d};
+}
+
 }  // namespace
+
+int launch_gathered_relu_mean(const bf16_t* src, const int* idx, const float* count, float* out, int64_t batch,
+                              int64_t n_src, int64_t n_out, int slots, int channels, hipStream_t stream) {
+  if (!src || !idx || !count || !out || batch <= 0 || n_src <= 0 || n_out <= 0 || slots <= 0 || slots > 32 ||
+      channels <= 0 || (channels & 7))
+    return AF3_ERR_BAD_ARG;
+  if (((uintptr_t)src & 15) || ((uintptr_t)out & 15)) return AF3_ERR_BAD_ARG;
+  const int64_t items = batch * n_out * (channels >> 3);
+  const int64_t blocks = (items + 255) / 256;
+  if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  const dim3 grid((unsigned)blocks), block(256);
+  if (slots <= 8)
+    hipLaunchKernelGGL(gathered_relu_mean_kernel<8>, grid, block, 0, stream, src, idx, count, out, batch, n_src, n_out, slots, channels);
+  else if (slots <= 24)
+    hipLaunchKernelGGL(gathered_relu_mean_kernel<24>, grid, block, 0, stream, src, idx, count, out, batch, n_src, n_out, slots, channels);
+  else
+    hipLaunchKernelGGL(gathered_relu_mean_kernel<32>, grid, block, 0, stream, src, idx, count, out, batch, n_src, n_out, slots, channels);
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
 
 int launch_transpose(const bf16_t* in, bf16_t* out, int64_t rows, int64_t cols, hipStream_t stream) {
   if (!in || !out || rows <= 0 || cols <= 0 || (rows & 7) || (cols & 7)) return AF3_ERR_BAD_ARG;

@@ -218,11 +218,26 @@ class AtomCrossAttEncoder(HipModule):
             agg = check._lin(q_act.contiguous(), self.project_atom_features_for_aggr)
         else:
             agg = ops.linear(q_act.to(torch.bfloat16).contiguous(), self.packed()["w_aggr"])
-        tok_atoms = convert(aca.queries_to_token_atoms, agg, (-3, -2))
         tm = batch.predicted_structure_info.atom_mask.float()
-        # mask_mean over the atoms of a token (:328-331); the gather has zeroed the absent atoms already
-        count = torch.clamp(tm.sum(-1), min=1e-10)[..., None]
-        tok_act = torch.relu(tok_atoms).float().sum(-2) / count
+        # mask_mean over the atoms of a token (:328-331); the gather zeroes the absent atoms
+        count = torch.clamp(tm.sum(-1), min=1e-10)
+        if in_check_mode():
+            tok_atoms = convert(aca.queries_to_token_atoms, agg, (-3, -2))
+            tok_act = torch.relu(tok_atoms).float().sum(-2) / count[..., None]
+        else:
+            # conversion to the token-atom layout, ReLU and the mean in one pass over the atoms that exist
+            gi = aca.queries_to_token_atoms
+            rows = getattr(gi, "_af3_rows32", None)
+            if rows is None or rows.device != agg.device:
+                rows = torch.where(gi.gather_mask, gi.gather_idxs, -1).to(torch.int32).contiguous()
+                try:
+                    gi._af3_rows32 = rows          # the layout of a batch does not change between evaluations
+                except AttributeError:
+                    pass
+            n_src = agg.shape[-3] * agg.shape[-2]
+            tok_act = ops.gathered_relu_mean(agg.reshape(-1, n_src, agg.shape[-1]), rows, count.contiguous())
+            if not batched:
+                tok_act = tok_act[0]
         return AtomCrossAttEncoderOutput(tok_act, skip, c.queries_mask, c.queries_single_cond, c.keys_mask,
                                          c.keys_single_cond, c.pair_cond, c.transformer_cond)
 

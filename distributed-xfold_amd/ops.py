@@ -204,6 +204,32 @@ def batch_diffusion_self_attention(q_data, key_mask, nonbatched_bias, w_qkvg, qu
     return out
 
 
+def gathered_relu_mean(src, idx, count):
+    """out[b, t] = sum_a relu(src[b, idx[t, a]]) / count[t] over the slots with idx >= 0
+    (af3_gathered_relu_mean_forward).  src [B, n_src, C] bf16, idx [T, A] int32,
+    count [T] fp32 -> [B, T, C] fp32."""
+    lib = _L.load()
+    _gpu(src, "src", torch.bfloat16)
+    if src.dim() != 3:
+        raise ValueError("src: expected [B, n_src, C]")
+    b, n_src, c = src.shape
+    if idx.dtype != torch.int32 or idx.dim() != 2 or not idx.is_contiguous() or idx.device != src.device:
+        raise ValueError("idx: expected a contiguous int32 [T, A] tensor on the device of src")
+    t, a = idx.shape
+    if a > 32 or c % 8:
+        raise ValueError("at most 32 slots, channels a multiple of 8")
+    if not getattr(idx, "_af3_checked_rows", None) == n_src:
+        if int(idx.max()) >= n_src:
+            raise ValueError("idx: row index beyond src")
+        idx._af3_checked_rows = n_src          # one device round trip per index tensor
+    _gpu(count, "count", torch.float32, (t,))
+    out = torch.empty((b, t, c), dtype=torch.float32, device=src.device)
+    rc = lib.af3_gathered_relu_mean_forward(_p(src), _p(idx), _p(count), _p(out), b, n_src, t, a, c,
+                                            _stream(src.device))
+    _L.check(rc, "af3_gathered_relu_mean_forward")
+    return out
+
+
 def quad_major_bias(bias):
     """[..., Sq, Sk] -> [..., Sk/4, Sq, 4]: the pair-bias order in which the
     attention kernel's loads are contiguous (Sk a multiple of 4).  One strided

@@ -212,6 +212,22 @@ int af3_batched_nt_product_forward(
 int af3_transpose_bf16_forward(const uint16_t* in, uint16_t* out, int64_t rows, int64_t cols, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Aggregation of per-atom activations to tokens, the tail of the atom
+ * cross-attention encoder (nn/d_atom_cross_attention.py:322-331: conversion of
+ * the projected query activations to the token-atom layout, ReLU, masked mean
+ * over the atom slots of a token):
+ *   out[b][t][c] = (sum over slots a with idx[t][a] >= 0 of
+ *                   max(src[b][idx[t][a]][c], 0)) / count[t]
+ * src [batch][n_src][channels] bf16, idx [n_out][slots] int32 (row of src, or
+ * negative for an absent atom; every index < n_src), count [n_out] fp32 (the
+ * divisor, > 0), out [batch][n_out][channels] fp32.  slots <= 32, channels a
+ * multiple of 8.  The sum is taken in slot order in fp32.
+ */
+int af3_gathered_relu_mean_forward(const uint16_t* src, const int32_t* idx, const float* count, float* out,
+                                   int64_t batch, int64_t n_src, int64_t n_out, int slots, int channels,
+                                   af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Pair-logit projection: out[h][i][j] = (LayerNorm(pair)[i][j] . w[h]).
  * Replaces the eager `single_pair_logits_projection(single_pair_logits_norm(
  * pair)).permute(2,0,1)` of nn/d_pairformer.py:160-162 and the

@@ -122,6 +122,15 @@ def test_quad_major_bias_layout_and_its_argument_check(pkg):
                                                           one, 1 << 30, None) == -1
 
 
+def test_gathered_relu_mean_rejects_bad_arguments(pkg):
+    lib = pkg.lib.load()
+    one = 1 << 20
+    assert lib.af3_gathered_relu_mean_forward(one, None, one, one, 1, 8, 8, 4, 128, None) == -1    # no index table
+    assert lib.af3_gathered_relu_mean_forward(one, one, one, one, 1, 8, 8, 33, 128, None) == -1    # too many slots
+    assert lib.af3_gathered_relu_mean_forward(one, one, one, one, 1, 8, 8, 4, 100, None) == -1     # channels % 8
+    assert lib.af3_gathered_relu_mean_forward(one + 2, one, one, one, 1, 8, 8, 4, 128, None) == -1  # misaligned
+
+
 def test_new_modules_share_the_reference_parameter_names(pkg):
     from oracle import af3_head_oracle as H
     from oracle import af3_msa_oracle as M

@@ -191,3 +191,27 @@ def test_encoder_without_positions_and_trunk_conditioning(gpu_pkg):
         live = want.queries_mask[..., None]
         compare(f"skip connection {mode}", got.skip_connection.float().cpu() * live, want.skip_connection * live,
                 rms_tol, max_tol)
+
+
+@pytest.mark.parametrize("b,n_src,t,a,c", [(1, 40, 7, 5, 16), (3, 500, 61, 24, 768), (2, 96, 10, 32, 128)])
+def test_gathered_relu_mean(gpu_pkg, b, n_src, t, a, c):
+    """Atoms -> tokens aggregation (conversion to the token-atom layout, ReLU,
+    masked mean) in one kernel against the same steps in torch."""
+    print(f"test_gathered_relu_mean b={b} n_src={n_src} t={t} a={a} c={c}", flush=True)
+    g = torch.Generator().manual_seed(t)
+    src = torch.randn(b, n_src, c, generator=g).bfloat16()
+    idx = torch.randint(0, n_src, (t, a), generator=g)
+    present = torch.rand(t, a, generator=g) > 0.3
+    present[0] = False                       # a token without atoms: zero sum over the clamped count
+    present[1] = True
+    count = torch.clamp(present.float().sum(-1), min=1e-10)
+    rows = torch.where(present, idx, -1).to(torch.int32)
+    dev = torch.device("cuda:0")
+    got = gpu_pkg.ops.gathered_relu_mean(src.to(dev), rows.to(dev), count.to(dev)).cpu()
+    gathered = src.float()[:, idx.reshape(-1)].reshape(b, t, a, c) * present[None, :, :, None]
+    want = torch.relu(gathered).double().sum(-2) / count.double()[None, :, None]
+    assert got.shape == (b, t, c)
+    assert float((got.double() - want).abs().max()) <= 1e-6 * float(want.abs().max()) + 1e-30
+    assert torch.all(got[:, 0] == 0)
+    with pytest.raises(ValueError):
+        gpu_pkg.ops.gathered_relu_mean(src.to(dev), (rows + n_src).to(dev), count.to(dev))
