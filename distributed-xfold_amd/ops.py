@@ -20,9 +20,10 @@ _workspaces: dict = {}
 
 
 def _ws(nbytes: int, device) -> torch.Tensor:
-    """Per-device scratch buffer, grown on demand and reused between calls
-    (calls on one stream are ordered, so reuse is safe)."""
-    key = (device.type, device.index)
+    """Scratch buffer per device and stream, grown on demand and reused between
+    calls (calls on one stream are ordered, so reuse is safe; calls on different
+    streams may run at the same time and get different buffers)."""
+    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
