@@ -260,6 +260,14 @@ int af3_gathered_relu_mean_forward(const uint16_t* src, const int32_t* idx, cons
                                    static_cast<hipStream_t>(stream));
 }
 
+int af3_atom_position_features_forward(const float* positions, const int32_t* rows, const float* weight,
+                                       const float* cond, void* out, int out_dtype, int64_t batch, int64_t n_slots,
+                                       int64_t n_queries, int channels, af3_stream_t stream) {
+  if (bad_dtype(out_dtype)) return AF3_ERR_BAD_ARG;
+  return launch_atom_position_features(positions, rows, weight, cond, out, out_dtype == AF3_F32, batch, n_slots,
+                                       n_queries, channels, static_cast<hipStream_t>(stream));
+}
+
 // ------------------------------------------------------------ batched NT product
 int af3_batched_nt_product_forward(
     const uint16_t* a, const uint16_t* b, uint16_t* c, int64_t batch, int64_t m, int64_t n, int64_t k,

@@ -63,6 +63,10 @@ int launch_row_norm(const RowNormArgs& a, hipStream_t stream);
 // out[b][t][:] = sum over slots a, idx[t][a] >= 0, of relu(src[b][idx[t][a]][:]) / count[t]  (fp32 out, <= 32 slots)
 int launch_gathered_relu_mean(const bf16_t* src, const int* idx, const float* count, float* out, int64_t batch,
                               int64_t n_src, int64_t n_out, int slots, int channels, hipStream_t stream);
+// out[b][q][:] = cond[q][:] + w pos[b][rows[q]]  (3 coordinates -> channels; rows[q] < 0: cond only)
+int launch_atom_position_features(const float* pos, const int* rows, const float* w, const float* cond, void* out,
+                                  int out_f32, int64_t batch, int64_t n_slots, int64_t n_q, int channels,
+                                  hipStream_t stream);
 int launch_transpose(const bf16_t* in, bf16_t* out, int64_t rows, int64_t cols, hipStream_t stream);
 
 // -------------------------------------------------------------- pair_tile.hip

@@ -3,6 +3,8 @@
 // row (or, for narrow rows, a group of 1..16 lanes does): 16-byte loads,
 // two-pass statistics in registers, a shuffle reduction, bf16 output ready to
 // be an MFMA operand.  HBM-bound.
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -227,7 +229,63 @@ __global__ __launch_bounds__(256) void gathered_relu_mean_kernel(const bf16_t* _
   *reinterpret_cast<f32x4*>(dst + 4) = f32x4{acc[4] / d, acc[5] / d, acc[6] / d, acc[7] / d};
 }
 
+// out[b][q][c] = cond[q][c] + sum_k pos[b][rows[q]][k] * w[c][k]  (rows[q] < 0: no position term)
+// One thread per (b, q, 8 channels).
+template <typename TOUT>
+__global__ __launch_bounds__(256) void atom_position_features_kernel(const float* __restrict__ pos,
+                                                                      const int* __restrict__ rows,
+                                                                      const float* __restrict__ w,
+                                                                      const float* __restrict__ cond,
+                                                                      TOUT* __restrict__ out, int64_t batch,
+                                                                      int64_t n_slots, int64_t n_q, int C) {
+  const int cch = C >> 3;
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (item >= batch * n_q * cch) return;
+  const int c0 = (int)(item % cch) * 8;
+  const int64_t q = (item / cch) % n_q, b = item / ((int64_t)cch * n_q);
+  const int r = rows[q];
+  const float* pp = pos + (b * n_slots + (r >= 0 ? r : 0)) * 3;
+  const float live = r >= 0 ? 1.f : 0.f;
+  const float x = pp[0] * live, y = pp[1] * live, z = pp[2] * live;
+  const float* cp = cond + q * C + c0;
+  const f32x4 ca = *reinterpret_cast<const f32x4*>(cp), cb = *reinterpret_cast<const f32x4*>(cp + 4);
+  const float cv[8] = {ca.x, ca.y, ca.z, ca.w, cb.x, cb.y, cb.z, cb.w};
+  float o[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float* we = w + (c0 + e) * 3;
+    // the order of the eager steps: ((x w0 + y w1) + z w2), then + cond
+    o[e] = ((x * we[0] + y * we[1]) + z * we[2]) + cv[e];
+  }
+  TOUT* dst = out + (b * n_q + q) * C + c0;
+  if constexpr (std::is_same<TOUT, float>::value) {
+    *reinterpret_cast<f32x4*>(dst) = f32x4{o[0], o[1], o[2], o[3]};
+    *reinterpret_cast<f32x4*>(dst + 4) = f32x4{o[4], o[5], o[6], o[7]};
+  } else {
+    *reinterpret_cast<u32x4*>(dst) = pack8(o);
+  }
+}
+
 }  // namespace
+
+int launch_atom_position_features(const float* pos, const int* rows, const float* w, const float* cond, void* out,
+                                  int out_f32, int64_t batch, int64_t n_slots, int64_t n_q, int channels,
+                                  hipStream_t stream) {
+  if (!pos || !rows || !w || !cond || !out || batch <= 0 || n_slots <= 0 || n_q <= 0 || channels <= 0 || (channels & 7))
+    return AF3_ERR_BAD_ARG;
+  if (((uintptr_t)cond & 15) || ((uintptr_t)out & 15)) return AF3_ERR_BAD_ARG;
+  const int64_t items = batch * n_q * (channels >> 3);
+  const int64_t blocks = (items + 255) / 256;
+  if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  const dim3 grid((unsigned)blocks), block(256);
+  if (out_f32)
+    hipLaunchKernelGGL(atom_position_features_kernel<float>, grid, block, 0, stream, pos, rows, w, cond,
+                       static_cast<float*>(out), batch, n_slots, n_q, channels);
+  else
+    hipLaunchKernelGGL(atom_position_features_kernel<bf16_t>, grid, block, 0, stream, pos, rows, w, cond,
+                       static_cast<bf16_t*>(out), batch, n_slots, n_q, channels);
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
 
 int launch_gathered_relu_mean(const bf16_t* src, const int* idx, const float* count, float* out, int64_t batch,
                               int64_t n_src, int64_t n_out, int slots, int channels, hipStream_t stream) {

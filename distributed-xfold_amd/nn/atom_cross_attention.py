@@ -118,6 +118,8 @@ class AtomCrossAttEncoder(HipModule):
         if self.with_trunk_pair_cond:
             d["tp_ln"] = f32(self.lnorm_trunk_pair_cond.weight)
             d["tp_w"] = bf16(self.embed_trunk_pair_cond.weight)
+        if hasattr(self, "atom_positions_to_features"):
+            d["w_pos"] = f32(self.atom_positions_to_features.weight)
         return d
 
     def _per_atom_conditioning(self, batch):
@@ -203,10 +205,27 @@ class AtomCrossAttEncoder(HipModule):
         qm = qm[None, ..., None] if batched else qm[..., None]
         if token_atoms_act is None:
             q_act = c.queries_single_cond.clone()
-        else:
+        elif in_check_mode():
             q_act = convert(aca.token_atoms_to_queries, token_atoms_act.float(), (-3, -2))
             q_act = _lin(q_act, self.atom_positions_to_features) * qm
             q_act = q_act + (c.queries_single_cond[None] if batched else c.queries_single_cond)
+        else:
+            # conversion to the query layout, 3 -> channels projection, query mask and conditioning in one pass
+            gi = aca.token_atoms_to_queries
+            rows = getattr(gi, "_af3_rows32", None)
+            if rows is None or rows.device != token_atoms_act.device:
+                live = gi.gather_mask & (c.queries_mask != 0)
+                rows = torch.where(live, gi.gather_idxs, -1).to(torch.int32).reshape(-1).contiguous()
+                try:
+                    gi._af3_rows32 = rows
+                except AttributeError:
+                    pass
+            cond = c.queries_single_cond
+            n_slots = token_atoms_act.shape[-3] * token_atoms_act.shape[-2]
+            q_act = ops.atom_position_features(token_atoms_act.float().reshape(-1, n_slots, 3).contiguous(), rows,
+                                               self.packed()["w_pos"],
+                                               cond.float().reshape(-1, cond.shape[-1]).contiguous(), out_dtype=act_dtype)
+            q_act = q_act.view(*token_atoms_act.shape[:-3], *cond.shape)
         q_act = q_act.to(act_dtype).contiguous()
         q_act = self.atom_transformer_encoder(
             queries_act=q_act, queries_mask=c.queries_mask, queries_to_keys=aca.queries_to_keys,

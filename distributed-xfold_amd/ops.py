@@ -205,6 +205,34 @@ def batch_diffusion_self_attention(q_data, key_mask, nonbatched_bias, w_qkvg, qu
     return out
 
 
+def atom_position_features(positions, rows, weight, cond, out_dtype=torch.bfloat16):
+    """out[b, q] = cond[q] + weight @ positions[b, rows[q]] (rows[q] < 0: cond[q] only)
+    (af3_atom_position_features_forward).  positions [B, n_slots, 3] fp32, rows [Q] int32,
+    weight [C, 3] fp32, cond [Q, C] fp32 -> [B, Q, C]."""
+    lib = _L.load()
+    _gpu(positions, "positions", torch.float32)
+    if positions.dim() != 3 or positions.shape[-1] != 3:
+        raise ValueError("positions: expected [B, n_slots, 3]")
+    b, n_slots = positions.shape[:2]
+    if rows.dtype != torch.int32 or rows.dim() != 1 or not rows.is_contiguous() or rows.device != positions.device:
+        raise ValueError("rows: expected a contiguous int32 [Q] tensor on the device of positions")
+    q = rows.shape[0]
+    c = weight.shape[0]
+    _gpu(weight, "weight", torch.float32, (c, 3))
+    _gpu(cond, "cond", torch.float32, (q, c))
+    if c % 8:
+        raise ValueError("channels must be a multiple of 8")
+    if getattr(rows, "_af3_checked_rows", None) != n_slots:
+        if int(rows.max()) >= n_slots:
+            raise ValueError("rows: slot index beyond positions")
+        rows._af3_checked_rows = n_slots
+    out = torch.empty((b, q, c), dtype=out_dtype, device=positions.device)
+    rc = lib.af3_atom_position_features_forward(_p(positions), _p(rows), _p(weight), _p(cond), _p(out), _dt(out),
+                                                b, n_slots, q, c, _stream(positions.device))
+    _L.check(rc, "af3_atom_position_features_forward")
+    return out
+
+
 def gathered_relu_mean(src, idx, count):
     """out[b, t] = sum_a relu(src[b, idx[t, a]]) / count[t] over the slots with idx >= 0
     (af3_gathered_relu_mean_forward).  src [B, n_src, C] bf16, idx [T, A] int32,

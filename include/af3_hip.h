@@ -228,6 +228,20 @@ int af3_gathered_relu_mean_forward(const uint16_t* src, const int32_t* idx, cons
                                    af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Embedding of the noisy atom positions, the head of the atom cross-attention
+ * encoder (nn/d_atom_cross_attention.py:195-207: conversion of the positions to
+ * the query layout, the 3 -> channels projection, query mask, + conditioning):
+ *   out[b][q][c] = cond[q][c] + sum_k positions[b][rows[q]][k] * weight[c][k]
+ * positions [batch][n_slots][3] fp32, rows [n_queries] int32 (slot of the
+ * query's atom, or negative for a query without atom / masked query: the
+ * position term is then zero), weight [channels][3] fp32, cond
+ * [n_queries][channels] fp32, out [batch][n_queries][channels] in out_dtype.
+ */
+int af3_atom_position_features_forward(const float* positions, const int32_t* rows, const float* weight,
+                                       const float* cond, void* out, int out_dtype, int64_t batch, int64_t n_slots,
+                                       int64_t n_queries, int channels, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Pair-logit projection: out[h][i][j] = (LayerNorm(pair)[i][j] . w[h]).
  * Replaces the eager `single_pair_logits_projection(single_pair_logits_norm(
  * pair)).permute(2,0,1)` of nn/d_pairformer.py:160-162 and the

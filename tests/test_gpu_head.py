@@ -215,3 +215,23 @@ def test_gathered_relu_mean(gpu_pkg, b, n_src, t, a, c):
     assert torch.all(got[:, 0] == 0)
     with pytest.raises(ValueError):
         gpu_pkg.ops.gathered_relu_mean(src.to(dev), (rows + n_src).to(dev), count.to(dev))
+
+
+@pytest.mark.parametrize("b,n_slots,q,c,dt", [(1, 30, 64, 16, torch.float32), (5, 720, 736, 128, torch.bfloat16)])
+def test_atom_position_features(gpu_pkg, b, n_slots, q, c, dt):
+    """Position embedding at the head of the atom encoder (layout conversion, 3 -> c
+    projection, query mask, + conditioning) in one kernel against the same steps in torch."""
+    print(f"test_atom_position_features b={b} n_slots={n_slots} q={q} c={c} {dt}", flush=True)
+    g = torch.Generator().manual_seed(q)
+    pos = torch.randn(b, n_slots, 3, generator=g)
+    rows = torch.randint(0, n_slots, (q,), generator=g)
+    live = torch.rand(q, generator=g) > 0.2
+    w, cond = torch.randn(c, 3, generator=g), torch.randn(q, c, generator=g)
+    dev = torch.device("cuda:0")
+    rows32 = torch.where(live, rows, -1).to(torch.int32)
+    got = gpu_pkg.ops.atom_position_features(pos.to(dev), rows32.to(dev), w.to(dev), cond.to(dev), out_dtype=dt).cpu()
+    want = (pos[:, rows].double() * live[None, :, None]) @ w.double().T + cond.double()
+    assert got.shape == (b, q, c) and got.dtype == dt
+    tol = 2.0 ** -8 if dt == torch.bfloat16 else 1e-6
+    assert float((got.double() - want).abs().max()) <= tol * float(want.abs().max())
+    assert torch.equal(got[:, ~live].float(), cond[~live].to(dt).float()[None].expand(b, -1, -1))
