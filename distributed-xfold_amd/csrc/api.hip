@@ -429,8 +429,9 @@ int af3_layer_norm_forward(
 int af3_linear_forward(
     const uint16_t* x, const uint16_t* w, const float* bias, void* y, int y_dtype,
     int64_t m, int n, int k, int mode, float alpha, int sigmoid,
-    const float* gate, int64_t gate_rows, const void* residual, int res_dtype, af3_stream_t stream) {
+    const float* gate, int64_t gate_rows, int64_t gate_ld, const void* residual, int res_dtype, af3_stream_t stream) {
   if (!x || !w || !y || bad_dtype(y_dtype) || m <= 0 || m > 0x7fffffff || n <= 0 || k <= 0) return AF3_ERR_BAD_ARG;
+  if (gate_ld != 0 && gate_ld < n) return AF3_ERR_BAD_ARG;
   if (mode != AF3_LINEAR_PLAIN && mode != AF3_LINEAR_SWIGLU && mode != AF3_LINEAR_GATE_RES &&
       mode != AF3_LINEAR_REGROUP32 && mode != AF3_LINEAR_ROWGATE_RES)
     return AF3_ERR_BAD_ARG;
@@ -452,7 +453,7 @@ int af3_linear_forward(
   g.ldc = mode == AF3_LINEAR_SWIGLU ? n / 2 : n;
   g.out_f32 = y_dtype == AF3_F32;
   g.epi = mode; g.alpha = alpha; g.bias = bias; g.act_sigmoid = sigmoid;
-  g.gate = gate; g.gate_rows = (int)gate_rows; g.ld_gate = n;
+  g.gate = gate; g.gate_rows = (int)gate_rows; g.ld_gate = gate_ld ? gate_ld : n;
   if (residual) {
     if (res_dtype == AF3_F32) g.res_f32 = static_cast<const float*>(residual);
     else g.res_bf16 = static_cast<const bf16_t*>(residual);

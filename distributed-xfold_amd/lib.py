@@ -41,7 +41,7 @@ SIGNATURES = {
     "af3_pair_logits_forward": (_i, [_vp, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp]),
     "af3_layer_norm_forward": (_i, [_vp, _i, _vp, _i64, _i, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "af3_linear_forward": (
-        _i, [_vp, _vp, _vp, _vp, _i, _i64, _i, _i, _i, _f, _i, _vp, _i64, _vp, _i, _vp]),
+        _i, [_vp, _vp, _vp, _vp, _i, _i64, _i, _i, _i, _f, _i, _vp, _i64, _i64, _vp, _i, _vp]),
     "af3_triangle_contraction_forward": (_i, [_vp, _vp, _vp, _i64, _vp]),
     "af3_grid_attention_core_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
     "af3_check_gemm_f32": (

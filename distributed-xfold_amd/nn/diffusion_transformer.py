@@ -270,7 +270,7 @@ class DiffusionTransformer(HipModule):
         ss_all = ss_all.view(rows, n_mod, 2 * c)                       # column slices, read in place
         gate_all = ops.linear(sc.to(torch.bfloat16), p["w_gate"], bias=p["b_gate"], out_dtype=torch.float32,
                               sigmoid=True)
-        gate_all = gate_all.view(rows, n_mod, c).permute(1, 0, 2).contiguous()   # [module][row][c]
+        gate_all = gate_all.view(rows, n_mod, c).permute(1, 0, 2)      # [module][row][c]: column slices, read in place
         for sb in range(self.num_super_blocks):
             if pair_logits is not None:
                 logits = pair_logits[sb]

@@ -458,14 +458,20 @@ def linear(x, w, bias=None, out_dtype=torch.bfloat16, mode=_L.LINEAR_PLAIN, alph
         out = torch.empty(shape, dtype=out_dtype, device=x.device)
     else:
         _gpu(out, "out", None, shape)
-    gate_rows = 0
+    gate_rows = gate_ld = 0
     if gate is not None and mode == _L.LINEAR_ROWGATE_RES:
         _gpu(gate, "gate", torch.float32)
         gate_rows = gate.numel()
         if m % gate_rows:
             raise ValueError("rows must be a multiple of the gate rows")
     elif gate is not None:
-        _gpu(gate, "gate", torch.float32)
+        if gate.dim() == 2 and not gate.is_contiguous() and gate.stride(1) == 1 and gate.stride(0) >= n:
+            # a column slice of a wider tensor, used in place: rows gate_ld floats apart
+            if not gate.is_cuda or gate.dtype != torch.float32:
+                raise ValueError("gate: expected an fp32 tensor on the GPU")
+            gate_ld = gate.stride(0)
+        else:
+            _gpu(gate, "gate", torch.float32)
         if gate.shape[-1] != n:
             raise ValueError("gate: last dimension must equal the output width")
         gate_rows = gate.numel() // n
@@ -476,7 +482,7 @@ def linear(x, w, bias=None, out_dtype=torch.bfloat16, mode=_L.LINEAR_PLAIN, alph
         _gpu(residual, "residual", None, shape)
         res_dt = _dt(residual)
     rc = lib.af3_linear_forward(_p(x), _p(w), _p(bias), _p(out), _dt(out), m, n, k, int(mode), float(alpha),
-                                int(bool(sigmoid)), _p(gate), gate_rows, _p(residual), res_dt,
+                                int(bool(sigmoid)), _p(gate), gate_rows, gate_ld, _p(residual), res_dt,
                                 _stream(x.device))
     _L.check(rc, "af3_linear_forward")
     return out

@@ -279,7 +279,9 @@ int af3_layer_norm_forward(
  *        blocks of 64: 32 rows of the silu half, then the 32 matching rows of
  *        the linear half
  *  mode AF3_LINEAR_GATE_RES: y = residual + gate[m % gate_rows] * (x W^T + bias)
- *        (gate fp32 [gate_rows,N] or NULL; residual in res_dtype or NULL)
+ *        (gate fp32 [gate_rows,N] or NULL, its rows gate_ld floats apart
+ *        (0 = N: contiguous), so that one slice of a wider projection can be
+ *        used in place; residual in res_dtype or NULL)
  *  mode AF3_LINEAR_REGROUP32: PLAIN, with element (m, n) stored at
  *        y[(m/32, n/32)][(m%32, n%32)], y [(M/32)*(N/32), 1024] (M, N multiples
  *        of 32).  With x = [(token b, channel c), msa row] and w = [(token d,
@@ -298,7 +300,7 @@ int af3_linear_forward(
     const uint16_t* x, const uint16_t* w, const float* bias,
     void* y, int y_dtype, int64_t m, int n, int k,
     int mode, float alpha, int sigmoid,
-    const float* gate, int64_t gate_rows,
+    const float* gate, int64_t gate_rows, int64_t gate_ld,
     const void* residual, int res_dtype, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------

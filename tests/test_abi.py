@@ -72,7 +72,7 @@ def test_null_and_bad_arguments_are_rejected_without_a_gpu(pkg):
     """Argument validation happens before any launch, so it can run here."""
     lib = pkg.lib.load()
     assert lib.af3_transition_forward(None, 0, None, None, None, None, 512, None, 0, 10, None) == -1
-    assert lib.af3_linear_forward(None, None, None, None, 0, 1, 8, 8, 0, 1.0, 0, None, 0, None, 0, None) == -1
+    assert lib.af3_linear_forward(None, None, None, None, 0, 1, 8, 8, 0, 1.0, 0, None, 0, 0, None, 0, None) == -1
     assert lib.af3_triangle_multiplication_forward(None, 0, None, 0, None, None, None, None, None, None, None,
                                                    None, 0, 8, None, 0, None) == -1
 
@@ -97,10 +97,11 @@ def test_gathered_cross_attention_and_regrouped_store_reject_bad_arguments(pkg):
     assert call(wsb=16) == -2                          # workspace too small
     assert lib.af3_gathered_cross_attention_workspace_bytes(8, 32, 2, 128, 128) >= (8 * 32 + 2 * 128) * 256 * 2
     # regrouped store: rows of both operands in multiples of 32, no gate / residual
-    assert lib.af3_linear_forward(one, one, None, one, 0, 48, 64, 8, 4, 1.0, 0, None, 0, None, 0, None) == -1
-    assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 4, 1.0, 0, one, 1, None, 0, None) == -1
-    assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 5, 1.0, 0, None, 0, None, 0, None) == -1   # row gate missing
-    assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 6, 1.0, 0, None, 0, None, 0, None) == -1   # unknown mode
+    assert lib.af3_linear_forward(one, one, None, one, 0, 48, 64, 8, 4, 1.0, 0, None, 0, 0, None, 0, None) == -1
+    assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 4, 1.0, 0, one, 1, 0, None, 0, None) == -1
+    assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 5, 1.0, 0, None, 0, 0, None, 0, None) == -1   # row gate missing
+    assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 6, 1.0, 0, None, 0, 0, None, 0, None) == -1   # unknown mode
+    assert lib.af3_linear_forward(one, one, None, one, 0, 64, 64, 8, 3, 1.0, 0, one, 1, 32, None, 0, None) == -1  # gate rows overlap
 
 
 def test_quad_major_bias_layout_and_its_argument_check(pkg):
