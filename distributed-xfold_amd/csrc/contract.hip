@@ -103,8 +103,18 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   const int per_xcd = (total + 7) / 8;
   const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (logical >= total) return;
-  const int tm = logical % tiles_m, tn = (logical / tiles_m) % tiles_n;
+  int tm = logical % tiles_m, tn = (logical / tiles_m) % tiles_n;
   const int bz = logical / (tiles_m * tiles_n);
+  if (g.batch == 1 && (tiles_m & 3) == 0 && (tiles_n & 1) == 0) {
+    // One large product: an XCD that walks whole columns of tiles re-reads all of
+    // A for every column, and A (8 MB at 4096 x 1024) does not stay in its 4 MB
+    // L2.  Deal the XCDs a 4 x 2 grid of rectangles instead: a quarter of A stays
+    // resident while the XCD streams through its half of B once.
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int mq = tiles_m >> 2, nh = tiles_n >> 1;
+    tm = (xcd & 3) * mq + slot % mq;
+    tn = (xcd >> 2) * nh + slot / mq;
+  }
   const int m0 = tm * CM, n0 = tn * CN;
 
   const char* A = reinterpret_cast<const char*>(g.A + (int64_t)bz * g.sA);
