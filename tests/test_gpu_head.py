@@ -235,3 +235,25 @@ def test_atom_position_features(gpu_pkg, b, n_slots, q, c, dt):
     tol = 2.0 ** -8 if dt == torch.bfloat16 else 1e-6
     assert float((got.double() - want).abs().max()) <= tol * float(want.abs().max())
     assert torch.equal(got[:, ~live].float(), cond[~live].to(dt).float()[None].expand(b, -1, -1))
+
+
+def test_head_without_batch_inference_matches_the_batched_head(gpu_pkg):
+    """use_batch_infer=False (one sample, positions [N, A, 3], as the reference's
+    unbatched modules take them) runs the same kernels on a batch of one: the
+    update equals the batched head's on the same sample."""
+    g, batch, p, emb, pos, head = case(gpu_pkg, 20, 2, seed=77, samples=2)
+    single = gpu_pkg.nn.DiffusionHead(False, num_blocks=2)
+    single.load_state_dict(p)
+    single.to(dev())
+    gb, ge = batch.to(dev()), on_gpu(emb)
+    levels, t_hat, _ = H.sampler_schedule(4)
+    t = t_hat[1].float().to(dev())
+    sc, pc = head.pre_conditioning(gb, ge, t_hat.float().to(dev()), True)
+    noisy = (pos * float(t_hat[1])).to(dev())
+    want = head(noisy, t, gb, ge, sc[1], pc)
+    for i in range(2):
+        got = single(noisy[i], t, gb, ge, sc[1], pc)
+        assert got.shape == want[i].shape
+        err = float((got - want[i]).abs().max()) / float(want[i].abs().max())
+        print(f"unbatched head, sample {i}: max difference {err:.3e}", flush=True)
+        assert err <= 1e-6
