@@ -268,6 +268,19 @@ int af3_atom_position_features_forward(const float* positions, const int32_t* ro
                                        n_queries, channels, static_cast<hipStream_t>(stream));
 }
 
+int af3_gather_rows_add_forward(const uint16_t* src, const int32_t* rows, const uint16_t* add, uint16_t* out,
+                                int64_t batch, int64_t n_src, int64_t n_queries, int channels, af3_stream_t stream) {
+  return launch_gather_rows_add(src, rows, add, out, batch, n_src, n_queries, channels,
+                                static_cast<hipStream_t>(stream));
+}
+
+int af3_position_update_forward(const uint16_t* x, const int32_t* rows, const float* ln_weight, const float* weight,
+                                float* out, int64_t batch, int64_t n_src, int64_t n_out, int channels,
+                                af3_stream_t stream) {
+  return launch_ln_project3_gather(x, rows, ln_weight, weight, out, batch, n_src, n_out, channels,
+                                   static_cast<hipStream_t>(stream));
+}
+
 // ------------------------------------------------------------ batched NT product
 int af3_batched_nt_product_forward(
     const uint16_t* a, const uint16_t* b, uint16_t* c, int64_t batch, int64_t m, int64_t n, int64_t k,

@@ -67,6 +67,12 @@ int launch_gathered_relu_mean(const bf16_t* src, const int* idx, const float* co
 int launch_atom_position_features(const float* pos, const int* rows, const float* w, const float* cond, void* out,
                                   int out_f32, int64_t batch, int64_t n_slots, int64_t n_q, int channels,
                                   hipStream_t stream);
+// out[b][q][:] = (rows[q] >= 0 ? src[b][rows[q]][:] : 0) + add[b][q][:]   (all bf16)
+int launch_gather_rows_add(const bf16_t* src, const int* rows, const bf16_t* add, bf16_t* out, int64_t batch,
+                           int64_t n_src, int64_t n_q, int channels, hipStream_t stream);
+// out[b][t][0..2] = w LayerNorm(x[b][rows[t]]) * ln_w  (rows[t] < 0: zeros); channels = 128, fp32 out
+int launch_ln_project3_gather(const bf16_t* x, const int* rows, const float* ln_w, const float* w, float* out,
+                              int64_t batch, int64_t n_src, int64_t n_out, int channels, hipStream_t stream);
 int launch_transpose(const bf16_t* in, bf16_t* out, int64_t rows, int64_t cols, hipStream_t stream);
 
 // -------------------------------------------------------------- pair_tile.hip

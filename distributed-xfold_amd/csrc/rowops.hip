@@ -266,7 +266,94 @@ __global__ __launch_bounds__(256) void atom_position_features_kernel(const float
   }
 }
 
+// out[b][q][:] = bf16((rows[q] >= 0 ? src[b][rows[q]][:] : 0) + add[b][q][:]), one thread per 8 channels
+__global__ __launch_bounds__(256) void gather_rows_add_kernel(const bf16_t* __restrict__ src,
+                                                               const int* __restrict__ rows,
+                                                               const bf16_t* __restrict__ add, bf16_t* __restrict__ out,
+                                                               int64_t batch, int64_t n_src, int64_t n_q, int C) {
+  const int cch = C >> 3;
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (item >= batch * n_q * cch) return;
+  const int c0 = (int)(item % cch) * 8;
+  const int64_t q = (item / cch) % n_q, b = item / ((int64_t)cch * n_q);
+  const int r = rows[q];
+  const u32x4 sv = *reinterpret_cast<const u32x4*>(src + (b * n_src + (r >= 0 ? r : 0)) * C + c0);
+  const u32x4 av = *reinterpret_cast<const u32x4*>(add + (b * n_q + q) * C + c0);
+  float f[8], g[8];
+  unpack8(sv, f);
+  unpack8(av, g);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = (r >= 0 ? f[e] : 0.f) + g[e];
+  *reinterpret_cast<u32x4*>(out + (b * n_q + q) * C + c0) = pack8(f);
+}
+
+// out[b][t][k] = rows[t] >= 0 ? sum_c bf16(LayerNorm(x[b][rows[t]])[c] * ln_w[c]) * w[k][c] : 0   (k < 3, C = 128)
+// One thread per output position: its row is 256 contiguous bytes.
+__global__ __launch_bounds__(256) void ln_project3_gather_kernel(const bf16_t* __restrict__ x,
+                                                                  const int* __restrict__ rows,
+                                                                  const float* __restrict__ ln_w,
+                                                                  const float* __restrict__ w, float* __restrict__ out,
+                                                                  int64_t batch, int64_t n_src, int64_t n_out) {
+  constexpr int C = 128;
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (item >= batch * n_out) return;
+  const int64_t t = item % n_out, b = item / n_out;
+  const int r = rows[t];
+  float* dst = out + item * 3;
+  if (r < 0) {
+    dst[0] = dst[1] = dst[2] = 0.f;
+    return;
+  }
+  const bf16_t* row = x + (b * n_src + r) * C;
+  float v[C];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < C / 8; ++i) {
+    unpack8(*reinterpret_cast<const u32x4*>(row + 8 * i), v + 8 * i);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += v[8 * i + e];
+  }
+  const float mean = s / (float)C;
+  float q = 0.f;
+#pragma unroll
+  for (int c = 0; c < C; ++c) { const float d = v[c] - mean; q += d * d; }
+  const float rstd = rsqrtf(q / (float)C + LN_EPS);
+  float o0 = 0.f, o1 = 0.f, o2 = 0.f;
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const float y = bf2f(f2bf((v[c] - mean) * rstd * ln_w[c]));  // the normalised row is a bf16 tensor in the eager steps
+    o0 += y * w[c];
+    o1 += y * w[C + c];
+    o2 += y * w[2 * C + c];
+  }
+  dst[0] = o0; dst[1] = o1; dst[2] = o2;
+}
+
 }  // namespace
+
+int launch_gather_rows_add(const bf16_t* src, const int* rows, const bf16_t* add, bf16_t* out, int64_t batch,
+                           int64_t n_src, int64_t n_q, int channels, hipStream_t stream) {
+  if (!src || !rows || !add || !out || batch <= 0 || n_src <= 0 || n_q <= 0 || channels <= 0 || (channels & 7))
+    return AF3_ERR_BAD_ARG;
+  if (((uintptr_t)src & 15) || ((uintptr_t)add & 15) || ((uintptr_t)out & 15)) return AF3_ERR_BAD_ARG;
+  const int64_t blocks = (batch * n_q * (channels >> 3) + 255) / 256;
+  if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  hipLaunchKernelGGL(gather_rows_add_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, src, rows, add, out, batch,
+                     n_src, n_q, channels);
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+int launch_ln_project3_gather(const bf16_t* x, const int* rows, const float* ln_w, const float* w, float* out,
+                              int64_t batch, int64_t n_src, int64_t n_out, int channels, hipStream_t stream) {
+  if (!x || !rows || !ln_w || !w || !out || batch <= 0 || n_src <= 0 || n_out <= 0) return AF3_ERR_BAD_ARG;
+  if (channels != 128) return AF3_ERR_UNSUPPORTED;
+  if ((uintptr_t)x & 15) return AF3_ERR_BAD_ARG;
+  const int64_t blocks = (batch * n_out + 255) / 256;
+  if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  hipLaunchKernelGGL(ln_project3_gather_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, rows, ln_w, w, out, batch,
+                     n_src, n_out);
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
 
 int launch_atom_position_features(const float* pos, const int* rows, const float* w, const float* cond, void* out,
                                   int out_f32, int64_t batch, int64_t n_slots, int64_t n_q, int channels,

@@ -30,6 +30,8 @@ SIGNATURES = {
     "af3_batched_nt_product_forward": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "af3_transpose_bf16_forward": (_i, [_vp, _vp, _i64, _i64, _vp]),
     "af3_atom_position_features_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i64, _i, _vp]),
+    "af3_gather_rows_add_forward": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i, _vp]),
+    "af3_position_update_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i, _vp]),
     "af3_gathered_relu_mean_forward": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i, _i, _vp]),
     "af3_batch_diffusion_cross_attention_workspace_bytes": (_sz, [_i64, _i64, _i64, _i]),
     "af3_batch_diffusion_cross_attention_forward": (

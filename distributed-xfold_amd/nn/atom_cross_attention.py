@@ -280,7 +280,8 @@ class AtomCrossAttDecoder(HipModule):
 
     def _pack(self):
         return dict(w_bcast=bf16(self.project_token_features_for_broadcast.weight),
-                    ln_w=f32(self.atom_features_layer_norm.weight))
+                    ln_w=f32(self.atom_features_layer_norm.weight),
+                    w_upd=f32(self.atom_features_to_position_update.weight))
 
     @torch.no_grad()
     def conditioning(self, enc, queries_to_keys=None):
@@ -307,15 +308,44 @@ class AtomCrossAttDecoder(HipModule):
         # conversion to the query layout is the gather of token rows
         ta2q = aca.token_atoms_to_queries
         n_dense = aca.queries_to_token_atoms.gather_idxs.shape[1]
-        q_act = convert(GatherInfo(ta2q.gather_idxs // n_dense, ta2q.gather_mask, (t.shape[-2],)), t, (-2,))
-        q_act = q_act + enc.skip_connection.to(q_act.dtype)
-        qm = enc.queries_mask.to(q_act.dtype)
+        qm = enc.queries_mask.to(t.dtype)
         qm = qm[None, ..., None] if batched else qm[..., None]
-        q_act = (q_act * qm).to(enc.skip_connection.dtype).contiguous()
+        fused = not in_check_mode() and enc.skip_connection.dtype == torch.bfloat16
+        if fused:
+            # gather, + skip connection and query mask in one pass (the skip connection is zero where the mask is)
+            rows = getattr(ta2q, "_af3_token_rows32", None)
+            if rows is None or rows.device != t.device:
+                live = ta2q.gather_mask & (enc.queries_mask != 0)
+                rows = torch.where(live, ta2q.gather_idxs // n_dense, -1).to(torch.int32).reshape(-1).contiguous()
+                try:
+                    ta2q._af3_token_rows32 = rows
+                except AttributeError:
+                    pass
+            skip = enc.skip_connection
+            q_act = ops.gather_rows_add(t.reshape(-1, t.shape[-2], t.shape[-1]), rows,
+                                        skip.reshape(-1, rows.shape[0], skip.shape[-1]).contiguous()).view(skip.shape)
+        else:
+            q_act = convert(GatherInfo(ta2q.gather_idxs // n_dense, ta2q.gather_mask, (t.shape[-2],)), t, (-2,))
+            q_act = q_act + enc.skip_connection.to(q_act.dtype)
+            q_act = (q_act * qm.to(q_act.dtype)).to(enc.skip_connection.dtype).contiguous()
         q_act = self.atom_transformer_decoder(
             queries_act=q_act, queries_mask=enc.queries_mask, queries_to_keys=aca.queries_to_keys,
             keys_mask=enc.keys_mask, queries_single_cond=enc.queries_single_cond,
             keys_single_cond=enc.keys_single_cond, pair_cond=enc.pair_cond, cond=transformer_cond)
+        if fused:
+            # LayerNorm, projection to the position update and conversion to the token-atom layout in one
+            # pass over the atoms that exist (their query mask is one)
+            gi = aca.queries_to_token_atoms
+            rows = getattr(gi, "_af3_rows32_flat", None)
+            if rows is None or rows.device != q_act.device:
+                rows = torch.where(gi.gather_mask, gi.gather_idxs, -1).to(torch.int32).reshape(-1).contiguous()
+                try:
+                    gi._af3_rows32_flat = rows
+                except AttributeError:
+                    pass
+            n_src = q_act.shape[-3] * q_act.shape[-2]
+            upd = ops.position_update(q_act.reshape(-1, n_src, q_act.shape[-1]), rows, p["ln_w"], p["w_upd"])
+            return upd.view(*q_act.shape[:-3], *gi.gather_idxs.shape, 3)
         q_act = q_act * qm.to(q_act.dtype)
         if in_check_mode():
             q_act = check._ln(q_act.contiguous(), self.atom_features_layer_norm)

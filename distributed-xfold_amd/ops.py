@@ -233,6 +233,53 @@ def atom_position_features(positions, rows, weight, cond, out_dtype=torch.bfloat
     return out
 
 
+def _rows32(rows, n_src, device, name="rows"):
+    if rows.dtype != torch.int32 or rows.dim() != 1 or not rows.is_contiguous() or rows.device != device:
+        raise ValueError(f"{name}: expected a contiguous int32 vector on the device of the data")
+    if getattr(rows, "_af3_checked_rows", None) != n_src:
+        if int(rows.max()) >= n_src:
+            raise ValueError(f"{name}: row index beyond the source")
+        rows._af3_checked_rows = n_src             # one device round trip per index tensor
+
+
+def gather_rows_add(src, rows, add):
+    """out[b, q] = (src[b, rows[q]] if rows[q] >= 0 else 0) + add[b, q], all bf16
+    (af3_gather_rows_add_forward).  src [B, n_src, C], rows [Q] int32, add [B, Q, C]."""
+    lib = _L.load()
+    _gpu(src, "src", torch.bfloat16)
+    if src.dim() != 3:
+        raise ValueError("src: expected [B, n_src, C]")
+    b, n_src, c = src.shape
+    _rows32(rows, n_src, src.device)
+    q = rows.shape[0]
+    _gpu(add, "add", torch.bfloat16, (b, q, c))
+    if c % 8:
+        raise ValueError("channels must be a multiple of 8")
+    out = torch.empty_like(add)
+    rc = lib.af3_gather_rows_add_forward(_p(src), _p(rows), _p(add), _p(out), b, n_src, q, c, _stream(src.device))
+    _L.check(rc, "af3_gather_rows_add_forward")
+    return out
+
+
+def position_update(x, rows, ln_weight, weight):
+    """out[b, t] = weight @ bf16(LayerNorm(x[b, rows[t]]) * ln_weight), zeros where rows[t] < 0
+    (af3_position_update_forward).  x [B, n_src, 128] bf16, rows [T] int32, ln_weight [128],
+    weight [3, 128] fp32 -> [B, T, 3] fp32."""
+    lib = _L.load()
+    _gpu(x, "x", torch.bfloat16)
+    if x.dim() != 3 or x.shape[-1] != 128:
+        raise ValueError("x: expected [B, n_src, 128]")
+    b, n_src, c = x.shape
+    _rows32(rows, n_src, x.device)
+    _gpu(ln_weight, "ln_weight", torch.float32, (c,))
+    _gpu(weight, "weight", torch.float32, (3, c))
+    out = torch.empty((b, rows.shape[0], 3), dtype=torch.float32, device=x.device)
+    rc = lib.af3_position_update_forward(_p(x), _p(rows), _p(ln_weight), _p(weight), _p(out), b, n_src,
+                                         rows.shape[0], c, _stream(x.device))
+    _L.check(rc, "af3_position_update_forward")
+    return out
+
+
 def gathered_relu_mean(src, idx, count):
     """out[b, t] = sum_a relu(src[b, idx[t, a]]) / count[t] over the slots with idx >= 0
     (af3_gathered_relu_mean_forward).  src [B, n_src, C] bf16, idx [T, A] int32,

@@ -242,6 +242,36 @@ int af3_atom_position_features_forward(const float* positions, const int32_t* ro
                                        int64_t n_queries, int channels, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Broadcast of the token activations to the atoms at the head of the atom
+ * cross-attention decoder (nn/d_atom_cross_attention.py:371-392: the projected
+ * token rows converted to the query layout, + the encoder's skip connection,
+ * query mask):
+ *   out[b][q][c] = (rows[q] >= 0 ? src[b][rows[q]][c] : 0) + add[b][q][c]
+ * src [batch][n_src][channels] bf16 (one row per token), rows [n_queries] int32
+ * (token of the query's atom, negative for none), add and out
+ * [batch][n_queries][channels] bf16 (the skip connection is zero where the
+ * query mask is, so no further masking is needed).  The sum is taken in fp32
+ * and rounded once.
+ */
+int af3_gather_rows_add_forward(const uint16_t* src, const int32_t* rows, const uint16_t* add, uint16_t* out,
+                                int64_t batch, int64_t n_src, int64_t n_queries, int channels, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * The tail of the atom cross-attention decoder
+ * (nn/d_atom_cross_attention.py:404-414: LayerNorm of the query activations,
+ * projection to a position update, conversion to the token-atom layout):
+ *   out[b][t][k] = rows[t] >= 0 ? sum_c y[c] * weight[k][c] : 0,   k = 0..2,
+ *   y = LayerNorm(x[b][rows[t]]) * ln_weight, rounded to bf16 as the eager
+ *   LayerNorm output is.
+ * x [batch][n_src][128] bf16, rows [n_out] int32 (query of the atom slot, or
+ * negative for an absent atom), ln_weight [128] fp32, weight [3][128] fp32,
+ * out [batch][n_out][3] fp32.  channels must be 128.
+ */
+int af3_position_update_forward(const uint16_t* x, const int32_t* rows, const float* ln_weight, const float* weight,
+                                float* out, int64_t batch, int64_t n_src, int64_t n_out, int channels,
+                                af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Pair-logit projection: out[h][i][j] = (LayerNorm(pair)[i][j] . w[h]).
  * Replaces the eager `single_pair_logits_projection(single_pair_logits_norm(
  * pair)).permute(2,0,1)` of nn/d_pairformer.py:160-162 and the

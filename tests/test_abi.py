@@ -131,6 +131,10 @@ def test_gathered_relu_mean_rejects_bad_arguments(pkg):
     assert lib.af3_gathered_relu_mean_forward(one, one, one, one, 1, 8, 8, 4, 100, None) == -1     # channels % 8
     assert lib.af3_gathered_relu_mean_forward(one + 2, one, one, one, 1, 8, 8, 4, 128, None) == -1  # misaligned
     assert lib.af3_atom_position_features_forward(one, None, one, one, one, 0, 1, 8, 8, 128, None) == -1   # no rows
+    assert lib.af3_gather_rows_add_forward(one, one, None, one, 1, 8, 8, 128, None) == -1                   # no addend
+    assert lib.af3_gather_rows_add_forward(one, one, one, one, 1, 8, 8, 100, None) == -1                    # channels % 8
+    assert lib.af3_position_update_forward(one, one, one, one, one, 1, 8, 8, 64, None) != 0                  # channels != 128
+    assert lib.af3_position_update_forward(one, None, one, one, one, 1, 8, 8, 128, None) == -1               # no rows
     assert lib.af3_atom_position_features_forward(one, one, one, one, one, 2, 1, 8, 8, 128, None) == -1    # dtype
     assert lib.af3_atom_position_features_forward(one, one, one, one, one, 0, 1, 8, 8, 100, None) == -1    # channels % 8
 

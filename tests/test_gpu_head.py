@@ -257,3 +257,36 @@ def test_head_without_batch_inference_matches_the_batched_head(gpu_pkg):
         err = float((got - want[i]).abs().max()) / float(want[i].abs().max())
         print(f"unbatched head, sample {i}: max difference {err:.3e}", flush=True)
         assert err <= 1e-6
+
+
+def test_decoder_layout_kernels(gpu_pkg):
+    """The two fused steps of the atom decoder against the same steps in torch:
+    token rows gathered to the queries + skip connection (bit-identical), and
+    LayerNorm -> position update -> token-atom layout."""
+    print("test_decoder_layout_kernels", flush=True)
+    g = torch.Generator().manual_seed(5)
+    d = torch.device("cuda:0")
+    b, n_tok, q, c = 3, 50, 416, 128
+    src = torch.randn(b, n_tok, c, generator=g).bfloat16()
+    add = torch.randn(b, q, c, generator=g).bfloat16()
+    tok = torch.randint(0, n_tok, (q,), generator=g)
+    live = torch.rand(q, generator=g) > 0.25
+    rows = torch.where(live, tok, -1).to(torch.int32)
+    got = gpu_pkg.ops.gather_rows_add(src.to(d), rows.to(d), add.to(d)).cpu()
+    want = (src[:, tok] * live[None, :, None].to(torch.bfloat16)) + add
+    assert torch.equal(got, want)
+    # position update
+    x = (torch.randn(b, q, c, generator=g) * 2 + 0.3).bfloat16()
+    ln_w, w = torch.randn(c, generator=g), torch.randn(3, c, generator=g) * 0.1
+    t_out = 77
+    qi = torch.randint(0, q, (t_out,), generator=g)
+    present = torch.rand(t_out, generator=g) > 0.3
+    rows2 = torch.where(present, qi, -1).to(torch.int32)
+    got = gpu_pkg.ops.position_update(x.to(d), rows2.to(d), ln_w.to(d), w.to(d)).cpu()
+    y = torch.nn.functional.layer_norm(x.double(), (c,), ln_w.double(), None, 1e-5).float().bfloat16().double()
+    want = (y @ w.double().T)[:, qi] * present[None, :, None]
+    assert got.shape == (b, t_out, 3)
+    err = float((got.double() - want).abs().max()) / float(want.abs().max())
+    print(f"  position update: max difference {err:.3e} of the largest value", flush=True)
+    assert err <= 2e-3        # a bf16 rounding of a normalised value may fall the other way
+    assert torch.all(got[:, ~present] == 0)
