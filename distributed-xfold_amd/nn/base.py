@@ -86,10 +86,11 @@ class HipModule(nn.Module):
         self._packed = None
 
     def invalidate(self):
-        self._packed = None
-        for m in self.children():
+        """Drop the packed weights of this module and of every HIP module below
+        it, however deeply nested (blocks usually sit in an nn.ModuleList)."""
+        for m in self.modules():
             if isinstance(m, HipModule):
-                m.invalidate()
+                m._packed = None
 
     def _apply(self, fn, *a, **k):  # .to() / .cuda() move parameters: repack afterwards
         self._packed = None
@@ -103,10 +104,9 @@ class HipModule(nn.Module):
         raise NotImplementedError
 
     def load_hip_params(self):
-        self._packed = self._pack()
-        for m in self.children():
+        for m in self.modules():
             if isinstance(m, HipModule):
-                m.load_hip_params()
+                m._packed = m._pack()
         return self
 
     def packed(self):

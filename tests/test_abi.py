@@ -236,3 +236,31 @@ def test_library_is_not_older_than_its_sources(pkg):
     srcs = [os.path.join(csrc, f) for f in os.listdir(csrc) if f.endswith((".hip", ".h"))] + [HEADER]
     stale = [os.path.basename(f) for f in srcs if os.path.getmtime(f) > so_time + 1]
     assert not stale, f"rebuild libaf3hip.so (make -C {csrc}): newer sources {stale}"
+
+
+def test_weight_reload_reaches_blocks_inside_module_lists(pkg):
+    """Packed device weights are a cache of the nn.Parameters.  A reload through
+    a container (blocks live in nn.ModuleList) must drop every nested cache:
+    otherwise forward keeps computing with the old weights."""
+    g = torch.Generator().manual_seed(5)
+    stack = pkg.nn.PairformerStack(num_blocks=2)
+    inner = stack.trunk_pairformer[1].triangle_multiplication_outgoing
+    old = inner.packed()["w_out"].clone()
+    assert inner._packed is not None
+    new_state = {k: torch.randn(v.shape, generator=g) for k, v in stack.state_dict().items()}
+    stack.load_state_dict(new_state)
+    assert inner._packed is None
+    key = "trunk_pairformer.1.triangle_multiplication_outgoing.output_projection.weight"
+    assert torch.equal(inner.packed()["w_out"], new_state[key].to(torch.bfloat16))
+    assert not torch.equal(inner.packed()["w_out"], old)
+    # load_hip_params on the container packs every nested module as well
+    stack.invalidate()
+    assert all(m._packed is None for m in stack.modules() if isinstance(m, pkg.nn.base.HipModule))
+    stack.load_hip_params()
+    assert all(m._packed is not None for m in stack.modules() if isinstance(m, pkg.nn.base.HipModule))
+    dt = pkg.nn.DiffusionTransformer(num_blocks=2, super_block_size=2, use_batch_infer=True)
+    dt.load_hip_params()
+    blk = dt.self_attention[1]
+    assert blk._packed is not None
+    dt.load_state_dict(dt.state_dict())
+    assert blk._packed is None

@@ -38,17 +38,10 @@ pytestmark = pytest.mark.gpu
 RMS_TOL = 1e-2       # north-star bf16 tolerance, in the rms sense (see module docstring)
 TOL_EXACT = 4e-2     # loose max-norm bound used only for single rows / padded-query checks
 D = torch.float64
-LOG = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out", "parity.log")
 
 
 def note(msg):
     print(msg, flush=True)
-    try:
-        os.makedirs(os.path.dirname(LOG), exist_ok=True)
-        with open(LOG, "a") as f:
-            f.write(msg + "\n")
-    except OSError:
-        pass
 
 
 def gen(seed):

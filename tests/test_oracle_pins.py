@@ -309,6 +309,54 @@ def test_adaptive_layer_norm_forms():
 
 
 @pytest.mark.parametrize("cond", [False, True])
+def test_adaln_zero_explicit(cond):
+    """nn/d_diffusion_transformer.py:99-118 written out with plain matmuls."""
+    g = gen(31 + int(cond))
+    cin, cout, cs = 10, 6, 4
+    p = O.cast_params(O.make_adaln_zero_params(g, cin, cout, cs, cond, std=0.4), D)
+    x, s = randn(g, 2, 5, cin), randn(g, 5, cs)
+    want = x @ p["transition2.weight"].T
+    if cond:
+        z = s @ p["adaptive_zero_cond.weight"].T + p["adaptive_zero_cond.bias"]
+        want = want / (1.0 + torch.exp(-z))
+    assert torch.allclose(O.adaln_zero(x, s if cond else None, p), want, atol=1e-10)
+
+
+@pytest.mark.parametrize("cond", [False, True])
+def test_diffusion_transition_explicit(cond):
+    """DistributeDiffusionTransition.forward (nn/d_diffusion_transformer.py:142-145) restated
+    without any oracle helper: F.layer_norm, F.silu, explicit sigmoid gates, element loops
+    for the GLU pairing (hidden unit f pairs transition1 rows f and factor*c + f)."""
+    g = gen(41 + int(cond))
+    cx, cs, f = 8, 6, 2
+    p = O.cast_params(O.make_diffusion_transition_params(g, cx, cs, f, cond, std=0.4), D)
+    x, s = randn(g, 3, 5, cx), randn(g, 5, cs)
+    if cond:
+        sn = F.layer_norm(s, (cs,), p["adaptive_layernorm.single_cond_layer_norm.weight"], None, 1e-5)
+        scale = sn @ p["adaptive_layernorm.single_cond_scale.weight"].T + p["adaptive_layernorm.single_cond_scale.bias"]
+        shift = sn @ p["adaptive_layernorm.single_cond_bias.weight"].T
+        xa = torch.sigmoid(scale) * F.layer_norm(x, (cx,), None, None, 1e-5) + shift
+    else:
+        xa = F.layer_norm(x, (cx,), p["adaptive_layernorm.layer_norm.weight"],
+                          p["adaptive_layernorm.layer_norm.bias"], 1e-5)
+    w1 = p["transition1.weight"]                       # [2 f c, c]
+    hidden = torch.empty(3, 5, f * cx, dtype=D)
+    for u in range(f * cx):                            # unit u: silu(row u) * (row f c + u)
+        a = (xa * w1[u]).sum(-1)
+        b = (xa * w1[f * cx + u]).sum(-1)
+        hidden[..., u] = F.silu(a) * b
+    want = hidden @ p["adaptive_zero_init.transition2.weight"].T
+    if cond:
+        z = s @ p["adaptive_zero_init.adaptive_zero_cond.weight"].T + p["adaptive_zero_init.adaptive_zero_cond.bias"]
+        want = torch.sigmoid(z) * want
+    got = O.diffusion_transition(x, s if cond else None, p)
+    assert got.shape == (3, 5, cx)
+    assert torch.allclose(got, want, atol=1e-10)
+    # a dropped gate, a swapped GLU half or a missing shift each fail this
+    assert not torch.allclose(got, hidden[..., :cx], atol=1e-3)
+
+
+@pytest.mark.parametrize("cond", [False, True])
 def test_self_attention_vs_sdpa(cond):
     g = gen(15)
     N, c, cs, H = 9, 24, 10, 4
