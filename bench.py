@@ -99,35 +99,88 @@ def gpu_time_ms(fn, iters, warmup=2, warm_ms=0.0):
     return start.elapsed_time(stop) / iters
 
 
-def cpu_baseline(n_metric, budget_s=25.0):
-    """The CPU oracle on this host's cores: one Pairformer block, fp32, at the
-    largest of N in {128, 256, 384} that fits the time budget; scaled to the
-    metric's N by algorithmic FLOPs and flagged as such."""
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _timed(fn, max_iters, budget_s):
+    """1 warm-up + up to `max_iters` timed calls (fewer when `budget_s` runs out; at
+    least one), wall clock: the method of the reference's own kernel tests
+    (kernel_test/triangle_multiplication.py:192-231).  Returns (mean_s, min_s, iterations)."""
+    t0 = time.perf_counter()
+    fn()
+    warm = time.perf_counter() - t0
+    times = []
+    spent = warm
+    while len(times) < max_iters and (not times or spent + times[-1] <= budget_s):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+        spent += times[-1]
+    return sum(times) / len(times), min(times), len(times)
+
+
+def cpu_baseline(n_metric):
+    """The CPU oracle (this build's eager-PyTorch restatement of the reference
+    formulas; the reference's own xfold + libxsmm path cannot be built here) on
+    this host's cores, on a bounded sample: one Pairformer block at N=384 in fp32
+    and in torch.bfloat16 with all threads, and the 4-block N=128 fp32 stack with
+    all threads and with one.  `value` is the fp32 N=384 mean scaled by algorithmic
+    FLOPs to the metric's N (flagged as extrapolated)."""
     import torch
     from oracle import af3_oracle as O
     g = torch.Generator().manual_seed(0)
-    p = O.make_pairformer_block_params(g)
     threads = torch.get_num_threads()
-    measured = None
-    for n in (128, 256, 384):
-        if measured is not None:
-            est = measured[1] * flops_block(n) / flops_block(measured[0]) * 1.5
-            if est > budget_s:
-                break
-        pair, single = torch.randn(n, n, 128, generator=g), torch.randn(n, 384, generator=g)
-        seq = (torch.arange(n) < int(0.9 * n)).float()
+    affinity = len(os.sched_getaffinity(0))
+
+    def block_case(n, dtype, nblocks=1):
+        blocks = [O.cast_params(O.make_pairformer_block_params(g), dtype) for _ in range(nblocks)]
+        pair = torch.randn(n, n, 128, generator=g).to(dtype)
+        single = torch.randn(n, 384, generator=g).to(dtype)
+        seq = (torch.arange(n) < (int(0.9 * n) if nblocks == 1 else n)).to(dtype)
         pm = seq[:, None] * seq[None, :]
-        t0 = time.perf_counter()
-        with torch.no_grad():
-            O.pairformer_block(pair, pm, single, seq, p)
-        measured = (n, time.perf_counter() - t0)
-    n, secs = measured
-    scaled_ms = secs * 1e3 * flops_block(n_metric) / flops_block(n)
+
+        def run():
+            with torch.no_grad():
+                O.pairformer_stack(pair, pm, single, seq, blocks)
+        return run
+
+    legs = {}
+    n_cpu = 384
+    mean, mn, it = _timed(block_case(n_cpu, torch.float32), 10, 14.0)
+    legs["block_n384_fp32"] = {"mean_ms": round(mean * 1e3, 1), "min_ms": round(mn * 1e3, 1), "iterations": it,
+                               "threads": threads}
+    fp32_mean = mean
+    mean, mn, it = _timed(block_case(n_cpu, torch.bfloat16), 10, 8.0)
+    legs["block_n384_bf16"] = {"mean_ms": round(mean * 1e3, 1), "min_ms": round(mn * 1e3, 1), "iterations": it,
+                               "threads": threads}
+    mean, mn, it = _timed(block_case(128, torch.float32, 4), 10, 5.0)
+    legs["stack4_n128_fp32"] = {"mean_ms": round(mean * 1e3, 1), "min_ms": round(mn * 1e3, 1), "iterations": it,
+                                "threads": threads}
+    torch.set_num_threads(1)
+    try:
+        mean, mn, it = _timed(block_case(128, torch.float32, 4), 10, 6.0)
+    finally:
+        torch.set_num_threads(threads)
+    legs["stack4_n128_fp32_1thread"] = {"mean_ms": round(mean * 1e3, 1), "min_ms": round(mn * 1e3, 1),
+                                        "iterations": it, "threads": 1}
+    scaled_ms = fp32_mean * 1e3 * flops_block(n_metric) / flops_block(n_cpu)
     return {
         "value": round(scaled_ms, 1), "unit": "ms/block", "cores": threads, "kind": "port",
-        "sample": (f"CPU oracle (eager PyTorch fp32 restatement of the reference formulas), one Pairformer "
-                   f"block at N={n}: {secs * 1e3:.0f} ms measured on {threads} threads; value is that time "
-                   f"scaled by algorithmic FLOPs to N={n_metric} (extrapolated)"),
+        "extrapolated": n_metric != n_cpu,
+        "sample": (f"CPU oracle (eager PyTorch restatement of the reference formulas; not xfold+TPP, which cannot be "
+                   f"built here), 1 warm-up + up to 10 timed runs each, wall clock: one Pairformer block at "
+                   f"N={n_cpu} (10% padded) fp32 and bf16, the 4-block N=128 fp32 stack with all threads and with "
+                   f"one; value = fp32 N={n_cpu} mean ({fp32_mean * 1e3:.0f} ms on {threads} threads) scaled by "
+                   f"algorithmic FLOPs to N={n_metric} (extrapolated)"),
+        "legs": legs, "torch_threads": threads, "sched_affinity": affinity, "cpu_model": _cpu_model(),
     }
 
 

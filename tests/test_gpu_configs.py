@@ -1,0 +1,297 @@
+"""The benchmark configurations, each run on the GPU through the C ABI and
+checked:
+
+  configs[0]  4-block Pairformer stack, N=128, fp32 residual stream, masks all
+              ones                          -> float64 CPU oracle
+  configs[1]  one block, N=384, bf16, tokens 346.. masked
+                                            -> float64 CPU oracle and fp32 check mode
+  configs[2]  triangle multiplication out/in and triangle attention start/end
+              alone at N in {512, 1024}, seeded 0-15% trailing pad
+                                            -> fp32 check mode
+  configs[3]  N=1536: one block -> fp32 check mode; the 48-block trunk with
+              distinct weights stays finite and commutes with a relabelling of
+              the tokens
+plus the operator-level contract of the triangle attention entry point: an
+external fp32 `nonbatched_bias [H, N, N]` with or without the LayerNorm inside
+(the reference operator's own argument list, csrc/Alpha_Attention.cpp:182-185,
+as DistributeGridSelfAttention.xsmm_forward feeds it, nn/d_attention.py:58-85).
+
+bf16 tolerances are those of tests/test_gpu_parity.py (rms of the error over
+rms of the expected update <= 1e-2; the accepted maximum per operator is stated
+where it is asserted); fp32 storage is held to 1e-4 in the max norm only in the
+check mode, the MFMA operands being bf16 either way.
+"""
+
+import time
+
+import pytest
+import torch
+
+from oracle import af3_oracle as O
+
+pytestmark = pytest.mark.gpu
+D = torch.float64
+RMS_TOL = 1e-2
+# accepted max |err| / rms(expected) per operator for bf16 operands over 10^7..10^8 outputs
+MAX_TOL = {"trimul": 6e-2, "triattn": 6e-2, "block": 6e-2, "single": 4e-2}
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def rparams(p):
+    return {k: O.round_bf16(v) for k, v in p.items()}
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+def errs(got, ref):
+    """(max, rms) of got - ref over the rms of ref; computed where `got` lives."""
+    ref = ref.to(got.device).double()
+    got = got.double()
+    scale = float((ref * ref).mean().sqrt())
+    assert scale > 0
+    d = got - ref
+    return float(d.abs().max()) / scale, float((d * d).mean().sqrt()) / scale
+
+
+def compare(name, got, ref, rms_tol, max_tol):
+    assert torch.isfinite(got).all(), f"{name}: non-finite output"
+    mx, rms = errs(got, ref)
+    say(f"configs {name}: rms {rms:.3e} max {mx:.3e}")
+    assert rms <= rms_tol, (name, rms)
+    assert mx <= max_tol, (name, mx)
+
+
+def trailing_masks(n, live):
+    seq = (torch.arange(n) < live).float()
+    return seq, (seq[:, None] * seq[None, :]).contiguous()
+
+
+# ------------------------------------------------------------------ configs[0]
+def test_config0_four_block_stack_n128_fp32(gpu_pkg):
+    say("test_config0_four_block_stack_n128_fp32")
+    n, nb = 128, 4
+    g = gen(100)
+    blocks = [rparams(O.make_pairformer_block_params(g)) for _ in range(nb)]
+    pair = O.round_bf16(torch.randn(n, n, 128, generator=g))
+    single = O.round_bf16(torch.randn(n, 384, generator=g))
+    seq, pm = torch.ones(n), torch.ones(n, n)
+    stack = gpu_pkg.nn.PairformerStack(num_blocks=nb)
+    stack.load_state_dict({f"trunk_pairformer.{i}.{k}": v for i, p in enumerate(blocks) for k, v in p.items()})
+    stack.to(dev())
+    gp, gs = stack(pair.to(dev()).clone(), pm.to(dev()), single.to(dev()).clone(), seq.to(dev()))
+    t0 = time.perf_counter()
+    ep, es = O.pairformer_stack(pair.double(), pm.double(), single.double(), seq.double(),
+                                [O.cast_params(p, D) for p in blocks])
+    say(f"  float64 oracle, 4 blocks at N=128: {time.perf_counter() - t0:.1f} s")
+    compare("[0] stack pair update (fp32 stream)", gp.cpu() - pair, ep - pair.double(), RMS_TOL, MAX_TOL["block"])
+    compare("[0] stack single update (fp32 stream)", gs.cpu() - single, es - single.double(), RMS_TOL,
+            MAX_TOL["single"])
+    # the same stack in the fp32 check mode carries the strict bound
+    with gpu_pkg.nn.check_mode():
+        cp, cs = stack(pair.to(dev()), pm.to(dev()), single.to(dev()), seq.to(dev()))
+    compare("[0] stack pair, fp32 check mode", cp.cpu(), ep, 1e-5, 1e-4)
+    compare("[0] stack single, fp32 check mode", cs.cpu(), es, 1e-5, 1e-4)
+
+
+# ------------------------------------------------------------------ configs[1]
+def test_config1_one_block_n384_bf16_padded(gpu_pkg):
+    say("test_config1_one_block_n384_bf16_padded")
+    n, live = 384, 346
+    g = gen(101)
+    p = rparams(O.make_pairformer_block_params(g))
+    pair = O.round_bf16(torch.randn(n, n, 128, generator=g))
+    single = O.round_bf16(torch.randn(n, 384, generator=g))
+    seq, pm = trailing_masks(n, live)
+    blk = gpu_pkg.nn.PairformerBlock()
+    blk.load_state_dict(p)
+    blk.to(dev())
+    bp, bs = blk(pair.to(dev()).bfloat16(), pm.to(dev()), single.to(dev()).bfloat16(), seq.to(dev()))
+    with gpu_pkg.nn.check_mode():
+        cp, cs = blk(pair.to(dev()), pm.to(dev()), single.to(dev()), seq.to(dev()))
+    # The whole output tensor, padding included, against the check mode.  A bf16 stream is rounded once per
+    # sub-operation (2^-9 of each value, five times), which is of the order of the update itself for a block with
+    # N(0, 0.02) weights: so the bf16 stream is compared as the stream (relative to ITS rms), the update below on
+    # an fp32 stream.
+    compare("[1] pair stream, bf16 vs fp32 check", bp.float().cpu(), cp.cpu(), RMS_TOL, MAX_TOL["block"])
+    compare("[1] single stream, bf16 vs fp32 check", bs.float().cpu(), cs.cpu(), RMS_TOL, MAX_TOL["single"])
+    t0 = time.perf_counter()
+    ep, es = O.pairformer_block(pair.double(), pm.double(), single.double(), seq.double(), O.cast_params(p, D))
+    say(f"  float64 oracle, one block at N=384: {time.perf_counter() - t0:.1f} s")
+    compare("[1] pair update, fp32 check vs oracle", cp.cpu() - pair, ep - pair.double(), 1e-5, 1e-4)
+    compare("[1] single update, fp32 check vs oracle", cs.cpu() - single, es - single.double(), 1e-5, 1e-4)
+    # bf16 update against the oracle on an fp32 stream (so that only operand rounding is measured)
+    fp, fs = blk(pair.to(dev()).clone(), pm.to(dev()), single.to(dev()).clone(), seq.to(dev()))
+    lp = pm.bool()[..., None]
+    compare("[1] pair update vs oracle (live pixels)", (fp.cpu() - pair) * lp, (ep - pair.double()) * lp, RMS_TOL,
+            MAX_TOL["block"])
+    compare("[1] single update vs oracle", fs.cpu() - single, es - single.double(), RMS_TOL, MAX_TOL["single"])
+
+
+# ------------------------------------------------------------------ configs[2]
+@pytest.mark.parametrize("n", [512, 1024])
+def test_config2_triangle_operators_alone(gpu_pkg, n):
+    say(f"test_config2_triangle_operators_alone n={n}")
+    g = gen(200 + n)
+    pad = int(torch.randint(0, 16, (1,), generator=g))            # 0..15 % of the tokens, from the seed
+    live = n - n * pad // 100
+    say(f"  trailing pad {pad}% -> {live} live tokens")
+    pair = O.round_bf16(torch.randn(n, n, 128, generator=g)).to(dev())
+    _, pm = trailing_masks(n, live)
+    pm = pm.to(dev())
+    for outgoing in (True, False):
+        p = rparams(O.make_triangle_multiplication_params(g))
+        mod = gpu_pkg.nn.TriangleMultiplication(c_pair=128, _outgoing=outgoing)
+        mod.load_state_dict(p)
+        mod.to(dev())
+        got = mod(pair.bfloat16(), pm)
+        with gpu_pkg.nn.check_mode():
+            ref = mod(pair, pm)
+        compare(f"[2] trimul {'out' if outgoing else 'in'} n={n}", got.float(), ref, RMS_TOL, MAX_TOL["trimul"])
+    for transpose in (False, True):
+        p = rparams(O.make_grid_self_attention_params(g, std=0.05))
+        mod = gpu_pkg.nn.GridSelfAttention(c_pair=128, num_head=4, transpose=transpose)
+        mod.load_state_dict(p)
+        mod.to(dev())
+        got = mod(pair.bfloat16(), pm)
+        with gpu_pkg.nn.check_mode():
+            ref = mod(pair, pm)
+        lp = pm.bool()[..., None]         # rows / columns that are padding carry nothing the reference defines
+        if transpose:
+            lp = lp.transpose(0, 1)
+        compare(f"[2] triattn {'end' if transpose else 'start'} n={n}", got.float() * lp, ref * lp, RMS_TOL,
+                MAX_TOL["triattn"])
+
+
+# ------------------------------------------------------------------ configs[3]
+def test_config3_one_block_n1536_against_check_mode(gpu_pkg):
+    say("test_config3_one_block_n1536_against_check_mode")
+    n = 1536
+    g = gen(300)
+    p = rparams(O.make_pairformer_block_params(g))
+    pair = O.round_bf16(torch.randn(n, n, 128, generator=g))
+    single = O.round_bf16(torch.randn(n, 384, generator=g))
+    seq, pm = torch.ones(n), torch.ones(n, n)
+    blk = gpu_pkg.nn.PairformerBlock()
+    blk.load_state_dict(p)
+    blk.to(dev())
+    d = dev()
+    pair_d, single_d = pair.to(d), single.to(d)
+    t0 = time.perf_counter()
+    with gpu_pkg.nn.check_mode():
+        cp, cs = blk(pair_d, pm.to(d), single_d, seq.to(d))
+    torch.cuda.synchronize()
+    say(f"  fp32 check mode, one block at N=1536: {time.perf_counter() - t0:.1f} s")
+    bp, bs = blk(pair_d.clone(), pm.to(d), single_d.clone(), seq.to(d))
+    compare("[3] pair update, bf16 MFMA vs fp32 check", bp - pair_d, cp - pair_d, RMS_TOL, MAX_TOL["block"])
+    compare("[3] single update, bf16 MFMA vs fp32 check", bs - single_d, cs - single_d, RMS_TOL, MAX_TOL["single"])
+
+
+def test_config3_trunk_48_blocks_n1536_bf16(gpu_pkg):
+    """The target run: 48 Pairformer blocks with distinct random weights on one
+    resident [1536, 1536, 128] bf16 pair tensor.  Random weights make no claim
+    about values; what must hold at any depth is that the activations stay
+    finite and that relabelling the tokens relabels the result (up to the bf16
+    operand rounding of sums taken in another order, which 48 blocks compound:
+    the bound is on the rms of the difference)."""
+    say("test_config3_trunk_48_blocks_n1536_bf16")
+    n, nb = 1536, 48
+    d = dev()
+    g = gen(301)
+    stack = gpu_pkg.nn.PairformerStack(num_blocks=nb)
+    with torch.no_grad():
+        for name, prm in stack.named_parameters():
+            noise = torch.randn(prm.shape, generator=g) * 0.02
+            if prm.dim() == 1 and name.endswith("weight"):
+                noise += 1.0
+            prm.copy_(noise)
+    stack.to(d)
+    stack.load_hip_params()
+    pair = torch.randn(n, n, 128, generator=g).bfloat16().to(d)
+    single = torch.randn(n, 384, generator=g).bfloat16().to(d)
+    seq, pm = trailing_masks(n, n - 154)                      # 10 % trailing pad
+    seq, pm = seq.to(d), pm.to(d)
+    perm = torch.randperm(n, generator=g).to(d)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    op, os_ = stack(pair.clone(), pm, single.clone(), seq)
+    torch.cuda.synchronize()
+    say(f"  48 blocks at N=1536: {(time.perf_counter() - t0) * 1e3:.0f} ms (first call, includes weight packing)")
+    assert torch.isfinite(op.float()).all() and torch.isfinite(os_.float()).all()
+    upd = (op.float() - pair.float())
+    say(f"  rms of the pair stream {float(op.float().pow(2).mean().sqrt()):.3f}, of its update "
+        f"{float(upd.pow(2).mean().sqrt()):.3f}")
+    assert float(upd.pow(2).mean().sqrt()) > 0.1             # 48 blocks did move the stream
+    del upd
+    pp = pair[perm][:, perm].contiguous()
+    qp, qs = stack(pp.clone(), pm[perm][:, perm].contiguous(), single[perm].contiguous(), seq[perm].contiguous())
+    live2 = pm[perm][:, perm].bool()[..., None]
+    a = ((qp.float() - pp.float()) * live2)
+    b = ((op.float() - pair.float())[perm][:, perm] * live2)
+    mx, rms = errs(a, b)
+    say(f"configs [3] 48-block pair update under a token permutation: rms {rms:.3e} max {mx:.3e}")
+    assert rms <= 5e-2
+    live1 = seq[perm].bool()[:, None]
+    mx, rms = errs((qs.float() - single[perm].float()) * live1, (os_.float() - single.float())[perm] * live1)
+    say(f"configs [3] 48-block single update under a token permutation: rms {rms:.3e} max {mx:.3e}")
+    assert rms <= 5e-2
+
+
+# ------------------------------------------- operator-level triangle attention
+@pytest.mark.parametrize("n,transpose,skip_ln", [(37, False, False), (37, True, False), (130, False, True),
+                                                 (130, True, True), (130, True, False)])
+def test_grid_self_attn_operator_level_external_bias(gpu_pkg, n, transpose, skip_ln):
+    """af3_grid_self_attn_forward with the reference operator's own operands: a
+    precomputed fp32 nonbatched_bias [H, N, N] taken from the UN-transposed
+    LayerNorm(pair) (nn/d_attention.py:60-62), and optionally an input that the
+    caller has normalised already (act_norm_* = NULL).  Must agree with the
+    fused branch (bias projected inside) and with the oracle."""
+    say(f"test_grid_self_attn_operator_level_external_bias n={n} transpose={transpose} skip_ln={skip_ln}")
+    g = gen(400 + n + int(transpose) + 2 * int(skip_ln))
+    p = rparams(O.make_grid_self_attention_params(g, std=0.1))
+    pair = O.round_bf16(torch.randn(n, n, 128, generator=g))
+    mask = (torch.rand(n, n, generator=g) > 0.2).float()
+    mask[:, 0] = 1
+    pd = O.cast_params(p, D)
+    exact = O.grid_self_attention(pair.double(), mask.double(), pd, 4, transpose)
+    with O.bf16_emulation():
+        emu = O.grid_self_attention(pair.double(), mask.double(), pd, 4, transpose)
+    mod = gpu_pkg.nn.GridSelfAttention(c_pair=128, num_head=4, transpose=transpose)
+    mod.load_state_dict(p)
+    mod.to(dev())
+    pk = mod.packed()
+    d = dev()
+    x_ln = O.layer_norm(pair.double(), pd["act_norm.weight"], pd["act_norm.bias"])
+    bias = (O.round_bf16(x_ln.float()).double() @ pd["pair_bias_projection.weight"].T).permute(2, 0, 1)
+    bias = bias.float().contiguous().to(d)                        # [H, q, k], un-transposed frame
+    fused = gpu_pkg.ops.grid_self_attn(pair.to(d), mask.to(d), transpose, pk["ln_w"], pk["ln_b"], pk["w_bias"], None,
+                                       pk["w_qkvg"], pk["w_out"], 4)
+    if skip_ln:
+        src = O.round_bf16(x_ln.float()).to(d)                    # the caller normalised (and rounded) already
+        got = gpu_pkg.ops.grid_self_attn(src, mask.to(d), transpose, None, None, None, bias,
+                                         pk["w_qkvg"], pk["w_out"], 4)
+    else:
+        got = gpu_pkg.ops.grid_self_attn(pair.to(d), mask.to(d), transpose, pk["ln_w"], pk["ln_b"], None, bias,
+                                         pk["w_qkvg"], pk["w_out"], 4)
+    e_max, e_rms = errs(got.cpu(), exact)
+    n_max, n_rms = errs(emu, exact)
+    f_max, f_rms = errs(got.cpu(), fused.cpu())
+    say(f"  operator-level vs oracle rms {e_rms:.3e} max {e_max:.3e} | emulation floor rms {n_rms:.3e} max "
+        f"{n_max:.3e} | vs fused branch rms {f_rms:.3e} max {f_max:.3e}")
+    assert e_rms <= RMS_TOL and e_rms <= 1.3 * n_rms + 3e-4
+    assert e_max <= 1.6 * n_max + 5e-3
+    assert f_rms <= RMS_TOL
+    # residual form writes pair + update in place
+    if not skip_ln:
+        acc = pair.to(d).clone()
+        gpu_pkg.ops.grid_self_attn(acc, mask.to(d), transpose, pk["ln_w"], pk["ln_b"], None, bias,
+                                   pk["w_qkvg"], pk["w_out"], 4, residual=True)
+        assert torch.allclose(acc - pair.to(d), got, atol=2e-6 * float(pair.abs().max()) + 1e-6)
