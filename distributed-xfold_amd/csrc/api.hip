@@ -2,6 +2,7 @@
 // workspace carving and kernel sequencing.  No allocation, no synchronisation.
 #include "../../include/af3_hip.h"
 #include "kernels.h"
+#include <mutex>
 
 namespace {
 
@@ -30,6 +31,41 @@ inline bool misaligned(const void* p) { return ((uintptr_t)p & 15) != 0; }
 
 }  // namespace
 
+// ---------------------------------------------------------------------------
+// Library-owned scratch of the allocation-free entry point.  The array lives in
+// this code object's device data segment: every GPU the library runs on holds
+// its own copy, at its own address, from the moment the code object is loaded
+// there until the process ends.  In host code the NAME `scratch` is only a
+// handle for hipGetSymbolAddress, never an address a kernel could use; the
+// device address is looked up once per device and kept.
+// ---------------------------------------------------------------------------
+constexpr size_t STATIC_SCRATCH_BYTES = AF3_STATIC_SCRATCH_BYTES;   // 32 MiB
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_lock;
+void* scratch_dev_ptr[MAX_DEVICES] = {};
+
+// Device address of `scratch` on the CURRENT device, or null on failure.
+void* static_scratch_ptr() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> hold(scratch_lock);
+  if (!scratch_dev_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    scratch_dev_ptr[dev] = p;
+  }
+  return scratch_dev_ptr[dev];
+}
+
+}  // namespace
+
 extern "C" {
 
 int af3_abi_version(void) { return 1; }
@@ -41,6 +77,7 @@ const char* af3_error_string(int code) {
     case AF3_ERR_WORKSPACE: return "workspace missing or too small";
     case AF3_ERR_LAUNCH: return "kernel launch failed";
     case AF3_ERR_UNSUPPORTED: return "unsupported shape (channels / head dimension)";
+    case AF3_ERR_TOO_LARGE: return "problem exceeds the library-owned scratch of the allocation-free entry point";
     default: return "unknown error";
   }
 }
@@ -205,11 +242,12 @@ size_t af3_batch_diffusion_self_attention_workspace_bytes(int64_t batch, int64_t
   return align_up((size_t)batch * seq * 4 * channels * sizeof(bf16_t), 256);
 }
 
-int af3_batch_diffusion_self_attention_forward(
-    const uint16_t* q_data, const float* key_mask, int64_t mask_batches, const float* nonbatched_bias,
-    int bias_quad_major, const uint16_t* w_qkvg, const float* query_b, int num_head,
-    void* out, int out_dtype, int64_t batch, int64_t seq, int channels,
-    void* workspace, size_t workspace_bytes, af3_stream_t stream) {
+// Argument checks and the two launches (q/k/v/gate product, flash kernel) shared by the
+// workspace-taking entry point and the allocation-free one: `qkvg` is the scratch
+// [batch * seq][4 * channels] bf16, wherever it lives.
+static int self_attention_args_ok(
+    const uint16_t* q_data, const float* key_mask, int64_t mask_batches, int bias_quad_major,
+    const uint16_t* w_qkvg, void* out, int out_dtype, int num_head, int64_t batch, int64_t seq, int channels) {
   if (!q_data || !w_qkvg || !out) return AF3_ERR_BAD_ARG;
   if (bias_quad_major != 0 && (bias_quad_major != 1 || (seq & 3))) return AF3_ERR_BAD_ARG;
   if (bad_dtype(out_dtype) || batch <= 0 || seq <= 0 || channels <= 0 || (channels & 7) || num_head <= 0 ||
@@ -219,11 +257,14 @@ int af3_batch_diffusion_self_attention_forward(
   if (key_mask && mask_batches != 1 && mask_batches != batch) return AF3_ERR_BAD_ARG;
   const int d = channels / num_head;
   if (d != 16 && d != 24 && d != 32 && d != 48) return AF3_ERR_UNSUPPORTED;
-  Carver ws(workspace, workspace_bytes);
-  bf16_t* qkvg = ws.take<bf16_t>((size_t)batch * seq * 4 * channels);
-  if (!ws.ok) return AF3_ERR_WORKSPACE;
-  hipStream_t s = static_cast<hipStream_t>(stream);
+  return AF3_OK;
+}
 
+static int self_attention_run(
+    const uint16_t* q_data, const float* key_mask, int64_t mask_batches, const float* nonbatched_bias,
+    int bias_quad_major, const uint16_t* w_qkvg, const float* query_b, int num_head,
+    void* out, int out_dtype, int64_t batch, int64_t seq, int channels, bf16_t* qkvg, hipStream_t s) {
+  const int d = channels / num_head;
   GemmArgs g;
   g.A = q_data; g.B = w_qkvg; g.C = qkvg;
   g.M = (int)(batch * seq); g.N = 4 * channels; g.K = channels;
@@ -245,6 +286,38 @@ int af3_batch_diffusion_self_attention_forward(
   if (bias_quad_major) { f.bias_sq = 4; f.bias_squad = seq * 4; }
   f.key_mask = key_mask; f.km_sb = mask_batches == batch && batch > 1 ? seq : 0;
   return launch_flash_attention(f, s);
+}
+
+int af3_batch_diffusion_self_attention_forward(
+    const uint16_t* q_data, const float* key_mask, int64_t mask_batches, const float* nonbatched_bias,
+    int bias_quad_major, const uint16_t* w_qkvg, const float* query_b, int num_head,
+    void* out, int out_dtype, int64_t batch, int64_t seq, int channels,
+    void* workspace, size_t workspace_bytes, af3_stream_t stream) {
+  int rc = self_attention_args_ok(q_data, key_mask, mask_batches, bias_quad_major, w_qkvg, out, out_dtype, num_head,
+                                  batch, seq, channels);
+  if (rc) return rc;
+  Carver ws(workspace, workspace_bytes);
+  bf16_t* qkvg = ws.take<bf16_t>((size_t)batch * seq * 4 * channels);
+  if (!ws.ok) return AF3_ERR_WORKSPACE;
+  return self_attention_run(q_data, key_mask, mask_batches, nonbatched_bias, bias_quad_major, w_qkvg, query_b,
+                            num_head, out, out_dtype, batch, seq, channels, qkvg, static_cast<hipStream_t>(stream));
+}
+
+int af3_batch_diffusion_self_attention_forward_static(
+    const uint16_t* q_data, const float* key_mask, int64_t mask_batches, const float* nonbatched_bias,
+    int bias_quad_major, const uint16_t* w_qkvg, const float* query_b, int num_head,
+    void* out, int out_dtype, int64_t batch, int64_t seq, int channels, af3_stream_t stream) {
+  int rc = self_attention_args_ok(q_data, key_mask, mask_batches, bias_quad_major, w_qkvg, out, out_dtype, num_head,
+                                  batch, seq, channels);
+  if (rc) return rc;
+  const size_t need = align_up((size_t)batch * seq * 4 * channels * sizeof(bf16_t), 256);
+  if (need > STATIC_SCRATCH_BYTES) return AF3_ERR_TOO_LARGE;
+  bf16_t* qkvg = static_cast<bf16_t*>(static_scratch_ptr());
+  if (!qkvg) return AF3_ERR_LAUNCH;
+  // The q/k/v/gate product writes every element of [batch * seq][4 * channels] before the attention kernel reads
+  // any of them, so nothing left in the array by an earlier (possibly larger) call is ever read: no clearing.
+  return self_attention_run(q_data, key_mask, mask_batches, nonbatched_bias, bias_quad_major, w_qkvg, query_b,
+                            num_head, out, out_dtype, batch, seq, channels, qkvg, static_cast<hipStream_t>(stream));
 }
 
 // -------------------------------------------------------------------- transpose

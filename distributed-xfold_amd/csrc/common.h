@@ -10,6 +10,7 @@
 #define AF3_ERR_WORKSPACE (-2)
 #define AF3_ERR_LAUNCH (-3)
 #define AF3_ERR_UNSUPPORTED (-4)
+#define AF3_ERR_TOO_LARGE (-5)
 
 typedef uint16_t bf16_t;  // raw bf16 bits in memory
 

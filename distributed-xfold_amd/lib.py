@@ -9,6 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libaf3hip.so")
 
 AF3_BF16, AF3_F32 = 0, 1
+STATIC_SCRATCH_BYTES = 32 << 20      # AF3_STATIC_SCRATCH_BYTES
 LINEAR_PLAIN, LINEAR_SWIGLU, LINEAR_GATE_RES, LINEAR_REGROUP32, LINEAR_ROWGATE_RES = 0, 2, 3, 4, 5
 
 _vp, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
@@ -27,6 +28,8 @@ SIGNATURES = {
     "af3_batch_diffusion_self_attention_workspace_bytes": (_sz, [_i64, _i64, _i]),
     "af3_batch_diffusion_self_attention_forward": (
         _i, [_vp, _vp, _i64, _vp, _i, _vp, _vp, _i, _vp, _i, _i64, _i64, _i, _vp, _sz, _vp]),
+    "af3_batch_diffusion_self_attention_forward_static": (
+        _i, [_vp, _vp, _i64, _vp, _i, _vp, _vp, _i, _vp, _i, _i64, _i64, _i, _vp]),
     "af3_batched_nt_product_forward": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "af3_transpose_bf16_forward": (_i, [_vp, _vp, _i64, _i64, _vp]),
     "af3_atom_position_features_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i64, _i, _vp]),

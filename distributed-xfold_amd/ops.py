@@ -170,8 +170,10 @@ def transition128(act, layernorm_weight, layernorm_bias, w1_packed, w2, residual
 
 
 def batch_diffusion_self_attention(q_data, key_mask, nonbatched_bias, w_qkvg, query_b, num_head,
-                                   out_dtype=torch.bfloat16):
+                                   out_dtype=torch.bfloat16, out=None, static_scratch=False):
     """batch_diffusion_self_attention_forward (csrc/Alpha_Attention.cpp:72-92).
+    With `static_scratch` (and a caller-provided `out`) the call goes to the
+    allocation-free entry point, whose scratch is a device array the library owns.
     q_data [B, S, C] bf16 (already normalised); key_mask [S] (shared) or [B, S];
     nonbatched_bias [H, S, S] fp32, or [H, S/4, S, 4] as `quad_major_bias` makes it;
     returns [B, S, H, C/H]."""
@@ -195,7 +197,17 @@ def batch_diffusion_self_attention(q_data, key_mask, nonbatched_bias, w_qkvg, qu
     _gpu(w_qkvg, "w_qkvg", torch.bfloat16, (4 * c, c))
     if query_b is not None:
         _gpu(query_b, "query_b", torch.float32, (c,))
-    out = torch.empty((b, s, num_head, c // num_head), dtype=out_dtype, device=q_data.device)
+    if out is None:
+        out = torch.empty((b, s, num_head, c // num_head), dtype=out_dtype, device=q_data.device)
+    else:
+        _gpu(out, "out", out_dtype, (b, s, num_head, c // num_head))
+    if static_scratch:
+        # allocation-free entry point: the scratch is the library's own device array
+        rc = lib.af3_batch_diffusion_self_attention_forward_static(
+            _p(q_data), _p(km), mask_batches, _p(nonbatched_bias), quad_major, _p(w_qkvg), _p(query_b),
+            int(num_head), _p(out), _dt(out), b, s, c, _stream(q_data.device))
+        _L.check(rc, "af3_batch_diffusion_self_attention_forward_static")
+        return out
     nbytes = lib.af3_batch_diffusion_self_attention_workspace_bytes(b, s, c)
     ws = _ws(nbytes, q_data.device)
     rc = lib.af3_batch_diffusion_self_attention_forward(

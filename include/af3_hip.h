@@ -36,6 +36,7 @@ extern "C" {
 #define AF3_ERR_WORKSPACE (-2)
 #define AF3_ERR_LAUNCH (-3)
 #define AF3_ERR_UNSUPPORTED (-4)
+#define AF3_ERR_TOO_LARGE (-5)
 
 #define AF3_BF16 0
 #define AF3_F32 1
@@ -142,6 +143,32 @@ int af3_batch_diffusion_self_attention_forward(
     int bias_quad_major, const uint16_t* w_qkvg, const float* query_b, int num_head,
     void* out, int out_dtype, int64_t batch, int64_t seq, int channels,
     void* workspace, size_t workspace_bytes, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * The same operator for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops (the diffusion sampler evaluates this attention
+ * 24 x 200 times per batch), harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  Arguments and result are exactly those of
+ * af3_batch_diffusion_self_attention_forward minus the workspace: the q / k /
+ * v / gate scratch [batch * seq][4 * channels] bf16 lives in a device array the
+ * library owns (AF3_STATIC_SCRATCH_BYTES on every GPU the library is used on,
+ * held until the process ends).  The call allocates and frees nothing.
+ * Limit: batch * seq * channels * 8 bytes <= AF3_STATIC_SCRATCH_BYTES (e.g. 5
+ * samples x 768 tokens x 768 channels, or 1536 tokens x 384 channels);
+ * beyond it the call returns AF3_ERR_TOO_LARGE and enqueues nothing.
+ * All calls on one GPU share that GPU's array: calls that may overlap in time
+ * on one GPU (different streams, different threads) race on it - serialise
+ * them, or use the workspace-taking entry point.  The array keeps the previous
+ * call's contents; nothing in it needs clearing (every element a call reads
+ * was written by that call first).  The first call on a device looks the
+ * array's device address up (no allocation); make that call outside of graph
+ * capture.
+ */
+#define AF3_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+int af3_batch_diffusion_self_attention_forward_static(
+    const uint16_t* q_data, const float* key_mask, int64_t mask_batches, const float* nonbatched_bias,
+    int bias_quad_major, const uint16_t* w_qkvg, const float* query_b, int num_head,
+    void* out, int out_dtype, int64_t batch, int64_t seq, int channels, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
  * Windowed (atom) cross-attention without output projection.  Replaces
