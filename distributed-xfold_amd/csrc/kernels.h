@@ -159,23 +159,29 @@ struct FlashArgs {
 };
 int launch_flash_attention(const FlashArgs& a, hipStream_t stream);
 
-// ---------------------------------------------------------------- triattn.hip
-// Head-major scratch of the triangle-attention fast path (all bf16):
-//   q, k, g [b][h][s][32];  vt [b][h][32][ldn];  bias [h][q][ldn] (times log2 e, pad columns zero)
-// Pair bias of the triangle attention in MFMA-fragment order.  The attention
-// core adds the bias through the matrix unit (S^T += I * bias^T) and wants, per
-// (head, 32-query block, 64-key tile), the four B fragments of that product as
-// four contiguous 1 KB runs: element (h, q, k) lives at
-//   ((((h * QB + q / 32) * KT + k / 64) * 4 + (k % 64) / 16) * 32 + q % 32) * 16 + k % 16
-// with QB = ceil(N / 32), KT = ceil(N / 64); entries whose key is >= N are zero.
+// ------------------------------------------- triattn.hip, triattn_core.hip
+// Scratch of the triangle-attention fast path, in the frame of the (possibly
+// transposed) operator, rows b:
+//   q, k, g  bf16 [b][h][s][32]   (q times log2(e)/sqrt(32); g = sigmoid gate)
+//   vt       bf16 [b][h][32][ldn] V transposed, ldn = N rounded up to 16, columns >= N zero,
+//            key k of a row stored at column tri_vt_pos(k): inside every aligned group of 16
+//            keys the two middle quads are swapped, which makes the 8 keys one lane feeds to
+//            a P.V MFMA (k, k+1, k+2, k+3, k+8, ..., k+11 with k % 8 == 0 or 4) 16 contiguous bytes
+//   bias     fp32, pair bias times log2(e), in the order of the attention core's score
+//            accumulator: per (head, 32-query block, 64-key tile) eight contiguous 1 KB runs,
+//            run (k % 64) / 8, lane ((k % 8) / 4) * 32 + q % 32, element k % 4, so that one
+//            16-byte load per lane fills four accumulator registers of the S^T tile.
+//            Entries whose key is >= N are zero; query rows >= N of the last block are unused.
+__host__ __device__ inline int64_t tri_ldn(int64_t n) { return (n + 15) / 16 * 16; }
+__host__ __device__ inline int tri_vt_pos(int k) { return (k & ~12) | ((k & 8) >> 1) | ((k & 4) << 1); }
 __host__ __device__ inline int64_t tri_bias_qblocks(int64_t n) { return (n + 31) / 32; }
 __host__ __device__ inline int64_t tri_bias_ktiles(int64_t n) { return (n + 63) / 64; }
 __host__ __device__ inline int64_t tri_bias_elems(int64_t n, int64_t heads) {
   return heads * tri_bias_qblocks(n) * tri_bias_ktiles(n) * 2048;
 }
 __host__ __device__ inline int64_t tri_bias_offset(int64_t n, int h, int q, int k) {
-  return ((((int64_t)h * tri_bias_qblocks(n) + (q >> 5)) * tri_bias_ktiles(n) + (k >> 6)) * 4 + ((k & 63) >> 4)) * 512 +
-         (q & 31) * 16 + (k & 15);
+  return ((((int64_t)h * tri_bias_qblocks(n) + (q >> 5)) * tri_bias_ktiles(n) + (k >> 6)) * 8 + ((k & 63) >> 3)) * 256 +
+         (((k & 7) >> 2) * 32 + (q & 31)) * 4 + (k & 3);
 }
 
 struct TriAttnProjArgs {
@@ -187,14 +193,14 @@ struct TriAttnProjArgs {
   int n_bias = 0;                  // 0 or 4
   float q_scale = 1.f, bias_scale = 1.f;
   bf16_t *q = nullptr, *k = nullptr, *vt = nullptr, *g = nullptr;
-  bf16_t* bias = nullptr;  // fragment order, tri_bias_elems(N, 4) elements
-  int64_t ldn = 0;
+  float* bias = nullptr;  // accumulator order, tri_bias_elems(N, 4) elements
+  int64_t ldn = 0;        // tri_ldn(N)
 };
 int launch_triattn_proj(const TriAttnProjArgs& a, hipStream_t stream);
 
 struct TriAttnArgs {
   const bf16_t *q = nullptr, *k = nullptr, *vt = nullptr, *g = nullptr;
-  const bf16_t* bias = nullptr;  // fragment order (tri_bias_offset), or null
+  const float* bias = nullptr;   // accumulator order (tri_bias_offset), or null
   const float* mask = nullptr;   // [N][N] 0/1 or null
   bf16_t* og = nullptr;          // [(b*N + s)][128]
   int N = 0;

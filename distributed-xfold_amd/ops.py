@@ -566,36 +566,49 @@ def triangle_contraction(a, b, out=None):
 
 
 def pack_pair_bias(bias):
-    """[4, N, >=N] pair bias (already multiplied by log2(e)) -> the MFMA-fragment
-    order the attention core reads: [4, ceil(N/32), ceil(N/64), 4, 32, 16] bf16 with
-    packed[h, qb, kt, i, j, c] = bias[h, 32 qb + j, 64 kt + 16 i + c], zero where
+    """[4, N, >=N] pair bias (already multiplied by log2(e)) -> the order of the
+    attention core's score accumulator: fp32 [4, ceil(N/32), ceil(N/64), 8, 2, 32, 4] with
+    packed[h, qb, kt, g, hh, j, e] = bias[h, 32 qb + j, 64 kt + 8 g + 4 hh + e], zero where
     the query or key index is >= N."""
     if bias.dim() != 3 or bias.shape[0] != 4 or bias.shape[2] < bias.shape[1]:
         raise ValueError("bias: expected [4, N, >=N]")
     n = bias.shape[1]
     qb, kt = (n + 31) // 32, (n + 63) // 64
-    full = torch.zeros((4, qb * 32, kt * 64), dtype=torch.bfloat16, device=bias.device)
-    full[:, :n, :n] = bias[:, :, :n].to(torch.bfloat16)
-    return full.view(4, qb, 32, kt, 4, 16).permute(0, 1, 3, 4, 2, 5).contiguous()
+    full = torch.zeros((4, qb * 32, kt * 64), dtype=torch.float32, device=bias.device)
+    full[:, :n, :n] = bias[:, :, :n].to(torch.float32)
+    return full.view(4, qb, 32, kt, 8, 2, 4).permute(0, 1, 3, 4, 5, 2, 6).contiguous()
+
+
+def pack_vt(vt):
+    """[N, 4, 32, >=N] transposed values -> the column order the attention core reads:
+    bf16 [N, 4, 32, ld], ld = N rounded up to 16, key k at column
+    (k & ~12) | ((k & 8) >> 1) | ((k & 4) << 1), columns of keys >= N zero."""
+    if vt.dim() != 4 or vt.shape[1] != 4 or vt.shape[2] != 32 or vt.shape[3] < vt.shape[0]:
+        raise ValueError("vt: expected [N, 4, 32, >=N]")
+    n = vt.shape[0]
+    ld = (n + 15) // 16 * 16
+    full = torch.zeros((n, 4, 32, ld), dtype=torch.bfloat16, device=vt.device)
+    full[..., :n] = vt[..., :n].to(torch.bfloat16)
+    # swapping the two middle quads of every group of 16 is its own inverse
+    return full.view(n, 4, 32, ld // 16, 4, 4)[..., [0, 2, 1, 3], :].reshape(n, 4, 32, ld).contiguous()
 
 
 def grid_attention_core(q, k, vt, g, pair_bias, mask, out=None):
     """The flash-attention stage of the triangle attention on projected, head-major
-    bf16 operands in base-2 form: q, k, g [N, 4, N, 32] (q and the bias
-    pre-multiplied by log2(e); g = sigmoid gate), vt [N, 4, 32, ld] with ld = N
-    rounded up to 8 and zero padding, pair_bias from pack_pair_bias() or None.
-    Returns the gated output [N*N, 128] bf16."""
+    operands in base-2 form: q, k, g bf16 [N, 4, N, 32] (q and the bias
+    pre-multiplied by log2(e); g = sigmoid gate), vt from pack_vt(), pair_bias
+    from pack_pair_bias() or None.  Returns the gated output [N*N, 128] bf16."""
     lib = _L.load()
     _gpu(q, "q", torch.bfloat16)
     if q.dim() != 4 or q.shape[1] != 4 or q.shape[3] != 32 or q.shape[0] != q.shape[2]:
         raise ValueError("q: expected [N, 4, N, 32]")
     n = q.shape[0]
-    ld = (n + 7) // 8 * 8
+    ld = (n + 15) // 16 * 16
     _gpu(k, "k", torch.bfloat16, q.shape)
     _gpu(g, "g", torch.bfloat16, q.shape)
     _gpu(vt, "vt", torch.bfloat16, (n, 4, 32, ld))
     if pair_bias is not None:
-        _gpu(pair_bias, "pair_bias", torch.bfloat16, (4, (n + 31) // 32, (n + 63) // 64, 4, 32, 16))
+        _gpu(pair_bias, "pair_bias", torch.float32, (4, (n + 31) // 32, (n + 63) // 64, 8, 2, 32, 4))
     maskf = _mask_f32(mask, (n, n), "mask")
     if out is None:
         out = torch.empty((n * n, 128), dtype=torch.bfloat16, device=q.device)

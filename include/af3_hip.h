@@ -372,15 +372,18 @@ int af3_linear_forward(
  *   n_token..ld-1 of a and b must be zero.
  * af3_grid_attention_core_forward: the flash attention stage of the triangle
  *   attention (csrc/grid_self_attention_bf16.h:226-481) on already projected
- *   operands, bf16, head-major, in base-2 form (4 heads of 32, ld = n_token
- *   rounded up to 8):
- *     q  [b][h][s][32] = query * log2(e)/sqrt(32);  k, g [b][h][s][32] (g = sigmoid gate);
- *     vt [b][h][32][ld] = value transposed, columns n_token..ld-1 zero;
- *     pair_bias = bias * log2(e) in MFMA-fragment order, or NULL: element (h, q, k) at
- *       ((((h*QB + q/32)*KT + k/64)*4 + (k%64)/16)*32 + q%32)*16 + k%16,
+ *   operands, head-major, in base-2 form (4 heads of 32, ld = n_token rounded
+ *   up to 16):
+ *     q  bf16 [b][h][s][32] = query * log2(e)/sqrt(32);  k, g bf16 [b][h][s][32] (g = sigmoid gate);
+ *     vt bf16 [b][h][32][ld] = value transposed, key k of a row stored at column
+ *       (k & ~12) | ((k & 8) >> 1) | ((k & 4) << 1) (inside every aligned group of 16 keys
+ *       the two middle quads are swapped), columns of keys >= n_token zero;
+ *     pair_bias fp32 = bias * log2(e) in the order of the kernel's score accumulator, or
+ *       NULL: element (h, q, k) at
+ *       ((((h*QB + q/32)*KT + k/64)*8 + (k%64)/8)*64 + ((k%8)/4)*32 + q%32)*4 + k%4,
  *       QB = ceil(N/32), KT = ceil(N/64), 4*QB*KT*2048 elements, keys >= N zero
- *       (per head, 32-query block and 64-key tile: four contiguous 1 KB runs, each
- *       the B operand of one identity-matrix MFMA that adds the bias to the logits);
+ *       (per head, 32-query block and 64-key tile: eight contiguous 1 KB runs, each
+ *       filling four accumulator registers of every lane with one 16-byte load);
  *   key mask [N][N] fp32 0/1 or NULL;
  *   og [(b*N + s)][128] = gate * softmax(q k^T + bias) v.
  */
@@ -388,7 +391,7 @@ int af3_triangle_contraction_forward(
     const uint16_t* a, const uint16_t* b, uint16_t* t, int64_t n_token, af3_stream_t stream);
 int af3_grid_attention_core_forward(
     const uint16_t* q, const uint16_t* k, const uint16_t* vt, const uint16_t* g,
-    const uint16_t* pair_bias, const float* mask, uint16_t* og, int64_t n_token, af3_stream_t stream);
+    const float* pair_bias, const float* mask, uint16_t* og, int64_t n_token, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
  * fp32 check mode.  Plain fp32 kernels (fp32 storage, fp32 FMA arithmetic, no

@@ -163,7 +163,7 @@ def test_attention_core_more_than_64_key_tiles(gpu_pkg):
     mask[:, 0] = 1
     mask[11, :] = 0                                   # a fully masked row
     mask[:, n - 100:] = 0                             # trailing padding: the last key tile is masked as a whole
-    og = gpu_pkg.ops.grid_attention_core(q, k, vt, gt, gpu_pkg.ops.pack_pair_bias(bias), mask)
+    og = gpu_pkg.ops.grid_attention_core(q, k, gpu_pkg.ops.pack_vt(vt), gt, gpu_pkg.ops.pack_pair_bias(bias), mask)
     og = og.view(n, n, 4, 32)
     log2e = 1.4426950408889634
     for b in (0, 11, 2077, n - 1):

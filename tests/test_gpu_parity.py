@@ -411,19 +411,14 @@ def test_kernel_level_contraction(gpu_pkg, n):
     assert_within_bf16_ulp("contraction", t[:, :, :n], want, ulps=1.01, atol=1e-3)
 
 
-@pytest.mark.parametrize("n,tiles", [(40, False), (200, False), (200, True), (330, True)])
-def test_kernel_level_attention_core(gpu_pkg, n, tiles):
-    """Base-2 operands in, gate * softmax(q k^T + bias, masked) v out.  `tiles`:
-    whole 64-key tiles masked (the kernel leaves such tiles out for rows that
-    have an unmasked key elsewhere, which must not change a bit of the result)."""
-    note(f"test_kernel_level_attention_core n={n} tiles={tiles}")
-    g = gen(n + tiles)
+def _attention_core_case(gpu_pkg, n, tiles, scale=0.7, bias_shift=0.0, seed=None):
+    g = gen(n + tiles if seed is None else seed)
     log2e = 1.4426950408889634
-    npad = (n + 7) // 8 * 8
-    qkvg = rb(torch.randn(n, n, 4, 4, 32, generator=g) * 0.7)       # [b, s, (q k v g), h, d]
-    qkvg[:, :, 3] = torch.sigmoid(qkvg[:, :, 3]).bfloat16().float()
-    bias = torch.zeros(4, n, npad)
-    bias[:, :, :n] = rb(torch.randn(4, n, n, generator=g))
+    d = dev()
+    qkvg = rb(torch.randn(n, n, 4, 4, 32, generator=g) * scale)     # [b, s, (q k v g), h, d]
+    qkvg[:, :, 2] = rb(qkvg[:, :, 2] * (0.7 / scale))
+    qkvg[:, :, 3] = torch.sigmoid(qkvg[:, :, 3] * (0.7 / scale)).bfloat16().float()
+    bias = rb(torch.randn(4, n, n, generator=g)) + bias_shift
     mask = (torch.rand(n, n, generator=g) > 0.2).float()
     mask[:, 0] = 1
     if tiles:
@@ -433,18 +428,53 @@ def test_kernel_level_attention_core(gpu_pkg, n, tiles):
         mask[:, n - 70:] = 0                                        # trailing padding, more than a tile
         mask[7, :] = 0
         mask[7, n - 3] = 1                                          # row 7 lives in the last, partial tile only
+        mask[8, :] = 0
+        mask[8, 70] = 1                                             # rows 8 and 9 share a wave when it takes two
+        mask[9, :] = 0
+        mask[9, 10] = 1
     mask[3, :] = 0                                                  # one fully masked row
     hm = lambda i: qkvg[:, :, i].permute(0, 2, 1, 3).contiguous()       # [b, h, s, d]
-    vt = torch.zeros(n, 4, 32, npad)
-    vt[..., :n] = hm(2).transpose(-1, -2)
-    t = lambda x: x.to(dev()).bfloat16()
-    og = gpu_pkg.ops.grid_attention_core(t(hm(0)), t(hm(1)), t(vt), t(hm(3)),
-                                         gpu_pkg.ops.pack_pair_bias(t(bias)), mask.to(dev()))
-    q, k, v, gt = (qkvg[:, :, i].permute(0, 2, 1, 3).double() for i in range(4))   # [b, h, s, d]
-    logits = (q @ k.transpose(-1, -2) + bias[None, :, :, :n].double()) / log2e
-    logits = logits.masked_fill(mask[:, None, None, :] == 0, -1e9)
-    want = (torch.softmax(logits, -1) @ v) * gt
-    want = want.permute(0, 2, 1, 3).reshape(n * n, 128)
-    e_max, e_rms = _errs(og.float().cpu(), want)
+    t = lambda x: x.to(d).bfloat16()
+    og = gpu_pkg.ops.grid_attention_core(t(hm(0)), t(hm(1)), gpu_pkg.ops.pack_vt(t(hm(2).transpose(-1, -2))),
+                                         t(hm(3)), gpu_pkg.ops.pack_pair_bias(bias.to(d)), mask.to(d))
+    og = og.view(n, n, 4, 32).float()
+    # the reference on the GPU in float64, a block of rows at a time
+    q, k, v, gt = (qkvg[:, :, i].permute(0, 2, 1, 3).to(d).double() for i in range(4))   # [b, h, s, d]
+    bd, md = bias.to(d).double(), mask.to(d)
+    want = torch.empty(n, n, 4, 32, dtype=torch.float64, device=d)
+    for b0 in range(0, n, 32):
+        sl = slice(b0, min(n, b0 + 32))
+        logits = (q[sl] @ k[sl].transpose(-1, -2) + bd[None]) / log2e
+        logits = logits.masked_fill(md[sl][:, None, None, :] == 0, -1e9)
+        want[sl] = ((torch.softmax(logits, -1) @ v[sl]) * gt[sl]).permute(0, 2, 1, 3)
+    return og, want
+
+
+@pytest.mark.parametrize("n,tiles", [(40, False), (200, False), (200, True), (330, True), (515, True), (576, False)])
+def test_kernel_level_attention_core(gpu_pkg, n, tiles):
+    """Base-2 operands in, gate * softmax(q k^T + bias, masked) v out.  `tiles`:
+    whole 64-key tiles masked (the kernel leaves such tiles out for rows that
+    have an unmasked key elsewhere, which must not change a bit of the result).
+    From 512 tokens on a wave takes two rows at a time (515: the last row has no partner)."""
+    note(f"test_kernel_level_attention_core n={n} tiles={tiles}")
+    og, want = _attention_core_case(gpu_pkg, n, tiles)
+    e_max, e_rms = _errs(og.cpu(), want.cpu())
     note(f"attention core n={n}: max {e_max:.3e} rms {e_rms:.3e}")
-    assert e_rms < 5e-3 and e_max < 4e-2                            # bf16 probabilities and output
+    # bf16 un-normalised probabilities (every one of them rounded, the largest of a row included,
+    # since the kernel does not subtract the row maximum) and a bf16 output; the maximum is taken
+    # over n * n * 128 outputs (1.3e8 at n = 576), so its bound grows slowly with n
+    assert e_rms < 5e-3 and e_max < (5e-2 if n <= 400 else 7e-2)
+
+
+@pytest.mark.parametrize("n,scale,shift", [(200, 2.5, 0.0), (200, 0.7, -300.0), (200, 0.7, 500.0), (520, 2.5, -100.0)])
+def test_kernel_level_attention_core_large_logits(gpu_pkg, n, scale, shift):
+    """Logits far from zero (|q.k| up to ~150 in base 2, biases of -300 / +500): the kernel's
+    softmax base, which it only moves when a tile's scores leave a window around it, has to
+    follow; the result must be the same softmax, which is shift-invariant."""
+    note(f"test_kernel_level_attention_core_large_logits n={n} scale={scale} shift={shift}")
+    og, want = _attention_core_case(gpu_pkg, n, True, scale=scale, bias_shift=shift, seed=7 * n + int(shift))
+    assert torch.isfinite(og).all()
+    e_max, e_rms = _errs(og.cpu(), want.cpu())
+    note(f"attention core n={n} scale={scale} shift={shift}: max {e_max:.3e} rms {e_rms:.3e}")
+    # sharp softmaxes put single bf16-rounded probabilities on single values: a looser maximum
+    assert e_rms < 8e-3 and e_max < 8e-2
