@@ -141,10 +141,10 @@ int af3_triangle_multiplication_forward(
 size_t af3_grid_self_attn_workspace_bytes(int64_t n, int num_head) {
   if (n <= 0 || num_head <= 0) return 0;
   const size_t e = sizeof(bf16_t), ldn = (size_t)tri_ldn(n);
-  // fast path: q, k, g planes, vt, og, fp32 bias
+  // fast path: q, k, g planes, vt, og, fp16 bias
   const size_t fast = 3 * align_up((size_t)n * n * C_PAIR * e, 256) + align_up((size_t)n * C_PAIR * ldn * e, 256) +
                       align_up((size_t)n * n * C_PAIR * e, 256) +
-                      align_up((size_t)tri_bias_elems(n, num_head) * sizeof(float), 256);
+                      align_up((size_t)tri_bias_elems(n, num_head) * sizeof(uint16_t), 256);
   // general path (external fp32 bias): qkvg + og
   const size_t general = align_up((size_t)n * n * 4 * C_PAIR * e, 256) + align_up((size_t)n * n * C_PAIR * e, 256);
   return fast > general ? fast : general;
@@ -169,7 +169,7 @@ int af3_grid_self_attn_forward(
   if (nonbatched_bias == nullptr) {
     // Fast path: the pair bias (if any) is projected here, so everything the
     // attention core needs is produced in its preferred form: base-2 logits,
-    // fp32 bias in accumulator order, head-major planes, V transposed.
+    // fp16 bias in fragment order, head-major planes, V transposed.
     const float LOG2E = 1.4426950408889634f;
     const int64_t ldn = tri_ldn(n);
     bf16_t* q = ws.take<bf16_t>((size_t)n * n * C_PAIR);
@@ -177,7 +177,7 @@ int af3_grid_self_attn_forward(
     bf16_t* g = ws.take<bf16_t>((size_t)n * n * C_PAIR);
     bf16_t* vt = ws.take<bf16_t>((size_t)n * C_PAIR * ldn);
     og = ws.take<bf16_t>((size_t)n * n * C_PAIR);
-    float* bias = ws.take<float>((size_t)tri_bias_elems(n, num_head));
+    uint16_t* bias = ws.take<uint16_t>((size_t)tri_bias_elems(n, num_head));
     if (!ws.ok) return AF3_ERR_WORKSPACE;
     TriAttnProjArgs p;
     p.pair = pair; p.io_f32 = io_dtype == AF3_F32; p.N = (int)n; p.transpose = transpose != 0;
@@ -564,7 +564,7 @@ int af3_triangle_contraction_forward(
 
 int af3_grid_attention_core_forward(
     const uint16_t* q, const uint16_t* k, const uint16_t* vt, const uint16_t* g,
-    const float* pair_bias, const float* mask, uint16_t* og, int64_t n, af3_stream_t stream) {
+    const uint16_t* pair_bias, const float* mask, uint16_t* og, int64_t n, af3_stream_t stream) {
   if (n <= 0 || n > 8192) return AF3_ERR_BAD_ARG;
   TriAttnArgs t;
   t.q = q; t.k = k; t.vt = vt; t.g = g; t.bias = pair_bias; t.mask = mask; t.og = og;

@@ -41,6 +41,12 @@ __device__ __forceinline__ uint32_t pack2bf(float lo, float hi) {
 __device__ __forceinline__ float bflo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bfhi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 
+// fp32 -> fp16 bits, round to nearest even, saturating at the largest finite fp16
+__device__ __forceinline__ uint16_t f2h_sat(float f) {
+  f = fminf(fmaxf(f, -65504.f), 65504.f);
+  return __builtin_bit_cast(uint16_t, (_Float16)f);
+}
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 // 8 consecutive bf16 (16 bytes) <-> 8 floats
 __device__ __forceinline__ void unpack8(const u32x4 v, float* f) {
   f[0] = bflo(v.x); f[1] = bfhi(v.x); f[2] = bflo(v.y); f[3] = bfhi(v.y);
@@ -115,6 +121,10 @@ __device__ __forceinline__ float sigmoidf_(float x) {
 __device__ __forceinline__ f32x16 mfma32(const bf16x8 a, const bf16x8 b, const f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
+__device__ __forceinline__ f32x16 mfma32_f16(const f16x8 a, const f16x8 b, const f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f16x8 as_frag_f16(const u32x4 v) { return __builtin_bit_cast(f16x8, v); }
 __device__ __forceinline__ bf16x8 as_frag(const u32x4 v) {
   return __builtin_bit_cast(bf16x8, v);
 }

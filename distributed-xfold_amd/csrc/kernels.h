@@ -167,10 +167,13 @@ int launch_flash_attention(const FlashArgs& a, hipStream_t stream);
 //            key k of a row stored at column tri_vt_pos(k): inside every aligned group of 16
 //            keys the two middle quads are swapped, which makes the 8 keys one lane feeds to
 //            a P.V MFMA (k, k+1, k+2, k+3, k+8, ..., k+11 with k % 8 == 0 or 4) 16 contiguous bytes
-//   bias     fp32, pair bias times log2(e), in the order of the attention core's score
-//            accumulator: per (head, 32-query block, 64-key tile) eight contiguous 1 KB runs,
-//            run (k % 64) / 8, lane ((k % 8) / 4) * 32 + q % 32, element k % 4, so that one
-//            16-byte load per lane fills four accumulator registers of the S^T tile.
+//   bias     fp16, pair bias times log2(e) (clamped to the fp16 range), in MFMA-fragment order:
+//            the attention core adds it to the scores on the matrix unit, S^T += I * bias^T with an
+//            fp16 identity, and wants per (head, 32-query block, 64-key tile) the four B fragments
+//            of that product as four contiguous 1 KB runs: run (k % 64) / 16, then [q % 32][k % 16].
+//            fp16 rather than fp32: at 8 MFMAs per key tile the kernel is paced by the bytes the
+//            CU's vector memory path can take, and the bias is most of them; fp16's 11 significant
+//            bits put its rounding (2^-12 of a logit) below that of the bf16 probabilities (2^-9).
 //            Entries whose key is >= N are zero; query rows >= N of the last block are unused.
 __host__ __device__ inline int64_t tri_ldn(int64_t n) { return (n + 15) / 16 * 16; }
 __host__ __device__ inline int tri_vt_pos(int k) { return (k & ~12) | ((k & 8) >> 1) | ((k & 4) << 1); }
@@ -180,8 +183,8 @@ __host__ __device__ inline int64_t tri_bias_elems(int64_t n, int64_t heads) {
   return heads * tri_bias_qblocks(n) * tri_bias_ktiles(n) * 2048;
 }
 __host__ __device__ inline int64_t tri_bias_offset(int64_t n, int h, int q, int k) {
-  return ((((int64_t)h * tri_bias_qblocks(n) + (q >> 5)) * tri_bias_ktiles(n) + (k >> 6)) * 8 + ((k & 63) >> 3)) * 256 +
-         (((k & 7) >> 2) * 32 + (q & 31)) * 4 + (k & 3);
+  return ((((int64_t)h * tri_bias_qblocks(n) + (q >> 5)) * tri_bias_ktiles(n) + (k >> 6)) * 4 + ((k & 63) >> 4)) * 512 +
+         (q & 31) * 16 + (k & 15);
 }
 
 struct TriAttnProjArgs {
@@ -193,14 +196,14 @@ struct TriAttnProjArgs {
   int n_bias = 0;                  // 0 or 4
   float q_scale = 1.f, bias_scale = 1.f;
   bf16_t *q = nullptr, *k = nullptr, *vt = nullptr, *g = nullptr;
-  float* bias = nullptr;  // accumulator order, tri_bias_elems(N, 4) elements
+  uint16_t* bias = nullptr;  // fp16 bits, fragment order, tri_bias_elems(N, 4) elements
   int64_t ldn = 0;        // tri_ldn(N)
 };
 int launch_triattn_proj(const TriAttnProjArgs& a, hipStream_t stream);
 
 struct TriAttnArgs {
   const bf16_t *q = nullptr, *k = nullptr, *vt = nullptr, *g = nullptr;
-  const float* bias = nullptr;   // accumulator order (tri_bias_offset), or null
+  const uint16_t* bias = nullptr;  // fp16 bits, fragment order (tri_bias_offset), or null
   const float* mask = nullptr;   // [N][N] 0/1 or null
   bf16_t* og = nullptr;          // [(b*N + s)][128]
   int N = 0;

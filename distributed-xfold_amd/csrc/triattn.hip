@@ -2,7 +2,7 @@
 // pass over the pair tensor, everything the attention core (triattn_core.hip)
 // reads, in the layouts it wants (described in kernels.h): head-major q (scaled),
 // k and sigmoid gate, V transposed with the key order the core's MFMA fragments
-// use, and the fp32 pair bias in the order of the core's score accumulator.
+// use, and the fp16 pair bias in the order of the core's MFMA fragments.
 #include "common.h"
 #include "kernels.h"
 #include <type_traits>
@@ -165,15 +165,15 @@ __global__ __launch_bounds__(256, 3) void triattn_proj_kernel(TriAttnProjArgs a)
         if (r < kpad) {
 #pragma unroll
           for (int h = 0; h < H; ++h)
-            a.bias[tri_bias_offset(a.N, h, t.o, r)] = t.valid(p) ? acc[0][h] * a.bias_scale : 0.f;
+            a.bias[tri_bias_offset(a.N, h, t.o, r)] = f2h_sat(t.valid(p) ? acc[0][h] * a.bias_scale : 0.f);
         }
       } else if (t.valid(p)) {
         // q = r, k = o
 #pragma unroll
         for (int h = 0; h < H; ++h) {
-          a.bias[tri_bias_offset(a.N, h, r, t.o)] = acc[0][h] * a.bias_scale;
+          a.bias[tri_bias_offset(a.N, h, r, t.o)] = f2h_sat(acc[0][h] * a.bias_scale);
           if (t.o == a.N - 1)
-            for (int k = a.N; k < kpad; ++k) a.bias[tri_bias_offset(a.N, h, r, k)] = 0.f;
+            for (int k = a.N; k < kpad; ++k) a.bias[tri_bias_offset(a.N, h, r, k)] = 0;
         }
       }
     }

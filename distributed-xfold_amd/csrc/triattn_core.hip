@@ -5,7 +5,7 @@
 //   Vt      : bf16 [b][h][32][ldn], V transposed, ldn = N rounded up to 16, columns
 //             permuted inside every aligned group of 16 (tri_vt_pos) so that the 8 keys one
 //             lane feeds to a P.V MFMA are 16 contiguous bytes
-//   bias    : fp32, pair bias * log2(e) in the order of the score accumulator (tri_bias_offset)
+//   bias    : fp16, pair bias * log2(e) in MFMA-fragment order (tri_bias_offset)
 //   mask    : fp32 [N][N] 0/1 or null
 //
 // What sets the pace on this machine (measured): a wave64 exp2 occupies the SIMD's issue port
@@ -14,9 +14,11 @@
 // wave has an MFMA waiting for the unit.  So vector and matrix work overlap only inside one
 // wave's own instruction stream, and the kernel is built around that:
 //   * one wave = 32 queries of R rows b; lane = one query; S^T = K Q^T so that the softmax
-//     reductions are per lane.  The fp32 pair bias tile is the INITIAL VALUE of the score
-//     accumulator; it does not depend on the row, so the rows of a wave share one load of it
-//     (with R = 2 the bias costs the CU's vector memory path as much as a bf16 bias would).
+//     reductions are per lane.  The pair bias enters on the matrix unit as well, S^T += I *
+//     bias^T with an fp16 identity; its fragments do not depend on the row, so the R rows of a
+//     wave share one load of them.  (With the fp32 bias as the accumulators' initial value the
+//     kernel ran 35 % slower than without any bias: at this rate the bytes the bias brings
+//     through the CU's vector memory path are what paces it; hence fp16 and two rows per wave.)
 //   * the key mask rides in the product as a third k-step (K side 0 / -1e9 / -inf, Q side 1.0),
 //     and so does the softmax's running base: the Q side of the next slot holds -base, so the
 //     accumulator comes out as s - base and exp2 takes it as it is.  `base` only moves when a
@@ -24,7 +26,8 @@
 //     O and l by an exact-in-fp32 factor and repeats the tile's score product); for ordinary
 //     logits it never moves and the softmax is computed without a single subtraction.
 //     The third k-step is left out (wave-uniformly) for a tile of 64 unmasked keys while no
-//     lane of the row has moved its base: eight MFMAs per key tile, the algorithm's own count.
+//     lane of the row has moved its base: eight MFMAs per key tile and row (the algorithm's
+//     own count) plus the four of the bias.
 //   * the probabilities of tile v go into O while the exponentials of tile v+1 are computed:
 //     each of those four MFMAs is issued in front of eight exponentials of the same wave, its
 //     V^T fragment read from LDS one group ahead.  Row sums are taken from the bf16
@@ -130,7 +133,8 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
   __shared__ __attribute__((aligned(1024))) char sV01[R > 1 ? TILE_BYTES : 16];
   __shared__ __attribute__((aligned(1024))) char sV10[TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) char sV11[R > 1 ? TILE_BYTES : 16];
-  __shared__ __attribute__((aligned(1024))) char sBias[HAS_BIAS ? 4 * 8192 : 16];  // one bias tile per wave
+  __shared__ __attribute__((aligned(1024))) char sBias0[HAS_BIAS ? 4 * 4096 : 16];  // a bias tile per wave, by key tile parity
+  __shared__ __attribute__((aligned(1024))) char sBias1[HAS_BIAS ? 4 * 4096 : 16];
   __shared__ uint32_t sLive[R * 5];  // per row: live tiles (2 words), any live key, wholly unmasked tiles (2 words)
   __shared__ float sMean[D];
   extern __shared__ __attribute__((aligned(16))) uint16_t sCode[];  // [R][nkt * 64] mask code per key
@@ -267,48 +271,48 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
     const int wave_blk = q0 + wave * 32 < N ? (q0 >> 5) + wave : 0;
     const char* bbase =
         HAS_BIAS ? reinterpret_cast<const char*>(a.bias + tri_bias_offset(N, h, wave_blk * 32, 0)) : nullptr;
-    // The bias tile of key tile t + 2 is fetched into the wave's own 8 KB of LDS at the end of
-    // tile t (a whole key tile of time for the load to land, behind a barrier), and tile t + 1's
-    // moves from there into the registers that seed the score accumulators as soon as the last
-    // row has used tile t's.
-    char* bstage = sBias + wave * 8192;
+    // The bias tile (four 1 KB fp16 fragments) of key tile t + 2 is fetched into the wave's own
+    // 4 KB of LDS (one of two buffers, by key tile parity) right after tile t's barrier, with the
+    // K / V^T tiles: two rows' worth of time for the load to land.  While the last row of tile
+    // t computes its exponentials, tile t + 1's fragments are read from LDS and turned into fp32
+    // on the matrix unit, bt = I * bias^T with an fp16 identity: the initial value of the score
+    // accumulators of every row of tile t + 1 (four MFMAs per key tile, each issued between two
+    // groups of exponentials).
     f32x16 bt[2];
-    auto dma_bias = [&](int tile) {
+    auto dma_bias = [&](int tile, char* buf) {
       if (!HAS_BIAS) return;
-      const char* p = bbase + (size_t)min(tile, nkt - 1) * 8192u;
-      dma16<0>(p, lane * 16u, bstage);
-      dma16<1024>(p, lane * 16u, bstage);
-      dma16<2048>(p, lane * 16u, bstage);
-      dma16<3072>(p, lane * 16u, bstage);
-      dma16<0>(p, lane * 16u + 4096u, bstage + 4096);
-      dma16<1024>(p, lane * 16u + 4096u, bstage + 4096);
-      dma16<2048>(p, lane * 16u + 4096u, bstage + 4096);
-      dma16<3072>(p, lane * 16u + 4096u, bstage + 4096);
+      const char* p = bbase + (size_t)min(tile, nkt - 1) * 4096u;
+      char* dst = buf + wave * 4096;
+      dma16<0>(p, lane * 16u, dst);
+      dma16<1024>(p, lane * 16u, dst);
+      dma16<2048>(p, lane * 16u, dst);
+      dma16<3072>(p, lane * 16u, dst);
     };
-    auto bias_from_lds = [&]() {
-      if (!HAS_BIAS) return;
+    // fragment i = 2 u + st: keys 32 u + 16 st + 8 hh .. + 8 of this lane's query, bytes (32 j + 16 hh) of run i
+    const int boff = wave * 4096 + j * 32 + hh * 16;
+    // Identity fragments (fp16): A-fragment of k-step st: lane (row i = j, half hh) holds
+    // I[i][16 st + 8 hh + e], e = 0..7: a single 1.0 where 16 st + 8 hh + e == i.
+    f16x8 idf[2];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const f32x4 v = *reinterpret_cast<const f32x4*>(bstage + 1024 * i + lane * 16);
-        bt[i >> 2][4 * (i & 3)] = v.x; bt[i >> 2][4 * (i & 3) + 1] = v.y;
-        bt[i >> 2][4 * (i & 3) + 2] = v.z; bt[i >> 2][4 * (i & 3) + 3] = v.w;
-      }
-    };
-    auto load_bias = [&](int tile) {  // straight from global memory (the first tile)
-      if (!HAS_BIAS) return;
-      const char* p = bbase + (size_t)min(tile, nkt - 1) * 8192u + lane * 16;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const f32x4 v = *reinterpret_cast<const f32x4*>(p + 1024 * i);
-        bt[i >> 2][4 * (i & 3)] = v.x; bt[i >> 2][4 * (i & 3) + 1] = v.y;
-        bt[i >> 2][4 * (i & 3) + 2] = v.z; bt[i >> 2][4 * (i & 3) + 3] = v.w;
-      }
-    };
-    if (!HAS_BIAS) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) bt[0][e] = bt[1][e] = 0.f;
+    for (int st = 0; st < 2; ++st) {
+      const int e1 = j - 16 * st - 8 * hh;
+      uint32_t w[4] = {0u, 0u, 0u, 0u};
+      if (e1 >= 0 && e1 < 8) w[e1 >> 1] = (e1 & 1) ? (0x3C00u << 16) : 0x3C00u;
+      idf[st] = as_frag_f16(u32x4{w[0], w[1], w[2], w[3]});
     }
-
+    f32x16 zero16;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) zero16[e] = 0.f;
+    // scores of one row's virtual tile: the two halves of the head dimension on top of the bias
+    auto scores = [&](const bf16x8& k00, const bf16x8& k01, const bf16x8& k10, const bf16x8& k11, const bf16x8* q,
+                      f32x16& s0, f32x16& s1) {
+      s0 = mfma32(k00, q[0], bt[0]);
+      s1 = mfma32(k10, q[0], bt[1]);
+      s0 = mfma32(k01, q[1], s0);
+      s1 = mfma32(k11, q[1], s1);
+    };
+#pragma unroll
+    for (int e = 0; e < 16; ++e) bt[0][e] = bt[1][e] = 0.f;
     bool based[R];  // some lane of the wave has moved this row's base off zero
 #pragma unroll
     for (int r = 0; r < R; ++r) based[r] = false;
@@ -325,7 +329,7 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
 
     // One virtual tile = (key tile, row RR): scores, softmax, and meanwhile the previous
     // virtual tile's probabilities go into its row sums and its O.
-    auto iter = [&](auto PHc, auto RRc, int tile, int tile_after_next) {
+    auto iter = [&](auto PHc, auto RRc, int tile) {
       constexpr int PH = decltype(PHc)::value, RR = decltype(RRc)::value;
       constexpr int PR = (RR + R - 1) % R, VPH = RR == 0 ? PH ^ 1 : PH;
       const char* kb = KBUF(PH, RR);
@@ -342,10 +346,7 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       bf16x8 af0, af1;
       f32x16 s0, s1;
       STAMP(4);
-      s0 = mfma32(k00, qf[RR][0], bt[0]);
-      s1 = mfma32(k10, qf[RR][0], bt[1]);
-      s0 = mfma32(k01, qf[RR][1], s0);
-      s1 = mfma32(k11, qf[RR][1], s1);
+      scores(k00, k01, k10, k11, qf[RR], s0, s1);
       if (step3) {
         const uint16_t* mc = sCode + RR * nk64 + tile * KT;
         const uint32_t c0 = mc[j], c1 = mc[32 + j];
@@ -388,27 +389,25 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
         } else {
           scale_in_place(o[RR], alpha);
         }
-        s0 = mfma32(k00, qf[RR][0], bt[0]);
-        s1 = mfma32(k10, qf[RR][0], bt[1]);
-        s0 = mfma32(k01, qf[RR][1], s0);
-        s1 = mfma32(k11, qf[RR][1], s1);
+        scores(k00, k01, k10, k11, qf[RR], s0, s1);
         s0 = mfma32(af0, as_frag(qm[RR]), s0);
         s1 = mfma32(af1, as_frag(qm[RR]), s1);
       } else {
         mrel[RR] = mnew;
       }
-      // the last row to use this key tile's bias takes the next tile's from LDS into the same
-      // registers (it landed before the last barrier)
-      if (RR == R - 1) bias_from_lds();
       STAMP(2);
-
       // From here to the end: one basic block in a fixed order.  Each of the four P.V MFMAs of the
       // previous virtual tile is issued in front of eight exponentials of this one (the matrix
       // unit works while the wave goes on issuing vector instructions; another wave's would not
       // get in), with its V^T fragment read from LDS one group ahead.
       bf16x8 vf = lds16(vb + va[0]);
+      u32x4 bfr[4];  // the next key tile's bias fragments (the last row of this one fetches them)
+      if (HAS_BIAS && RR == R - 1) {
+        const char* bsrc = (PH == 0 ? sBias1 : sBias0) + boff;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bfr[i] = *reinterpret_cast<const u32x4*>(bsrc + 1024 * i);
+      }
       __builtin_amdgcn_sched_barrier(0);
-      u32x4 pc[4];
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const bf16x8 vcur = vf;
@@ -419,21 +418,22 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
         o[PR] = mfma32(vcur, as_frag(pp[s]), o[PR]);
         float p8[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) p8[e] = __builtin_amdgcn_exp2f(s < 2 ? s0[8 * (s & 1) + e] : s1[8 * (s & 1) + e]);
-        pc[s] = pack8(p8);
-        lrun[RR] = dot2_ones(pc[s].w, dot2_ones(pc[s].z, dot2_ones(pc[s].y, dot2_ones(pc[s].x, lrun[RR]))));
+        for (int e = 0; e < 4; ++e) p8[e] = __builtin_amdgcn_exp2f(s < 2 ? s0[8 * (s & 1) + e] : s1[8 * (s & 1) + e]);
+        if (HAS_BIAS && RR == R - 1) {
+          // fragments 2 u + st: bt[u] = I(st = 0) * f(2 u) + I(st = 1) * f(2 u + 1); group s does (u, st) = (s / 2, s % 2)
+          asm volatile("" : "+v"(p8[0]), "+v"(p8[1]), "+v"(p8[2]), "+v"(p8[3]));
+          bt[s >> 1] = mfma32_f16(idf[s & 1], as_frag_f16(bfr[s]), (s & 1) ? bt[s >> 1] : zero16);
+        }
+#pragma unroll
+        for (int e = 4; e < 8; ++e) p8[e] = __builtin_amdgcn_exp2f(s < 2 ? s0[8 * (s & 1) + e] : s1[8 * (s & 1) + e]);
+        // this tile's probabilities take the place of the previous tile's, whose last reader (the
+        // MFMA above) has been issued
+        pp[s] = pack8(p8);
         // pins the exponentials to this group (without it they sink to where their values are used,
         // the next iteration's MFMAs)
-        asm volatile("" : "+v"(pc[s].x), "+v"(pc[s].y), "+v"(pc[s].z), "+v"(pc[s].w));
+        asm volatile("" : "+v"(pp[s].x), "+v"(pp[s].y), "+v"(pp[s].z), "+v"(pp[s].w));
+        lrun[RR] = dot2_ones(pp[s].w, dot2_ones(pp[s].z, dot2_ones(pp[s].y, dot2_ones(pp[s].x, lrun[RR]))));
         __builtin_amdgcn_sched_barrier(0);
-      }
-#pragma unroll
-      for (int s = 0; s < 4; ++s) pp[s] = pc[s];
-      if (RR == R - 1) {
-        // the staged tile is in registers by now (its reads were issued before the exponentials):
-        // the tile after it may overwrite it
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        dma_bias(tile_after_next);
       }
       STAMP(3);
     };
@@ -448,8 +448,15 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
     int t_cur = pop(), t_n1 = pop(), t_n2 = pop();
     // the buffer the first virtual tile reads its "previous" V^T from must hold finite data
     *reinterpret_cast<u32x4*>(VBUF(1, R - 1) + tid * 16) = u32x4{0u, 0u, 0u, 0u};
-    load_bias(t_cur);
-    dma_bias(t_n1);
+    if (HAS_BIAS) {
+      const char* p = bbase + (size_t)t_cur * 4096u + (j * 32 + hh * 16);
+      u32x4 f[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) f[i] = *reinterpret_cast<const u32x4*>(p + 1024 * i);
+      bt[0] = mfma32_f16(idf[1], as_frag_f16(f[1]), mfma32_f16(idf[0], as_frag_f16(f[0]), zero16));
+      bt[1] = mfma32_f16(idf[1], as_frag_f16(f[3]), mfma32_f16(idf[0], as_frag_f16(f[2]), zero16));
+    }
+    dma_bias(t_n1, sBias1);
     dma_k(t_cur, 0, KBUF(0, 0));
     if (R == 2) {
       dma_k(t_cur, 1, KBUF(0, 1));
@@ -470,22 +477,24 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       constexpr int PH = decltype(PHc)::value;
       using P0 = std::integral_constant<int, PH>;
       if (R == 2) {
-        iter(P0{}, std::integral_constant<int, 0>{}, t_cur, t_n2);
+        iter(P0{}, std::integral_constant<int, 0>{}, t_cur);
         STAMP(0);
         dma_barrier();
         STAMP(1);
+        dma_bias(t_n2, PH == 0 ? sBias0 : sBias1);
         dma_k(t_n1, 1, KBUF(PH ^ 1, 1));
         dma_k(t_n2, 0, KBUF(PH, 0));
         dma_v(t_n1, 0, VBUF(PH ^ 1, 0));
         dma_v(t_n1, 1, VBUF(PH ^ 1, 1));
-        iter(P0{}, std::integral_constant<int, R - 1>{}, t_cur, t_n2);
+        iter(P0{}, std::integral_constant<int, R - 1>{}, t_cur);
       } else {
         STAMP(0);
         dma_barrier();
         STAMP(1);
+        dma_bias(t_n2, PH == 0 ? sBias0 : sBias1);
         dma_k(t_n1, 0, KBUF(PH ^ 1, 0));
         dma_v(t_cur, 0, VBUF(PH, 0));
-        iter(P0{}, std::integral_constant<int, 0>{}, t_cur, t_n2);
+        iter(P0{}, std::integral_constant<int, 0>{}, t_cur);
       }
       t_cur = t_n1;
       t_n1 = t_n2;
@@ -585,14 +594,14 @@ int launch_triattn_flash(const TriAttnArgs& a, hipStream_t stream) {
   if (forced == 1 || forced == 2) R = forced;
   // static LDS: K / V buffers, the staged bias (32 KB), small arrays; dynamic: the mask codes.
   // Two workgroups must fit a CU's 160 KB.
-  const size_t stat2 = 8 * TILE_BYTES + (a.bias ? 4 * 8192 : 16) + 512;
+  const size_t stat2 = 8 * TILE_BYTES + (a.bias ? 8 * 4096 : 32) + 512;
   if (R == 2 && stat2 + 2 * (size_t)nkt * KT * sizeof(uint16_t) > 80 * 1024) R = 1;
   const int NG = (a.N + R - 1) / R;
   const int64_t blocks = ((int64_t)H * NG + 7) / 8 * 8 * QT;
   if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
   const size_t dyn = (size_t)R * nkt * KT * sizeof(uint16_t);
   const dim3 grid((unsigned)blocks), block(256);
-  const size_t stat = (R == 2 ? 8 : 4) * TILE_BYTES + (a.bias ? 4 * 8192 : 16) + 512;
+  const size_t stat = (R == 2 ? 8 : 4) * TILE_BYTES + (a.bias ? 8 * 4096 : 32) + 512;
   auto launch = [&](void (*kernel)(TriAttnArgs)) {
     // more than 64 KB of LDS per workgroup in all (static + dynamic) has to be asked for
     // (a per-function, per-device setting of the runtime: no allocation, no synchronisation)

@@ -566,17 +566,17 @@ def triangle_contraction(a, b, out=None):
 
 
 def pack_pair_bias(bias):
-    """[4, N, >=N] pair bias (already multiplied by log2(e)) -> the order of the
-    attention core's score accumulator: fp32 [4, ceil(N/32), ceil(N/64), 8, 2, 32, 4] with
-    packed[h, qb, kt, g, hh, j, e] = bias[h, 32 qb + j, 64 kt + 8 g + 4 hh + e], zero where
+    """[4, N, >=N] pair bias (already multiplied by log2(e)) -> the MFMA-fragment
+    order the attention core reads: fp16 [4, ceil(N/32), ceil(N/64), 4, 32, 16] with
+    packed[h, qb, kt, i, j, c] = bias[h, 32 qb + j, 64 kt + 16 i + c], zero where
     the query or key index is >= N."""
     if bias.dim() != 3 or bias.shape[0] != 4 or bias.shape[2] < bias.shape[1]:
         raise ValueError("bias: expected [4, N, >=N]")
     n = bias.shape[1]
     qb, kt = (n + 31) // 32, (n + 63) // 64
-    full = torch.zeros((4, qb * 32, kt * 64), dtype=torch.float32, device=bias.device)
-    full[:, :n, :n] = bias[:, :, :n].to(torch.float32)
-    return full.view(4, qb, 32, kt, 8, 2, 4).permute(0, 1, 3, 4, 5, 2, 6).contiguous()
+    full = torch.zeros((4, qb * 32, kt * 64), dtype=torch.float16, device=bias.device)
+    full[:, :n, :n] = bias[:, :, :n].float().clamp(-65504.0, 65504.0).to(torch.float16)
+    return full.view(4, qb, 32, kt, 4, 16).permute(0, 1, 3, 4, 2, 5).contiguous()
 
 
 def pack_vt(vt):
@@ -608,7 +608,7 @@ def grid_attention_core(q, k, vt, g, pair_bias, mask, out=None):
     _gpu(g, "g", torch.bfloat16, q.shape)
     _gpu(vt, "vt", torch.bfloat16, (n, 4, 32, ld))
     if pair_bias is not None:
-        _gpu(pair_bias, "pair_bias", torch.float32, (4, (n + 31) // 32, (n + 63) // 64, 8, 2, 32, 4))
+        _gpu(pair_bias, "pair_bias", torch.float16, (4, (n + 31) // 32, (n + 63) // 64, 4, 32, 16))
     maskf = _mask_f32(mask, (n, n), "mask")
     if out is None:
         out = torch.empty((n * n, 128), dtype=torch.bfloat16, device=q.device)

@@ -378,12 +378,11 @@ int af3_linear_forward(
  *     vt bf16 [b][h][32][ld] = value transposed, key k of a row stored at column
  *       (k & ~12) | ((k & 8) >> 1) | ((k & 4) << 1) (inside every aligned group of 16 keys
  *       the two middle quads are swapped), columns of keys >= n_token zero;
- *     pair_bias fp32 = bias * log2(e) in the order of the kernel's score accumulator, or
- *       NULL: element (h, q, k) at
- *       ((((h*QB + q/32)*KT + k/64)*8 + (k%64)/8)*64 + ((k%8)/4)*32 + q%32)*4 + k%4,
+ *     pair_bias fp16 = bias * log2(e) in MFMA-fragment order, or NULL: element (h, q, k) at
+ *       ((((h*QB + q/32)*KT + k/64)*4 + (k%64)/16)*32 + q%32)*16 + k%16,
  *       QB = ceil(N/32), KT = ceil(N/64), 4*QB*KT*2048 elements, keys >= N zero
- *       (per head, 32-query block and 64-key tile: eight contiguous 1 KB runs, each
- *       filling four accumulator registers of every lane with one 16-byte load);
+ *       (per head, 32-query block and 64-key tile: four contiguous 1 KB runs, each
+ *       the B operand of one identity-matrix MFMA that adds the bias to the logits);
  *   key mask [N][N] fp32 0/1 or NULL;
  *   og [(b*N + s)][128] = gate * softmax(q k^T + bias) v.
  */
@@ -391,7 +390,7 @@ int af3_triangle_contraction_forward(
     const uint16_t* a, const uint16_t* b, uint16_t* t, int64_t n_token, af3_stream_t stream);
 int af3_grid_attention_core_forward(
     const uint16_t* q, const uint16_t* k, const uint16_t* vt, const uint16_t* g,
-    const float* pair_bias, const float* mask, uint16_t* og, int64_t n_token, af3_stream_t stream);
+    const uint16_t* pair_bias, const float* mask, uint16_t* og, int64_t n_token, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
  * fp32 check mode.  Plain fp32 kernels (fp32 storage, fp32 FMA arithmetic, no
