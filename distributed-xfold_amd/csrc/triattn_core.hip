@@ -534,11 +534,24 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
     const int v_d = tid >> 3, c8 = (tid & 7) * 8;
     const bf16_t* vrow = a.vt + (((int64_t)brow[r] * H + h) * D + v_d) * a.ldn;
     float acc = 0.f;
-    for (int k0 = c8; k0 < ldn; k0 += 64) {  // columns N..ldn-1 are zero
-      float f[8];
-      unpack8(*reinterpret_cast<const u32x4*>(vrow + k0), f);
+    // columns N..ldn-1 are zero; eight loads in flight at a time (one at a time, each waits out a
+    // trip to memory, and a row of padding costs as much as a row of attention)
+    for (int kb = c8; kb < ldn; kb += 512) {
+      u32x4 raw[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc += f[e];
+      for (int i = 0; i < 8; ++i) {
+        const int k0 = kb + 64 * i;
+        raw[i] = *reinterpret_cast<const u32x4*>(vrow + (k0 < ldn ? k0 : c8));
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float f[8];
+        unpack8(raw[i], f);
+        if (kb + 64 * i < ldn) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc += f[e];
+        }
+      }
     }
     acc += __shfl_xor(acc, 1);
     acc += __shfl_xor(acc, 2);
