@@ -137,6 +137,7 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
   __shared__ __attribute__((aligned(1024))) char sBias1[HAS_BIAS ? 4 * 4096 : 16];
   __shared__ uint32_t sLive[R * 5];  // per row: live tiles (2 words), any live key, wholly unmasked tiles (2 words)
   __shared__ float sMean[D];
+  __shared__ uint32_t sRedo;  // a wave's unmasked-tile shortcut went wrong: the workgroup repeats its rows without it
   extern __shared__ __attribute__((aligned(16))) uint16_t sCode[];  // [R][nkt * 64] mask code per key
 #define KBUF(ph, r) ((ph) == 0 ? ((r) == 0 ? sK00 : sK01) : ((r) == 0 ? sK10 : sK11))
 #define VBUF(ph, r) ((ph) == 0 ? ((r) == 0 ? sV00 : sV01) : ((r) == 0 ? sV10 : sV11))
@@ -175,6 +176,7 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
 
   // ---- mask pass: per-key codes for the mask k-step, live key tiles, dead rows ----
   if (tid < R * 5) sLive[tid] = 0u;
+  if (tid == 0) sRedo = 0u;
   lds_barrier();
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -314,18 +316,22 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
 #pragma unroll
     for (int e = 0; e < 16; ++e) bt[0][e] = bt[1][e] = 0.f;
     bool based[R];  // some lane of the wave has moved this row's base off zero
-#pragma unroll
-    for (int r = 0; r < R; ++r) based[r] = false;
     float pend_alpha = 1.f;  // R == 1: a rescaling of O and l that waits for the tile in flight
     bool pend = false;
+    // Tiles of 64 unmasked keys take their exponentials without looking at the tile's maximum
+    // first ("fast").  Every lane of such a tile has 32 live keys, so the sum of what it got says
+    // afterwards where the scores lay: a sum that is not below 2^60 (an overflow included) means
+    // scores far above the base, a row total below 2^-30 scores far below it.  Either is rare,
+    // is only recorded here, and makes the whole workgroup repeat its rows with every tile on
+    // the careful route.
+    bool allow_fast = true;
+    uint64_t bad = 0ull;
 #ifdef AF3_PROF
     long long prof[6] = {0, 0, 0, 0, 0, 0};
     long long tlast = __builtin_readcyclecounter();
     const long long tstart = tlast;
 #endif
     u32x4 pp[4];  // probabilities of the previous virtual tile (bf16 B fragments), zero before the first
-#pragma unroll
-    for (int s = 0; s < 4; ++s) pp[s] = u32x4{0u, 0u, 0u, 0u};
 
     // One virtual tile = (key tile, row RR): scores, softmax, and meanwhile the previous
     // virtual tile's probabilities go into its row sums and its O.
@@ -340,7 +346,8 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       }
       // The third k-step carries the key mask and the base.  A tile of 64 unmasked keys whose row
       // still has base 0 in every lane needs neither (wave-uniform).
-      const bool step3 = based[RR] || tile >= 64 || ((plain[RR] >> tile) & 1ull) == 0ull;
+      const bool fast = allow_fast && tile < 64 && ((plain[RR] >> tile) & 1ull) != 0ull;
+      const bool step3 = based[RR] || !fast;
       const bf16x8 k00 = lds16(kb + ka0), k01 = lds16(kb + ka1);
       const bf16x8 k10 = lds16(kb + 2048 + ka0), k11 = lds16(kb + 2048 + ka1);
       bf16x8 af0, af1;
@@ -356,6 +363,7 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
         s1 = mfma32(af1, as_frag(qm[RR]), s1);
       }
 
+      if (!fast) {
       float mx = max32(s0, s1);
       mx = fmaxf(mx, half_swap(xaddr, mx));
       STAMP(5);
@@ -395,6 +403,8 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       } else {
         mrel[RR] = mnew;
       }
+      }
+      float linc = 0.f;
       STAMP(2);
       // From here to the end: one basic block in a fixed order.  Each of the four P.V MFMAs of the
       // previous virtual tile is issued in front of eight exponentials of this one (the matrix
@@ -432,8 +442,15 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
         // pins the exponentials to this group (without it they sink to where their values are used,
         // the next iteration's MFMAs)
         asm volatile("" : "+v"(pp[s].x), "+v"(pp[s].y), "+v"(pp[s].z), "+v"(pp[s].w));
-        lrun[RR] = dot2_ones(pp[s].w, dot2_ones(pp[s].z, dot2_ones(pp[s].y, dot2_ones(pp[s].x, lrun[RR]))));
+        linc = dot2_ones(pp[s].w, dot2_ones(pp[s].z, dot2_ones(pp[s].y, dot2_ones(pp[s].x, linc))));
         __builtin_amdgcn_sched_barrier(0);
+      }
+      lrun[RR] += linc;
+      if (fast) {
+        bad |= __ballot(!(linc < 0x1p60f) || lrun[RR] < 0x1p-30f);
+        // if that was fine, the row total is at least 2^-30 over at most 4096 keys: a lower bound of the
+        // running maximum, the same in both half-waves, all the careful route's lower guard needs
+        mrel[RR] = fmaxf(mrel[RR], -42.f);
       }
       STAMP(3);
     };
@@ -445,6 +462,25 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       for (int s = 0; s < 4; ++s) o[PR] = mfma32(lds16(vb + va[s]), as_frag(pp[s]), o[PR]);
     };
 
+#pragma nounroll
+    for (int pass = 0; pass < 2; ++pass) {
+    allow_fast = pass == 0;
+    bad = 0ull;
+    rest = live;
+    seq = 0;
+    pend = false;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) pp[s] = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[r][e] = 0.f;
+      lrun[r] = 0.f;
+      base[r] = 0.f;
+      mrel[r] = -__builtin_huge_valf();
+      qm[r].x = hh == 0 ? (BF16_ONE | 0x80000000u) : 0u;
+      based[r] = false;
+    }
     int t_cur = pop(), t_n1 = pop(), t_n2 = pop();
     // the buffer the first virtual tile reads its "previous" V^T from must hold finite data
     *reinterpret_cast<u32x4*>(VBUF(1, R - 1) + tid * 16) = u32x4{0u, 0u, 0u, 0u};
@@ -511,6 +547,11 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
     }
     dma_barrier();  // every load into LDS has landed (none is in flight when the workgroup ends)
     drain(last_ph == 0 ? VBUF(0, R - 1) : VBUF(1, R - 1));
+    if (pass == 1) break;
+    if (bad != 0ull && lane == 0) sRedo = 1u;
+    lds_barrier();  // also: every wave is done with the K / V^T tiles before a second pass loads over them
+    if (__builtin_amdgcn_readfirstlane(sRedo) == 0u) break;
+    }
 #ifdef AF3_PROF
     if (lane == 0) {
       long long* dst = reinterpret_cast<long long*>(a.og + ((int64_t)brow[0] * N + q0 + wave * 32) * 128 + h * D);

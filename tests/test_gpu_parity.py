@@ -411,17 +411,22 @@ def test_kernel_level_contraction(gpu_pkg, n):
     assert_within_bf16_ulp("contraction", t[:, :, :n], want, ulps=1.01, atol=1e-3)
 
 
-def _attention_core_case(gpu_pkg, n, tiles, scale=0.7, bias_shift=0.0, seed=None):
+def _attention_core_case(gpu_pkg, n, tiles, scale=0.7, bias_shift=0.0, seed=None, dense=False):
     g = gen(n + tiles if seed is None else seed)
     log2e = 1.4426950408889634
     d = dev()
     qkvg = rb(torch.randn(n, n, 4, 4, 32, generator=g) * scale)     # [b, s, (q k v g), h, d]
     qkvg[:, :, 2] = rb(qkvg[:, :, 2] * (0.7 / scale))
     qkvg[:, :, 3] = torch.sigmoid(qkvg[:, :, 3] * (0.7 / scale)).bfloat16().float()
-    bias = rb(torch.randn(4, n, n, generator=g)) + bias_shift
+    # the kernel-level entry point takes the bias in fp16: the reference sees the same values
+    bias = (rb(torch.randn(4, n, n, generator=g)) + bias_shift).half().float()
     mask = (torch.rand(n, n, generator=g) > 0.2).float()
     mask[:, 0] = 1
-    if tiles:
+    if dense:
+        # whole tiles of unmasked keys (the common case of the trunk); every third row padded at the end
+        mask[:] = 1
+        mask[::3, n - 37:] = 0
+    elif tiles:
         mask[:, 64:128] = 0                                         # tile 1 masked for every row ...
         mask[5, :] = 0
         mask[5, 100] = 1                                            # ... but the only live one of row 5
@@ -466,13 +471,29 @@ def test_kernel_level_attention_core(gpu_pkg, n, tiles):
     assert e_rms < 5e-3 and e_max < (5e-2 if n <= 400 else 7e-2)
 
 
-@pytest.mark.parametrize("n,scale,shift", [(200, 2.5, 0.0), (200, 0.7, -24.0), (200, 0.7, 40.0), (520, 2.5, -12.0)])
+@pytest.mark.parametrize("n,scale,shift", [(200, 0.7, 0.0), (576, 0.7, 0.0), (200, 2.5, 0.0), (330, 0.7, -45.0),
+                                           (200, 0.7, 70.0), (520, 2.5, -300.0), (515, 3.0, 500.0)])
+def test_kernel_level_attention_core_unmasked_tiles(gpu_pkg, n, scale, shift):
+    """Tiles of 64 unmasked keys take their exponentials before the kernel knows the tile's
+    maximum and check the sums afterwards.  Moderate logits (the first two cases) never fail that
+    check; |q.k| up to ~150 in base 2 and biases of -45 / +50 do, in both directions, and the
+    kernel then has to repair the tile and move its base (the softmax is shift-invariant)."""
+    note(f"test_kernel_level_attention_core_unmasked_tiles n={n} scale={scale} shift={shift}")
+    og, want = _attention_core_case(gpu_pkg, n, False, scale=scale, bias_shift=shift, seed=11 * n + int(shift),
+                                    dense=True)
+    assert torch.isfinite(og).all()
+    e_max, e_rms = _errs(og.cpu(), want.cpu())
+    note(f"attention core, unmasked tiles, n={n} scale={scale} shift={shift}: max {e_max:.3e} rms {e_rms:.3e}")
+    # as in the two tests beside this one
+    assert e_rms < 8e-3 and e_max < 8e-2
+
+
+@pytest.mark.parametrize("n,scale,shift", [(200, 2.5, 0.0), (200, 0.7, -300.0), (200, 0.7, 500.0), (520, 2.5, -12.0)])
 def test_kernel_level_attention_core_large_logits(gpu_pkg, n, scale, shift):
-    """Logits far from zero (|q.k| up to ~150 in base 2, biases shifted by -24 / +40): the kernel's
+    """Logits far from zero (|q.k| up to ~150 in base 2, biases shifted by -300 / +500): the kernel's
     softmax base, which it only moves when a tile's scores leave a window around it, has to
-    follow; the result must be the same softmax, which is shift-invariant.  (The kernel takes the
-    bias in fp16: its rounding, 2^-11 of the bias itself, stays below the bf16 rounding of the
-    probabilities for |bias| up to a few tens, which is why the shifts stop there.)"""
+    follow; the result must be the same softmax, which is shift-invariant.  (The reference takes
+    the bias as the kernel does, rounded to fp16.)"""
     note(f"test_kernel_level_attention_core_large_logits n={n} scale={scale} shift={shift}")
     og, want = _attention_core_case(gpu_pkg, n, True, scale=scale, bias_shift=shift, seed=7 * n + int(shift))
     assert torch.isfinite(og).all()
