@@ -331,6 +331,7 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
     long long tlast = __builtin_readcyclecounter();
     const long long tstart = tlast;
 #endif
+    bf16x8 kpre[4];  // R == 2: row 0's K fragments of the next key tile
     u32x4 pp[4];  // probabilities of the previous virtual tile (bf16 B fragments), zero before the first
 
     // One virtual tile = (key tile, row RR): scores, softmax, and meanwhile the previous
@@ -348,8 +349,11 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       // still has base 0 in every lane needs neither (wave-uniform).
       const bool fast = allow_fast && tile < 64 && ((plain[RR] >> tile) & 1ull) != 0ull;
       const bool step3 = based[RR] || !fast;
-      const bf16x8 k00 = lds16(kb + ka0), k01 = lds16(kb + ka1);
-      const bf16x8 k10 = lds16(kb + 2048 + ka0), k11 = lds16(kb + 2048 + ka1);
+      // Two rows per wave: row 0's K tile has been in LDS since the barrier before the previous
+      // virtual tile, whose last group of exponentials fetched these fragments (kpre).
+      const bool pre = R == 2 && RR == 0;
+      const bf16x8 k00 = pre ? kpre[0] : lds16(kb + ka0), k01 = pre ? kpre[1] : lds16(kb + ka1);
+      const bf16x8 k10 = pre ? kpre[2] : lds16(kb + 2048 + ka0), k11 = pre ? kpre[3] : lds16(kb + 2048 + ka1);
       bf16x8 af0, af1;
       f32x16 s0, s1;
       STAMP(4);
@@ -423,6 +427,13 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
         const bf16x8 vcur = vf;
         if (s < 3) {
           vf = lds16(vb + va[s + 1]);
+          __builtin_amdgcn_sched_barrier(0);
+        } else if (R == 2 && RR == 1) {
+          const char* kn = KBUF(PH ^ 1, 0);
+          kpre[0] = lds16(kn + ka0);
+          kpre[1] = lds16(kn + ka1);
+          kpre[2] = lds16(kn + 2048 + ka0);
+          kpre[3] = lds16(kn + 2048 + ka1);
           __builtin_amdgcn_sched_barrier(0);
         }
         o[PR] = mfma32(vcur, as_frag(pp[s]), o[PR]);
@@ -500,6 +511,10 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       dma_v(t_cur, 0, VBUF(0, 0));
       dma_v(t_cur, 1, VBUF(0, 1));
       dma_barrier();
+      kpre[0] = lds16(KBUF(0, 0) + ka0);
+      kpre[1] = lds16(KBUF(0, 0) + ka1);
+      kpre[2] = lds16(KBUF(0, 0) + 2048 + ka0);
+      kpre[3] = lds16(KBUF(0, 0) + 2048 + ka1);
     }
     // Every ordinary load issued so far (Q, the first bias tile) is waited for HERE, with a wait
     // the compiler can see: otherwise it keeps a vmcnt(0) for them at the top of the loop, where
