@@ -339,36 +339,36 @@ def main():
     seq_mask, pair_mask = masks(live)
     seq_ones, pair_ones = masks(n)
 
-    def step():
-        blk(pair, pair_mask, single, seq_mask)
+    # A step is one Pairformer block.  The timed steps run back to back the way the trunk runs its 48
+    # blocks (nn.pairformer_loop): block i's update of `single`, a chain of small kernels, goes on a second
+    # stream beside block i + 1's pair operators.  Everything launched is waited for before the clock stops.
+    # `isolated` is the same block called on its own, one stream, per call.
+    loop = pkg.nn.pairformer_loop
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-    if not torch.isfinite(pair.float()).all():
-        raise RuntimeError("non-finite pair activations after the timed steps")
+    def timed(pm, sm):
+        loop([blk] * args.warmup, pair, pm, single, sm)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        loop([blk] * args.steps, pair, pm, single, sm)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        if not torch.isfinite(pair.float()).all():
+            raise RuntimeError("non-finite pair activations after the timed steps")
+        pair.normal_(generator=None)
+        single.normal_(generator=None)
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            blk(pair, pm, single, sm)
+        torch.cuda.synchronize()
+        iso = (time.perf_counter() - t0) * 1e3 / args.steps
+        pair.normal_(generator=None)
+        single.normal_(generator=None)
+        return ms, iso
 
+    ms_per_step, ms_isolated = timed(pair_mask, seq_mask)
     # the same block with nothing masked: every kernel leaves out work on padding (fully masked prologue tiles,
     # rows without a live key, key tiles without one), so the padded figure flatters the kernels by that much
-    pair.normal_(generator=None)
-    single.normal_(generator=None)
-    for _ in range(args.warmup):
-        blk(pair, pair_ones, single, seq_ones)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        blk(pair, pair_ones, single, seq_ones)
-    torch.cuda.synchronize()
-    ms_unmasked = (time.perf_counter() - t0) * 1e3 / args.steps
-    if not torch.isfinite(pair.float()).all():
-        raise RuntimeError("non-finite pair activations after the timed steps (all-ones mask)")
-    pair.normal_(generator=None)
-    single.normal_(generator=None)
+    ms_unmasked, ms_unmasked_isolated = timed(pair_ones, seq_ones)
 
     # ---- per-operator breakdown (untimed with respect to the headline) ----
     it = max(3, min(args.steps, 10))
@@ -459,7 +459,10 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"one Pairformer block, N_token={n}, c_pair=128, c_single=384, "
                                f"{args.io} residual stream, bf16 MFMA operands / fp32 accumulate, "
-                               "10% trailing tokens masked, random-init weights N(0,0.02)"},
+                               "10% trailing tokens masked, random-init weights N(0,0.02); steps run back to "
+                               "back as the trunk loop runs its blocks (single update of one block on a second "
+                               "stream beside the pair operators of the next)"},
+        "isolated_block_ms": round(ms_isolated, 4),
         "block_tflops": round(flops_block(n) / ms_per_step / 1e9, 2),
         "per_op_ms": {k: round(v, 4) for k, v in per_op.items()},
         "tflops_per_op": {k: round(v, 2) for k, v in tflops_per_op.items()},
@@ -467,6 +470,7 @@ def main():
         "unmasked": {
             "workload": "the same block with all-ones masks (no padding: nothing is skipped)",
             "value": round(ms_unmasked, 4), "unit": "ms/block",
+            "isolated_block_ms": round(ms_unmasked_isolated, 4),
             "block_tflops": round(flops_block(n) / ms_unmasked / 1e9, 2),
             "per_op_ms": {k: round(v, 4) for k, v in per_op_un.items()},
             "tflops_per_op": {k: round(v, 2) for k, v in tflops_per_op_un.items()},

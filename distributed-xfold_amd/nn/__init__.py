@@ -8,7 +8,7 @@ from .attention import GridSelfAttention
 from .primitives import Transition
 from .diffusion_transformer import (AdaptiveLayerNorm, AdaLNZero, DiffusionTransition, SelfAttention,
                                     DiffusionTransformer, CrossAttention, DiffusionCrossAttTransformer)
-from .pairformer import PairformerBlock, PairformerStack
+from .pairformer import PairformerBlock, PairformerStack, pairformer_loop
 from .evoformer import OuterProductMean, MSAAttention, EvoformerBlock
 from .trunk import Evoformer
 from . import atom_layout
@@ -39,7 +39,7 @@ DistrubuteFourierEmbeddings = FourierEmbeddings
 __all__ = [
     "HipModule", "enable_hip", "check_mode", "in_check_mode", "TriangleMultiplication", "GridSelfAttention", "Transition",
     "AdaptiveLayerNorm", "AdaLNZero", "DiffusionTransition", "SelfAttention", "DiffusionTransformer",
-    "CrossAttention", "DiffusionCrossAttTransformer", "PairformerBlock", "PairformerStack",
+    "CrossAttention", "DiffusionCrossAttTransformer", "PairformerBlock", "PairformerStack", "pairformer_loop",
     "OuterProductMean", "MSAAttention", "EvoformerBlock", "Evoformer",
     "atom_layout", "AtomCrossAttEncoder", "AtomCrossAttDecoder", "AtomCrossAttEncoderOutput", "DiffusionHead",
     "DiffusionSampler", "FourierEmbeddings",

@@ -52,8 +52,15 @@ class PairformerBlock(HipModule):
                     w_logits=pad_rows(bf16(self.single_pair_logits_projection.weight), 32))
 
     def forward(self, pair: torch.Tensor, pair_mask: torch.Tensor, single: Optional[torch.Tensor] = None,
-                seq_mask: Optional[torch.Tensor] = None, head: int = 0):
-        """pair [N, N, c_pair], pair_mask [N, N], single [N, c_single], seq_mask [N]."""
+                seq_mask: Optional[torch.Tensor] = None, head: int = 0,
+                single_stream: Optional["torch.cuda.Stream"] = None):
+        """pair [N, N, c_pair], pair_mask [N, N], single [N, c_single], seq_mask [N].
+
+        `single_stream` (not in the reference): run the update of `single` (attention and
+        transition, a chain of small kernels that leave most of the GPU idle) on that
+        stream, behind the pair-bias projection, and return without waiting for it.  The
+        caller then owns the ordering: `single` may only be touched on that stream until
+        the caller's stream has waited for it (PairformerStack does both)."""
         if in_check_mode():
             return check.pairformer_block(self, pair, pair_mask, single, seq_mask)
         if not pair.is_contiguous():
@@ -68,23 +75,63 @@ class PairformerBlock(HipModule):
         if not single.is_contiguous():
             raise ValueError("single must be contiguous (it is updated in place)")
         p = self.packed()
+        # the only reader of `pair` on the single path: it stays on the caller's stream, in front of
+        # whatever updates `pair` next
         logits = ops.pair_logits(pair, p["ln_w"], p["ln_b"], p["w_logits"], self.n_heads)
-        self.single_attention_.run(single, seq_mask, logits, None, residual=True)
-        self.single_transition.run(single, residual=True)
+        if single_stream is None:
+            self.single_attention_.run(single, seq_mask, logits, None, residual=True)
+            self.single_transition.run(single, residual=True)
+            return pair, single
+        single_stream.wait_stream(torch.cuda.current_stream(pair.device))
+        logits.record_stream(single_stream)
+        with torch.cuda.stream(single_stream):
+            self.single_attention_.run(single, seq_mask, logits, None, residual=True)
+            self.single_transition.run(single, residual=True)
         return pair, single
 
 
-class PairformerStack(HipModule):
-    """The trunk loop of DistributeEvoformer.forward (d_alphafold3.py:242-244)."""
+_SIDE_STREAMS = {}
 
-    def __init__(self, num_blocks: int = 48, **block_kwargs) -> None:
+
+def _side_stream(device) -> "torch.cuda.Stream":
+    """One extra stream per device (default priority), shared by every trunk loop of the process."""
+    key = torch.device(device).index or 0
+    if key not in _SIDE_STREAMS:
+        _SIDE_STREAMS[key] = torch.cuda.Stream(device=device)
+    return _SIDE_STREAMS[key]
+
+
+def pairformer_loop(blocks, pair, pair_mask, single, seq_mask, overlap_single: bool = True):
+    """Run Pairformer blocks one after the other (the loop of d_alphafold3.py:242-244).
+
+    `overlap_single`: inside the loop nothing reads `single` but the next block's own
+    single update, so each block's single update runs on a second stream while the next
+    block's pair operators, which fill the GPU, run on the caller's; the caller's stream
+    waits for the second one before the loop returns.  The results are the same bits
+    either way."""
+    if in_check_mode() or not overlap_single or not pair.is_cuda:
+        for blk in blocks:
+            pair, single = blk(pair, pair_mask, single, seq_mask)
+        return pair, single
+    main = torch.cuda.current_stream(pair.device)
+    side = _side_stream(pair.device)
+    side.wait_stream(main)          # whatever produced `single` and `seq_mask`
+    for blk in blocks:
+        pair, single = blk(pair, pair_mask, single, seq_mask, single_stream=side)
+    main.wait_stream(side)
+    return pair, single
+
+
+class PairformerStack(HipModule):
+    """The trunk loop of DistributeEvoformer.forward (d_alphafold3.py:242-244); see pairformer_loop."""
+
+    def __init__(self, num_blocks: int = 48, overlap_single: bool = True, **block_kwargs) -> None:
         super().__init__()
         self.trunk_pairformer = nn.ModuleList([PairformerBlock(**block_kwargs) for _ in range(num_blocks)])
+        self.overlap_single = overlap_single
 
     def _pack(self):
         return {}
 
     def forward(self, pair, pair_mask, single, seq_mask):
-        for blk in self.trunk_pairformer:
-            pair, single = blk(pair, pair_mask, single, seq_mask)
-        return pair, single
+        return pairformer_loop(self.trunk_pairformer, pair, pair_mask, single, seq_mask, self.overlap_single)

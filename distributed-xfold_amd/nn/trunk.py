@@ -21,7 +21,7 @@ from .. import check, ops
 from .base import HipModule, bf16, drop_mesh, f32, in_check_mode
 from .diffusion_head import create_relative_encoding
 from .evoformer import EvoformerBlock
-from .pairformer import PairformerBlock
+from .pairformer import PairformerBlock, pairformer_loop
 
 
 def _pad_k(w: torch.Tensor) -> torch.Tensor:
@@ -136,8 +136,7 @@ class Evoformer(HipModule):
             single = single + ops.linear(ops.layer_norm(prev["single"].contiguous(), p["prevs_ln_w"], p["prevs_ln_b"]),
                                          p["w_prevs"], out_dtype=torch.float32)
         single = single.to(dt).contiguous()
-        for blk in self.trunk_pairformer:
-            pair, single = blk(pair, pair_mask, single, mask)
+        pair, single = pairformer_loop(self.trunk_pairformer, pair, pair_mask, single, mask)
         return {"single": single, "pair": pair, "target_feat": target_feat}
 
     @torch.no_grad()

@@ -102,6 +102,34 @@ def test_config0_four_block_stack_n128_fp32(gpu_pkg):
     compare("[0] stack single, fp32 check mode", cs.cpu(), es, 1e-5, 1e-4)
 
 
+def test_stack_single_update_on_second_stream_same_bits(gpu_pkg):
+    """Inside the stack each block's update of `single` runs on a second stream beside the
+    next block's pair operators.  Same kernels on the same data in the same order per tensor:
+    the results must not differ by a bit from the one-stream run, call after call."""
+    say("test_stack_single_update_on_second_stream_same_bits")
+    n, nb = 200, 6
+    g = gen(102)
+    blocks = [rparams(O.make_pairformer_block_params(g)) for _ in range(nb)]
+    state = {f"trunk_pairformer.{i}.{k}": v for i, p in enumerate(blocks) for k, v in p.items()}
+    pair = torch.randn(n, n, 128, generator=g).bfloat16().to(dev())
+    single = torch.randn(n, 384, generator=g).bfloat16().to(dev())
+    seq, pm = trailing_masks(n, n - 23)
+    seq, pm = seq.to(dev()), pm.to(dev())
+    outs = []
+    for overlap in (False, True, True):
+        stack = gpu_pkg.nn.PairformerStack(num_blocks=nb, overlap_single=overlap)
+        stack.load_state_dict(state)
+        stack.to(dev())
+        op, os_ = stack(pair.clone(), pm, single.clone(), seq)
+        # forward has made the caller's stream wait for the second one: this copy is ordered behind both
+        outs.append((op.cpu(), os_.cpu()))
+    assert torch.isfinite(outs[0][0].float()).all() and torch.isfinite(outs[0][1].float()).all()
+    assert float((outs[0][1].float() - single.cpu().float()).abs().max()) > 0
+    for op, os_ in outs[1:]:
+        assert torch.equal(op, outs[0][0])
+        assert torch.equal(os_, outs[0][1])
+
+
 # ------------------------------------------------------------------ configs[1]
 def test_config1_one_block_n384_bf16_padded(gpu_pkg):
     say("test_config1_one_block_n384_bf16_padded")
