@@ -45,10 +45,11 @@
 
 namespace {
 
-constexpr int CM = 256, CN = 256, CK = 32;
+// The block is 64 IT x 256: IT = 4 MFMA tiles per wave along i (256 x 256), or IT = 3 (192 x 256) where
+// that saves enough rounds of workgroups (N = 384: tiles of 256 would be half empty).
+constexpr int CN = 256, CK = 32;
 constexpr int ROWB = CK * 2;            // bytes of a slab row in LDS (unpadded)
-constexpr int SLAB_A = CM * ROWB;       // A rows first, then B rows
-constexpr int SLAB = (CM + CN) * ROWB;  // 32 KB
+constexpr int SLAB = (256 + CN) * ROWB;  // 32 KB at IT = 4: A rows first, then B rows
 constexpr int LDE = 128 + 8;            // LDS row stride of a wave's staged output quadrant (bf16)
 constexpr int EPI_BYTES = 128 * LDE * 2;  // one wave's output quadrant
 constexpr int BUF_BYTES = SLAB > EPI_BYTES ? SLAB : EPI_BYTES;
@@ -78,8 +79,11 @@ __device__ __forceinline__ void wait_loads_but() {
 //         matching "b" rows): output column 32 p + x = silu(a) * b of block p.
 enum { BIG_PLAIN = 0, BIG_COLUMN_OPS = 1, BIG_SWIGLU = 2 };
 
-template <int MODE>
+template <int MODE, int IT = 4>
 __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
+  constexpr int CM = 64 * IT, WM = 32 * IT;  // block and wave extent along i
+  constexpr int SLAB_A = CM * ROWB;
+  constexpr int NLOAD = IT + 4;              // loads per wave and slab
   // Four arrays, not one: the compiler then knows that a load in flight to one
   // buffer cannot alias a fragment read from another and does not make the
   // read wait for it.
@@ -92,7 +96,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hh = lane >> 5, l31 = lane & 31;
-  const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
+  const int wm = (wave >> 1) * WM, wn = (wave & 1) * 128;
 
   // XCD-aware mapping: workgroup ids are dealt round-robin to the 8 XCDs, so
   // id -> (xcd, slot) -> logical id makes each XCD walk a contiguous range of
@@ -120,8 +124,8 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   const char* A = reinterpret_cast<const char*>(g.A + (int64_t)bz * g.sA);
   const char* B = reinterpret_cast<const char*>(g.B + (int64_t)bz * g.sB);
 
-  // Per slab a wave issues four loads for A and four for B: load i covers rows
-  // 64 wave + 16 i .. + 16 (one 64-byte row per 4 lanes).  The lane at position
+  // Per slab a wave issues IT loads for A and four for B: load i covers rows
+  // 16 IT wave + 16 i .. + 16 of A, 64 wave + 16 i .. + 16 of B (one 64-byte row per 4 lanes).  The lane at position
   // pc of row r fetches chunk pc ^ ((r >> 2) & 3) = pc ^ (lane >> 4).  Rows past
   // the end repeat the last one (what they produce lands in output rows that
   // are never stored or in columns N..ldc-1 of T, which no consumer reads); a
@@ -132,19 +136,22 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   uint32_t offa[4], offb[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int row = 64 * wave + 16 * i + ld_r;
-    offa[i] = ((uint32_t)min(m0 + row, g.M - 1) * (uint32_t)g.lda + ld_c * 8) * 2u;
-    offb[i] = ((uint32_t)min(n0 + row, g.N - 1) * (uint32_t)g.ldb + ld_c * 8) * 2u;
+    const int rowa = 16 * IT * wave + 16 * i + ld_r, rowb = 64 * wave + 16 * i + ld_r;
+    offa[i] = ((uint32_t)min(m0 + rowa, g.M - 1) * (uint32_t)g.lda + ld_c * 8) * 2u;
+    offb[i] = ((uint32_t)min(n0 + rowb, g.N - 1) * (uint32_t)g.ldb + ld_c * 8) * 2u;
   }
-  // Half a slab: `first` = the wave's four loads of A, else its four of B.
+  // Half a slab: `first` = the wave's loads of A, else its four of B.
   // kt may run past the last slab (such loads re-read slab 0 and are never used).
   auto slab_load = [&](char* dst, int kt, bool first) {
     const int k0 = kt * CK;
     const uint32_t kb = k0 + ld_c * 8 < g.K ? (uint32_t)k0 * 2u : 0u;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      if (first) load_to_lds(A, offa[i] + kb, dst + (64 * wave + 16 * i) * ROWB);
-      else load_to_lds(B, offb[i] + kb, dst + SLAB_A + (64 * wave + 16 * i) * ROWB);
+      if (first) {
+        if (i < IT) load_to_lds(A, offa[i] + kb, dst + (16 * IT * wave + 16 * i) * ROWB);
+      } else {
+        load_to_lds(B, offb[i] + kb, dst + SLAB_A + (64 * wave + 16 * i) * ROWB);
+      }
     }
   };
   // Chunks at or past K of slab kt (the last slab, and the all-zero slabs that
@@ -155,7 +162,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
     const u32x4 z = {0, 0, 0, 0};
     const int swz = (tid >> 2) & 3;
     for (int c = valid; c < 4; ++c) {
-      *reinterpret_cast<u32x4*>(b + tid * ROWB + ((c ^ swz) << 4)) = z;
+      if (tid < CM) *reinterpret_cast<u32x4*>(b + tid * ROWB + ((c ^ swz) << 4)) = z;
       *reinterpret_cast<u32x4*>(b + SLAB_A + tid * ROWB + ((c ^ swz) << 4)) = z;
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -170,18 +177,18 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   const uint32_t a_base = (uint32_t)(wm * ROWB), b_base = (uint32_t)(SLAB_A + wn * ROWB);
 
   // acc[jt][it] = (T^T) tile: rows j = wn + 32 jt + .., columns i = wm + 32 it + ..
-  f32x16 acc[4][4];
+  f32x16 acc[4][IT];
 #pragma unroll
   for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
-    for (int it = 0; it < 4; ++it)
+    for (int it = 0; it < IT; ++it)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[jt][it][r] = 0.f;
 
-  bf16x8 fa[2][4], fb[2][4];  // set 0: first k-step of a slab, set 1: second
+  bf16x8 fa[2][IT], fb[2][4];  // set 0: first k-step of a slab, set 1: second
   auto frags = [&](int set, const char* b, int ks) {
 #pragma unroll
-    for (int it = 0; it < 4; ++it)
+    for (int it = 0; it < IT; ++it)
       fa[set][it] = as_frag(*reinterpret_cast<const u32x4*>(b + a_base + it * (32 * ROWB) + fo[ks]));
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt)
@@ -191,13 +198,13 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
-      for (int it = 0; it < 4; ++it) acc[jt][it] = mfma32(fb[set][jt], fa[set][it], acc[jt][it]);
+      for (int it = 0; it < IT; ++it) acc[jt][it] = mfma32(fb[set][jt], fa[set][it], acc[jt][it]);
   };
-  // 16 MFMAs with 8 fragment reads and 4 loads between them
+  // 4 IT MFMAs with IT + 4 fragment reads and up to 4 loads between them
   auto interleave = [&]() {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // two MFMAs
+      __builtin_amdgcn_sched_group_barrier(0x008, IT - 2, 0);  // two MFMAs (one when there are twelve)
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
       __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
@@ -209,7 +216,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   const int nk4 = (nk + 3) & ~3;  // stages come in fours (the buffers are addressed statically)
   // Loads in flight, oldest first, whenever a wave reaches the barrier of
   // slab kt: [slab kt + 1] [slab kt + 2] [slab kt + 3]; the barrier needs the
-  // first group, so 16 may stay outstanding.
+  // first group, so two slabs' worth may stay outstanding.
   slab_load(sb0, 0, true);
   slab_load(sb0, 0, false);
   slab_load(sb1, 1, true);
@@ -217,7 +224,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   slab_load(sb2, 2, true);
   slab_load(sb2, 2, false);
   slab_load(sb3, 3, true);
-  wait_loads_but<20>();
+  wait_loads_but<2 * NLOAD + IT>();  // everything but slab 0
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
   if (CK > g.K) slab_clear_tail(sb0, 0);
@@ -235,9 +242,9 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
     interleave();
     __builtin_amdgcn_sched_barrier(0);
     // This wave has read all it needs of slab kt; its share of slab kt + 1 has
-    // landed once at most 16 younger loads are outstanding.  Past the barrier
+    // landed once at most two slabs' worth of younger loads are outstanding.  Past the barrier
     // that holds for every wave: slab kt + 1 is complete, buffer b is free.
-    wait_loads_but<16>();
+    wait_loads_but<2 * NLOAD>();  // two slabs' worth
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     if ((kt + 2) * CK > g.K && kt + 1 < nk4) slab_clear_tail(nxt, kt + 1);
@@ -259,7 +266,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   // ------------------------------------------------------------- epilogue
   // Drain the loads that ran ahead (they target the buffers about to be
   // reused) and let every wave finish its fragment reads.  Then a wave stages
-  // its own 128x128 quadrant (rows i, columns j) in buffer `wave` and reads it
+  // its own (32 IT)x128 quadrant (rows i, columns j) in buffer `wave` and reads it
   // back itself (a wave's LDS operations execute in order): no further barrier.
   // Lane (l31, hh), register quad q of tile (jt, it): row i = 32 it + l31,
   // columns j = 32 jt + 8 q + 4 hh + 0..3.
@@ -296,7 +303,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
         }
       }
 #pragma unroll
-      for (int it = 0; it < 4; ++it) {
+      for (int it = 0; it < IT; ++it) {
         float o[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -320,7 +327,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
     const int c8 = lane & 7, rsub = lane >> 3;  // 8 chunks of 8 output columns per row, 8 rows per instruction
     const int col = (n0 + wn) / 2 + c8 * 8;
 #pragma unroll
-    for (int s = 0; s < 16; ++s) {
+    for (int s = 0; s < 4 * IT; ++s) {
       const int r = 8 * s + rsub;
       const int row = m0 + wm + r;
       const u32x4 v = *reinterpret_cast<const u32x4*>(sE + r * LDE + c8 * 8);
@@ -331,7 +338,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
     const int col = n0 + wn + c16 * 8;
     const int col_end = MODE == BIG_PLAIN ? g.ldc : g.N;
 #pragma unroll
-    for (int s = 0; s < 32; ++s) {
+    for (int s = 0; s < 8 * IT; ++s) {
       const int r = 4 * s + rsub;
       const int row = m0 + wm + r;
       const u32x4 v = *reinterpret_cast<const u32x4*>(sE + r * LDE + c16 * 8);
@@ -381,11 +388,29 @@ int launch_big_tile(const GemmArgs& g, int mode, hipStream_t stream) {
   if (!g.A || !g.B || !g.C) return AF3_ERR_BAD_ARG;
   if (mode != big_tile_mode(g) && !(mode == BIG_PLAIN && contract_supported(g))) return AF3_ERR_BAD_ARG;
   if (mode < BIG_PLAIN || mode > BIG_SWIGLU) return AF3_ERR_BAD_ARG;
-  const int64_t total = (int64_t)((g.M + CM - 1) / CM) * ((g.N + CN - 1) / CN) * g.batch;
+  const int64_t tiles_n = (g.N + CN - 1) / CN;
+  const int64_t total4 = (int64_t)((g.M + 255) / 256) * tiles_n * g.batch;
+  const int64_t total3 = (int64_t)((g.M + 191) / 192) * tiles_n * g.batch;
+  // Rounds of workgroups on the device's CUs (one workgroup per CU) times the cost of one.  A 192 x 256
+  // block costs 0.83 - 0.86 of a 256 x 256 one, not 0.75 (measured: pipeline fill and the epilogue do not
+  // shrink with it), so it is taken for the plain product only when it saves more rounds than that:
+  // N = 256 .. 576, not 768 (six rounds against five) or beyond.
+  static int cus = 0;
+  if (cus == 0) {
+    int dev_id = 0;
+    hipDeviceProp_t prop;
+    cus = hipGetDevice(&dev_id) == hipSuccess && hipGetDeviceProperties(&prop, dev_id) == hipSuccess &&
+                  prop.multiProcessorCount > 0
+              ? prop.multiProcessorCount
+              : 256;
+  }
+  const bool flat = mode == BIG_PLAIN && ((total3 + cus - 1) / cus) * 7 < ((total4 + cus - 1) / cus) * 8;
+  const int64_t total = flat ? total3 : total4;
   const int64_t blocks = (total + 7) / 8 * 8;
   if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
   const dim3 grid((unsigned)blocks), block(256);
-  if (mode == BIG_PLAIN) hipLaunchKernelGGL(contract_kernel<BIG_PLAIN>, grid, block, 0, stream, g);
+  if (flat) hipLaunchKernelGGL((contract_kernel<BIG_PLAIN, 3>), grid, block, 0, stream, g);
+  else if (mode == BIG_PLAIN) hipLaunchKernelGGL(contract_kernel<BIG_PLAIN>, grid, block, 0, stream, g);
   else if (mode == BIG_COLUMN_OPS) hipLaunchKernelGGL(contract_kernel<BIG_COLUMN_OPS>, grid, block, 0, stream, g);
   else hipLaunchKernelGGL(contract_kernel<BIG_SWIGLU>, grid, block, 0, stream, g);
   return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;

@@ -397,8 +397,10 @@ def test_bad_shape_is_rejected(gpu_pkg):
 
 
 # ---------------------------------------------------------- kernel-level entries
-@pytest.mark.parametrize("n", [70, 130, 256, 300, 360, 520])
+@pytest.mark.parametrize("n", [70, 130, 256, 300, 360, 520, 768, 1000])
 def test_kernel_level_contraction(gpu_pkg, n):
+    """The block is 192 x 256 or 256 x 256, whichever needs fewer (cost-weighted) rounds of
+    workgroups: 192 x 256 up to 520 here, 256 x 256 at 768 and 1000."""
     note(f"test_kernel_level_contraction n={n}")
     g = gen(n)
     npad = (n + 7) // 8 * 8
@@ -406,9 +408,12 @@ def test_kernel_level_contraction(gpu_pkg, n):
     b = torch.zeros(128, n, npad)
     a[:, :, :n] = rb(torch.randn(128, n, n, generator=g))
     b[:, :, :n] = rb(torch.randn(128, n, n, generator=g))
-    t = gpu_pkg.ops.triangle_contraction(a.to(dev()).bfloat16(), b.to(dev()).bfloat16())
-    want = torch.bmm(a.double(), b.double().transpose(1, 2))
-    assert_within_bf16_ulp("contraction", t[:, :, :n], want, ulps=1.01, atol=1e-3)
+    a, b = a.to(dev()), b.to(dev())
+    t = gpu_pkg.ops.triangle_contraction(a.bfloat16(), b.bfloat16())
+    want = torch.empty(128, n, n, dtype=torch.float64, device=dev())
+    for c0 in range(0, 128, 16):                                   # float64 on the GPU, 16 channels at a time
+        want[c0:c0 + 16] = torch.bmm(a[c0:c0 + 16].double(), b[c0:c0 + 16].double().transpose(1, 2))
+    assert_within_bf16_ulp("contraction", t[:, :, :n].cpu(), want.cpu(), ulps=1.01, atol=1e-3)
 
 
 def _attention_core_case(gpu_pkg, n, tiles, scale=0.7, bias_shift=0.0, seed=None, dense=False):
