@@ -9,5 +9,6 @@ library, or with tensors that are not on the GPU, every operator raises.
 
 from . import lib, ops  # noqa: F401
 from . import check, nn  # noqa: F401
+from . import torch_ops  # noqa: F401  (nothing is registered until torch_ops.register() is called)
 
-__all__ = ["lib", "ops", "nn", "check"]
+__all__ = ["lib", "ops", "nn", "check", "torch_ops"]
