@@ -96,13 +96,15 @@ size_t af3_triangle_multiplication_workspace_bytes(int64_t n) {
   return 3 * align_up((size_t)C_PAIR * n * pad8(n) * sizeof(bf16_t), 256);
 }
 
-int af3_triangle_multiplication_forward(
+static int triangle_multiplication_impl(
     const void* act, int io_dtype, const float* mask, int equation_flag,
     const float* ln_in_w, const float* ln_in_b, const uint16_t* w_proj_gate,
     const float* ln_c_w, const float* ln_c_b, const uint16_t* w_out, const uint16_t* w_gl,
-    void* out, int residual, int64_t n, void* workspace, size_t workspace_bytes, af3_stream_t stream) {
+    void* out, int residual, int64_t n, int valid_channels, void* workspace, size_t workspace_bytes,
+    af3_stream_t stream) {
   if (!act || !out || !ln_in_w || !ln_in_b || !w_proj_gate || !ln_c_w || !ln_c_b || !w_out || !w_gl)
     return AF3_ERR_BAD_ARG;
+  if (valid_channels < 8 || valid_channels > C_PAIR) return AF3_ERR_BAD_ARG;
   if (bad_dtype(io_dtype) || n <= 0 || n > 8192 || (equation_flag != 0 && equation_flag != 1)) return AF3_ERR_BAD_ARG;
   if (misaligned(act) || misaligned(out) || misaligned(mask)) return AF3_ERR_BAD_ARG;
   const int64_t np = pad8(n);
@@ -114,6 +116,7 @@ int af3_triangle_multiplication_forward(
   hipStream_t s = static_cast<hipStream_t>(stream);
 
   TriMulArgs a;
+  a.lw = ln_width(valid_channels);
   a.pair = act; a.mask = mask; a.out = out;
   a.io_f32 = io_dtype == AF3_F32; a.N = (int)n; a.Np = (int)np;
   a.outgoing = equation_flag == 0; a.residual = residual != 0;
@@ -150,18 +153,22 @@ size_t af3_grid_self_attn_workspace_bytes(int64_t n, int num_head) {
   return fast > general ? fast : general;
 }
 
-int af3_grid_self_attn_forward(
+static int grid_self_attn_impl(
     const void* pair, int io_dtype, const float* mask, int transpose,
     const float* ln_w, const float* ln_b, const uint16_t* w_pair_bias, const float* nonbatched_bias,
     const uint16_t* w_qkvg, const uint16_t* w_output, int num_head,
-    void* out, int residual, int64_t n, void* workspace, size_t workspace_bytes, af3_stream_t stream) {
+    void* out, int residual, int64_t n, int valid_channels, void* workspace, size_t workspace_bytes,
+    af3_stream_t stream) {
   if (!pair || !out || !w_qkvg || !w_output) return AF3_ERR_BAD_ARG;
+  if (valid_channels < num_head || valid_channels > C_PAIR || (num_head > 0 && valid_channels % num_head))
+    return AF3_ERR_BAD_ARG;
   if (bad_dtype(io_dtype) || n <= 0 || n > 8192 || num_head <= 0 || C_PAIR % num_head) return AF3_ERR_BAD_ARG;
   if ((ln_w == nullptr) != (ln_b == nullptr)) return AF3_ERR_BAD_ARG;
   if (w_pair_bias && nonbatched_bias) return AF3_ERR_BAD_ARG;
   if (misaligned(pair) || misaligned(out) || misaligned(mask) || misaligned(nonbatched_bias)) return AF3_ERR_BAD_ARG;
-  const int d = C_PAIR / num_head;
+  const int d = C_PAIR / num_head;  // head dimension of the (padded) operands
   if (d != 32 || num_head != 4) return AF3_ERR_UNSUPPORTED;
+  const float d_valid = (float)(valid_channels / num_head);  // what the logits are scaled by
   hipStream_t s = static_cast<hipStream_t>(stream);
   Carver ws(workspace, workspace_bytes);
   bf16_t* og = nullptr;
@@ -180,10 +187,11 @@ int af3_grid_self_attn_forward(
     uint16_t* bias = ws.take<uint16_t>((size_t)tri_bias_elems(n, num_head));
     if (!ws.ok) return AF3_ERR_WORKSPACE;
     TriAttnProjArgs p;
+    p.lw = ln_width(valid_channels);
     p.pair = pair; p.io_f32 = io_dtype == AF3_F32; p.N = (int)n; p.transpose = transpose != 0;
     p.skip_ln = ln_w == nullptr; p.ln_w = ln_w; p.ln_b = ln_b;
     p.w_qkvg = w_qkvg; p.w_bias = w_pair_bias; p.n_bias = w_pair_bias ? num_head : 0;
-    p.q_scale = LOG2E / sqrtf((float)d); p.bias_scale = LOG2E;
+    p.q_scale = LOG2E / sqrtf(d_valid); p.bias_scale = LOG2E;
     p.q = q; p.k = k; p.vt = vt; p.g = g; p.bias = bias; p.ldn = ldn;
     rc = launch_triattn_proj(p, s);
     if (rc) return rc;
@@ -198,11 +206,12 @@ int af3_grid_self_attn_forward(
     og = ws.take<bf16_t>((size_t)n * n * C_PAIR);
     if (!ws.ok) return AF3_ERR_WORKSPACE;
     AttnProjArgs p;
+    p.lw = ln_width(valid_channels);
     p.pair = pair; p.io_f32 = io_dtype == AF3_F32; p.N = (int)n; p.transpose = transpose != 0;
     p.ln_w = ln_w; p.ln_b = ln_b; p.skip_ln = ln_w == nullptr;
     p.w_main = w_qkvg; p.n_chunks = 4;
     p.chunk_ops = SEG_BIAS_SCALE | (SEG_PLAIN << 4) | (SEG_PLAIN << 8) | (SEG_SIGMOID << 12);
-    p.q_scale = 1.0f / sqrtf((float)d);
+    p.q_scale = 1.0f / sqrtf(d_valid);
     p.out_main = qkvg; p.ld_main = 4 * C_PAIR;
     rc = launch_attn_proj(p, s);
     if (rc) return rc;
@@ -225,16 +234,67 @@ int af3_grid_self_attn_forward(
 }
 
 // -------------------------------------------------------------------- transition
+static int transition_impl(
+    const void* act, int io_dtype, const float* ln_w, const float* ln_b,
+    const uint16_t* w1_packed, const uint16_t* w2, int hidden,
+    void* out, int residual, int64_t rows, int valid_channels, af3_stream_t stream) {
+  if (!act || !out || !ln_w || !ln_b || !w1_packed || !w2) return AF3_ERR_BAD_ARG;
+  if (bad_dtype(io_dtype) || rows <= 0 || rows > 0x7fffffff || hidden <= 0 || (hidden & 63)) return AF3_ERR_BAD_ARG;
+  if (valid_channels < 8 || valid_channels > C_PAIR) return AF3_ERR_BAD_ARG;
+  TransitionArgs t;
+  t.lw = ln_width(valid_channels);
+  t.x = act; t.out = out; t.io_f32 = io_dtype == AF3_F32; t.N = (int)rows; t.hidden = hidden;
+  t.residual = residual != 0; t.ln_w = ln_w; t.ln_b = ln_b; t.w1 = w1_packed; t.w2 = w2;
+  return launch_transition(t, static_cast<hipStream_t>(stream));
+}
+
+// The public forms: all 128 channels real, or the tensor and every weight zero-padded to 128 channels
+// with `valid_channels` of them real.
+int af3_triangle_multiplication_forward(
+    const void* act, int io_dtype, const float* mask, int equation_flag,
+    const float* ln_in_w, const float* ln_in_b, const uint16_t* w_proj_gate,
+    const float* ln_c_w, const float* ln_c_b, const uint16_t* w_out, const uint16_t* w_gl,
+    void* out, int residual, int64_t n, void* workspace, size_t workspace_bytes, af3_stream_t stream) {
+  return triangle_multiplication_impl(act, io_dtype, mask, equation_flag, ln_in_w, ln_in_b, w_proj_gate, ln_c_w, ln_c_b,
+                                      w_out, w_gl, out, residual, n, C_PAIR, workspace, workspace_bytes, stream);
+}
+int af3_triangle_multiplication_forward_padded(
+    const void* act, int io_dtype, const float* mask, int equation_flag,
+    const float* ln_in_w, const float* ln_in_b, const uint16_t* w_proj_gate,
+    const float* ln_c_w, const float* ln_c_b, const uint16_t* w_out, const uint16_t* w_gl,
+    void* out, int residual, int64_t n, int valid_channels, void* workspace, size_t workspace_bytes,
+    af3_stream_t stream) {
+  return triangle_multiplication_impl(act, io_dtype, mask, equation_flag, ln_in_w, ln_in_b, w_proj_gate, ln_c_w, ln_c_b,
+                                      w_out, w_gl, out, residual, n, valid_channels, workspace, workspace_bytes, stream);
+}
+int af3_grid_self_attn_forward(
+    const void* pair, int io_dtype, const float* mask, int transpose,
+    const float* ln_w, const float* ln_b, const uint16_t* w_pair_bias, const float* nonbatched_bias,
+    const uint16_t* w_qkvg, const uint16_t* w_output, int num_head,
+    void* out, int residual, int64_t n, void* workspace, size_t workspace_bytes, af3_stream_t stream) {
+  return grid_self_attn_impl(pair, io_dtype, mask, transpose, ln_w, ln_b, w_pair_bias, nonbatched_bias, w_qkvg, w_output,
+                             num_head, out, residual, n, C_PAIR, workspace, workspace_bytes, stream);
+}
+int af3_grid_self_attn_forward_padded(
+    const void* pair, int io_dtype, const float* mask, int transpose,
+    const float* ln_w, const float* ln_b, const uint16_t* w_pair_bias, const float* nonbatched_bias,
+    const uint16_t* w_qkvg, const uint16_t* w_output, int num_head,
+    void* out, int residual, int64_t n, int valid_channels, void* workspace, size_t workspace_bytes,
+    af3_stream_t stream) {
+  return grid_self_attn_impl(pair, io_dtype, mask, transpose, ln_w, ln_b, w_pair_bias, nonbatched_bias, w_qkvg, w_output,
+                             num_head, out, residual, n, valid_channels, workspace, workspace_bytes, stream);
+}
 int af3_transition_forward(
     const void* act, int io_dtype, const float* ln_w, const float* ln_b,
     const uint16_t* w1_packed, const uint16_t* w2, int hidden,
     void* out, int residual, int64_t rows, af3_stream_t stream) {
-  if (!act || !out || !ln_w || !ln_b || !w1_packed || !w2) return AF3_ERR_BAD_ARG;
-  if (bad_dtype(io_dtype) || rows <= 0 || rows > 0x7fffffff || hidden <= 0 || (hidden & 63)) return AF3_ERR_BAD_ARG;
-  TransitionArgs t;
-  t.x = act; t.out = out; t.io_f32 = io_dtype == AF3_F32; t.N = (int)rows; t.hidden = hidden;
-  t.residual = residual != 0; t.ln_w = ln_w; t.ln_b = ln_b; t.w1 = w1_packed; t.w2 = w2;
-  return launch_transition(t, static_cast<hipStream_t>(stream));
+  return transition_impl(act, io_dtype, ln_w, ln_b, w1_packed, w2, hidden, out, residual, rows, C_PAIR, stream);
+}
+int af3_transition_forward_padded(
+    const void* act, int io_dtype, const float* ln_w, const float* ln_b,
+    const uint16_t* w1_packed, const uint16_t* w2, int hidden,
+    void* out, int residual, int64_t rows, int valid_channels, af3_stream_t stream) {
+  return transition_impl(act, io_dtype, ln_w, ln_b, w1_packed, w2, hidden, out, residual, rows, valid_channels, stream);
 }
 
 // ------------------------------------------- pair-biased self-attention (single / diffusion)

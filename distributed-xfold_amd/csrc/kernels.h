@@ -77,7 +77,23 @@ int launch_transpose(const bf16_t* in, bf16_t* out, int64_t rows, int64_t cols, 
 
 // -------------------------------------------------------------- pair_tile.hip
 // Residual-stream tensors (`pair`, `out`, `x`) are bf16 or fp32 (io_f32).
+// LayerNorm over fewer than 128 real channels: the tensor and the weights are zero-padded to 128 and the
+// statistics are taken over `valid` channels (sums over all 128 are sums over the valid ones; the padded
+// channels' share of the squared deviations, pad * mean^2, is taken out again).  valid = 128: pad = 0,
+// the same arithmetic bit for bit.
+struct LnWidth {
+  float inv_c = 1.f / 128.f;  // 1 / valid channels
+  float pad = 0.f;            // 128 - valid channels
+};
+inline LnWidth ln_width(int valid) {
+  LnWidth w;
+  w.inv_c = 1.f / (float)valid;
+  w.pad = (float)(128 - valid);
+  return w;
+}
+
 struct TriMulArgs {
+  LnWidth lw;
   const void* pair = nullptr;   // [N][N][128]
   const float* mask = nullptr;  // [N][N] 0/1 or null
   void* out = nullptr;          // [N][N][128]; may alias pair when residual
@@ -93,6 +109,7 @@ int launch_trimul_prologue(const TriMulArgs& a, hipStream_t s);
 int launch_trimul_epilogue(const TriMulArgs& a, hipStream_t s);
 
 struct AttnProjArgs {
+  LnWidth lw;
   const void* pair = nullptr;  // [N][N][128]
   int io_f32 = 0, N = 0, transpose = 0;
   int skip_ln = 0;  // pair is already normalised
@@ -122,6 +139,7 @@ struct AttnOutArgs {
 int launch_attn_out(const AttnOutArgs& a, hipStream_t s);
 
 struct TransitionArgs {
+  LnWidth lw;
   const void* x = nullptr;  // [N][128]
   void* out = nullptr;
   int io_f32 = 0, N = 0, hidden = 0, residual = 0;
@@ -188,6 +206,7 @@ __host__ __device__ inline int64_t tri_bias_offset(int64_t n, int h, int q, int 
 }
 
 struct TriAttnProjArgs {
+  LnWidth lw;
   const void* pair = nullptr;  // [N][N][128]
   int io_f32 = 0, N = 0, transpose = 0, skip_ln = 0;
   const float *ln_w = nullptr, *ln_b = nullptr;

@@ -74,7 +74,7 @@ __global__ __launch_bounds__(256, 3) void trimul_prologue_kernel(TriMulArgs a) {
   }
   wload(0);
   if (tid < TM) sMask[tid] = mk;
-  load_ln_tile<TIO>(x, t, a.ln_in_w, a.ln_in_b, sX, tid);
+  load_ln_tile<TIO>(x, t, a.ln_in_w, a.ln_in_b, sX, tid, false, a.lw.inv_c, a.lw.pad);
   wstore();
   lds_barrier();
   bf16x8 xf[8];
@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256, 2) void trimul_epilogue_kernel(TriMulArgs a) {
   }
 
   // 1. output gate from the LayerNorm-ed input: sigmoid(LN(x) Wgl^T), T form, kept in registers
-  load_ln_tile<TIO>(x, t, a.ln_in_w, a.ln_in_b, sX, tid);
+  load_ln_tile<TIO>(x, t, a.ln_in_w, a.ln_in_b, sX, tid, false, a.lw.inv_c, a.lw.pad);
   wr.store(sW, tid);
   wr.load(a.w_out, tid);
   lds_barrier();
@@ -192,14 +192,14 @@ __global__ __launch_bounds__(256, 2) void trimul_epilogue_kernel(TriMulArgs a) {
         s1 += v[ks][e];
       }
     s1 += half_swap(xaddr, s1);
-    const float mean = s1 * (1.f / C);
+    const float mean = s1 * a.lw.inv_c;
     float s2 = 0.f;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
       for (int e = 0; e < 8; ++e) { const float d = v[ks][e] - mean; s2 += d * d; }
     s2 += half_swap(xaddr, s2);
-    const float rstd = rsqrtf(s2 * (1.f / C) + LN_EPS);
+    const float rstd = rsqrtf((s2 - a.lw.pad * mean * mean) * a.lw.inv_c + LN_EPS);
     const bool ok = t.valid(px);
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
@@ -238,7 +238,7 @@ __global__ __launch_bounds__(256, 2) void attn_proj_kernel(AttnProjArgs a) {
   // (b, s) = (o, r): for the transposed operator a tile is a column segment
   const Tile t = make_tile(a.N, a.transpose != 0);
   const TIO* x = reinterpret_cast<const TIO*>(a.pair);
-  load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0);
+  load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0, a.lw.inv_c, a.lw.pad);
   lds_barrier();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
@@ -359,7 +359,7 @@ __global__ __launch_bounds__(256, 2) void transition_kernel(TransitionArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const Tile t = make_tile(a.N, false);
   const TIO* x = reinterpret_cast<const TIO*>(a.x);
-  load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid);
+  load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, false, a.lw.inv_c, a.lw.pad);
   lds_barrier();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);

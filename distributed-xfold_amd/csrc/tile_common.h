@@ -58,7 +58,8 @@ __device__ __forceinline__ void load_param8(const float* p, float fill, float* o
 // value is touched at once, costs a full memory round trip per pixel.
 template <typename TIO>
 __device__ __forceinline__ void load_ln_tile(const TIO* x, const Tile& t, const float* lnw,
-                                             const float* lnb, bf16_t* sX, int tid, bool skip_ln = false) {
+                                             const float* lnb, bf16_t* sX, int tid, bool skip_ln = false,
+                                             float inv_c = 1.f / C, float pad = 0.f) {
   using E = Elem<TIO>;
   constexpr int NB = E::kBatch;
   const int chunk = tid & 15, prow = tid >> 4;
@@ -81,11 +82,12 @@ __device__ __forceinline__ void load_ln_tile(const TIO* x, const Tile& t, const 
       float s = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) s += v[e];
-      const float mean = group16_sum(s) * (1.f / C);
+      const float mean = group16_sum(s) * inv_c;
       float q = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) { const float d = v[e] - mean; q += d * d; }
-      const float rstd = rsqrtf(group16_sum(q) * (1.f / C) + LN_EPS);
+      // (zero-padded channels, if any, each put mean^2 into the sum)
+      const float rstd = rsqrtf((group16_sum(q) - pad * mean * mean) * inv_c + LN_EPS);
       float o[8];
       const bool ok = t.valid(p);
 #pragma unroll

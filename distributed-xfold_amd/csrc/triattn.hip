@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256, 3) void triattn_proj_kernel(TriAttnProjArgs a)
     }
   };
   wload(0);
-  load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0);
+  load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0, a.lw.inv_c, a.lw.pad);
   wstore(4);
   lds_barrier();
   bf16x8 xf[8];

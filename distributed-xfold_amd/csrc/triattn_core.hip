@@ -372,7 +372,8 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       mx = fmaxf(mx, half_swap(xaddr, mx));
       STAMP(5);
       const float mnew = fmaxf(mrel[RR], mx);
-      const bool want = mx > T_HI || (mnew < T_LO && mnew > LIVE_MIN);
+      // (lanes of queries past the end have no say: in a partly filled block they see bias values nobody wrote)
+      const bool want = qw < N && (mx > T_HI || (mnew < T_LO && mnew > LIVE_MIN));
       if (__any(want)) {
         // Move the base of every query of the wave to its running maximum (rounded to bf16, the
         // form the matrix unit takes it in), rescale what the row has accumulated, and repeat the
@@ -458,7 +459,9 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       }
       lrun[RR] += linc;
       if (fast) {
-        bad |= __ballot(!(linc < 0x1p60f) || lrun[RR] < 0x1p-30f);
+        // (lanes of queries past the end work on clamped operands and, in a partly filled bias block, on
+        // bias values nobody wrote: they have no say)
+        bad |= __ballot(qw < N && (!(linc < 0x1p60f) || lrun[RR] < 0x1p-30f));
         // if that was fine, the row total is at least 2^-30 over at most 4096 keys: a lower bound of the
         // running maximum, the same in both half-waves, all the careful route's lower guard needs
         mrel[RR] = fmaxf(mrel[RR], -42.f);

@@ -25,6 +25,11 @@ SIGNATURES = {
     "af3_grid_self_attn_forward": (
         _i, [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _vp, _sz, _vp]),
     "af3_transition_forward": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _vp]),
+    "af3_triangle_multiplication_forward_padded": (
+        _i, [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i, _vp, _sz, _vp]),
+    "af3_grid_self_attn_forward_padded": (
+        _i, [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _vp, _sz, _vp]),
+    "af3_transition_forward_padded": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _vp]),
     "af3_batch_diffusion_self_attention_workspace_bytes": (_sz, [_i64, _i64, _i]),
     "af3_batch_diffusion_self_attention_forward": (
         _i, [_vp, _vp, _i64, _vp, _i, _vp, _vp, _i, _vp, _i, _i64, _i64, _i, _vp, _sz, _vp]),

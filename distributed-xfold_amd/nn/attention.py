@@ -6,7 +6,7 @@ import torch
 import torch.nn as nn
 
 from .. import check, ops
-from .base import HipModule, bf16, drop_mesh, f32, in_check_mode, pad_rows
+from .base import HipModule, bf16, drop_mesh, f32, in_check_mode, pad_channels, pad_rows, pad_to
 
 
 class GridSelfAttention(HipModule):
@@ -21,6 +21,8 @@ class GridSelfAttention(HipModule):
         if c_pair % num_head or c_pair // num_head not in (16, 24, 32, 48):
             raise ValueError("head dim must be 16, 24, 32 or 48")
         self.fused = c_pair == 128 and c_pair // num_head == 32
+        # fewer channels, four heads of at most 32: the 128-channel kernels on zero-padded operands
+        self.padded = c_pair < 128 and c_pair % 8 == 0 and num_head == 4 and c_pair // num_head <= 32
         self.c_pair, self.num_head, self.transpose = c_pair, num_head, transpose
         self.qkv_dim = c_pair // num_head
         self.act_norm = nn.LayerNorm(c_pair)
@@ -32,6 +34,19 @@ class GridSelfAttention(HipModule):
         self.output_projection = nn.Linear(c_pair, c_pair, bias=False)
 
     def _pack(self):
+        if self.padded:
+            c, h, d = self.c_pair, self.num_head, self.qkv_dim
+
+            def heads_out(w):        # [h * d, c] -> [h * 32, 128]: each head's rows at the front of a 32-row slot
+                return pad_to(w.detach().reshape(h, d, c), h, 32, 128).reshape(128, 128)
+
+            w_out = pad_to(self.output_projection.weight.detach().reshape(c, h, d), 128, h, 32).reshape(128, 128)
+            vec = lambda t: f32(pad_to(t, 128))
+            return dict(
+                w_qkvg=bf16(torch.stack([heads_out(m.weight) for m in (self.q_projection, self.k_projection,
+                                                                       self.v_projection, self.gating_query)])),
+                w_out=bf16(w_out), w_bias=bf16(pad_to(self.pair_bias_projection.weight, 32, 128)),
+                ln_w=vec(self.act_norm.weight), ln_b=vec(self.act_norm.bias))
         if not self.fused:
             return dict(
                 w_qkvg=bf16(torch.cat([self.q_projection.weight, self.k_projection.weight,
@@ -69,7 +84,20 @@ class GridSelfAttention(HipModule):
             return pair
         return upd.contiguous()
 
+    def run_padded(self, pair128, mask, residual: bool):
+        """`pair128`: the [N, N, c_pair] tensor zero-padded to 128 channels; so is the result."""
+        p = self.packed()
+        return ops.grid_self_attn(pair128, mask, self.transpose, p["ln_w"], p["ln_b"], p["w_bias"], None,
+                                  p["w_qkvg"], p["w_out"], self.num_head, residual=residual,
+                                  valid_channels=self.c_pair)
+
     def run(self, pair, mask, residual: bool):
+        if self.padded:
+            res = self.run_padded(pad_channels(pair), mask, residual)[..., :self.c_pair]
+            if residual:
+                pair.copy_(res)
+                return pair
+            return res.contiguous()
         if not self.fused:
             return self._run_other_width(pair, mask, residual)
         p = self.packed()

@@ -48,6 +48,18 @@ def f32(t: torch.Tensor) -> torch.Tensor:
     return t.detach().to(torch.float32).contiguous()
 
 
+def pad_to(w: torch.Tensor, *shape: int) -> torch.Tensor:
+    """`w` in the leading corner of a zero tensor of `shape`."""
+    out = torch.zeros(shape, dtype=w.dtype, device=w.device)
+    out[tuple(slice(0, d) for d in w.shape)] = w.detach()
+    return out
+
+
+def pad_channels(x: torch.Tensor, width: int = 128) -> torch.Tensor:
+    """[..., c] -> [..., width] with zeros behind the c real channels (a new tensor)."""
+    return torch.nn.functional.pad(x, (0, width - x.shape[-1])).contiguous()
+
+
 def pad_rows(w: torch.Tensor, multiple: int) -> torch.Tensor:
     rows = w.shape[0]
     target = (rows + multiple - 1) // multiple * multiple

@@ -9,7 +9,7 @@ import torch.nn as nn
 
 from .. import check, ops
 from .attention import GridSelfAttention
-from .base import HipModule, bf16, drop_mesh, f32, in_check_mode, pad_rows
+from .base import HipModule, bf16, drop_mesh, f32, in_check_mode, pad_channels, pad_rows
 from .diffusion_transformer import SelfAttention
 from .primitives import Transition
 from .triangle_multiplication import TriangleMultiplication
@@ -65,6 +65,17 @@ class PairformerBlock(HipModule):
             return check.pairformer_block(self, pair, pair_mask, single, seq_mask)
         if not pair.is_contiguous():
             raise ValueError("pair must be contiguous (it is updated in place)")
+        if self.c_pair < 128 and not self.with_single and self.pair_attention1.padded:
+            # the 64-channel block of the template embedding (nn/d_template.py:198-201): the five operators run
+            # on the 128-channel kernels over one zero-padded copy of the tensor, which stays padded in between
+            x = pad_channels(pair)
+            self.triangle_multiplication_outgoing.run_padded(x, pair_mask, residual=True)
+            self.triangle_multiplication_incoming.run_padded(x, pair_mask, residual=True)
+            self.pair_attention1.run_padded(x, pair_mask, residual=True)
+            self.pair_attention2.run_padded(x, pair_mask, residual=True)
+            self.pair_transition.run_padded(x, residual=True)
+            pair.copy_(x[..., :self.c_pair])
+            return pair
         self.triangle_multiplication_outgoing.run(pair, pair_mask, residual=True)
         self.triangle_multiplication_incoming.run(pair, pair_mask, residual=True)
         self.pair_attention1.run(pair, pair_mask, residual=True)

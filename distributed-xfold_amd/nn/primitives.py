@@ -8,7 +8,7 @@ import torch.nn as nn
 from .. import check
 from .. import lib as L
 from .. import ops
-from .base import HipModule, bf16, drop_mesh, f32, in_check_mode, pack_swiglu
+from .base import HipModule, bf16, drop_mesh, f32, in_check_mode, pack_swiglu, pad_channels, pad_to
 
 
 class Transition(HipModule):
@@ -32,7 +32,21 @@ class Transition(HipModule):
         self.transition1 = nn.Linear(c_x, num_intermediate_factor * c_x * 2, bias=False)
         self.transition2 = nn.Linear(num_intermediate_factor * c_x, c_x, bias=False)
 
+    @property
+    def padded(self) -> bool:
+        """Fewer than 128 channels: run on the fused 128-channel kernel with zero-padded operands."""
+        return self.c_x < 128
+
     def _pack(self):
+        if self.padded:
+            hidden = self.num_intermediate_factor * self.c_x
+            hp = (hidden + 63) // 64 * 64            # zero hidden units give silu(0) * 0 = 0
+            w1 = self.transition1.weight.detach()
+            w1p = torch.cat([pad_to(w1[:hidden], hp, 128), pad_to(w1[hidden:], hp, 128)], dim=0)
+            return dict(ln_w=f32(pad_to(self.input_layer_norm.weight, 128)),
+                        ln_b=f32(pad_to(self.input_layer_norm.bias, 128)),
+                        w1=bf16(pack_swiglu(w1p, 64)).reshape(hp // 64, 128, 128),
+                        w2=bf16(pad_to(self.transition2.weight, 128, hp)))
         d = dict(ln_w=f32(self.input_layer_norm.weight), ln_b=f32(self.input_layer_norm.bias),
                  w2=bf16(self.transition2.weight))
         if self.c_x == 128:
@@ -42,7 +56,19 @@ class Transition(HipModule):
             d["w1"] = bf16(pack_swiglu(self.transition1.weight, 32))
         return d
 
+    def run_padded(self, x128, residual: bool):
+        """`x128`: the rows zero-padded to 128 channels; so is the result."""
+        p = self.packed()
+        return ops.transition128(x128, p["ln_w"], p["ln_b"], p["w1"], p["w2"], residual=residual,
+                                 valid_channels=self.c_x)
+
     def run(self, x, residual: bool):
+        if self.padded:
+            res = self.run_padded(pad_channels(x), residual)[..., :self.c_x]
+            if residual:
+                x.copy_(res)
+                return x
+            return res.contiguous()
         p = self.packed()
         if self.c_x == 128:
             return ops.transition128(x, p["ln_w"], p["ln_b"], p["w1"], p["w2"], residual=residual)

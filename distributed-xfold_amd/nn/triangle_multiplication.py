@@ -6,7 +6,7 @@ import torch
 import torch.nn as nn
 
 from .. import check, ops
-from .base import HipModule, bf16, drop_mesh, f32, in_check_mode
+from .base import HipModule, bf16, drop_mesh, f32, in_check_mode, pad_channels, pad_to
 
 
 class TriangleMultiplication(HipModule):
@@ -35,7 +35,27 @@ class TriangleMultiplication(HipModule):
         self.c_equation = "ikc,jkc->ijc" if _outgoing else "kjc,kic->ijc"
         self.equation = "cik,cjk->cij" if _outgoing else "ckj,cki->cij"
 
+    @property
+    def padded(self) -> bool:
+        """Fewer than 128 channels: run on the 128-channel kernels with zero-padded operands."""
+        return self.c_pair < 128 and self.c_pair % 8 == 0
+
     def _pack(self):
+        if self.padded:
+            c = self.c_pair
+            chunks = []
+            for half in (0, 1):              # a, b (d_triangle_multiplication.py:162-165)
+                p = pad_to(self.projection.weight[half::2], 128, 128)
+                g = pad_to(self.gate.weight[half::2], 128, 128)
+                for lo in (0, 64):
+                    chunks.append(torch.cat([p[lo:lo + 64], g[lo:lo + 64]], dim=0))
+            vec = lambda t: f32(pad_to(t, 128))
+            return dict(
+                w_proj_gate=bf16(torch.stack(chunks)),
+                w_out=bf16(pad_to(self.output_projection.weight, 128, 128)),
+                w_gl=bf16(pad_to(self.gating_linear.weight, 128, 128)),
+                ln_in_w=vec(self.left_norm_input.weight), ln_in_b=vec(self.left_norm_input.bias),
+                ln_c_w=vec(self.center_norm.weight), ln_c_b=vec(self.center_norm.bias))
         if self.c_pair != 128:
             return dict(
                 w_proj=bf16(self.projection.weight), w_gate=bf16(self.gate.weight),
@@ -85,7 +105,20 @@ class TriangleMultiplication(HipModule):
                           gate=out_gate.view(n * n, c), residual=pair if residual else None,
                           out=pair if residual else None)
 
+    def run_padded(self, pair128: torch.Tensor, mask, residual: bool):
+        """`pair128`: the [N, N, c_pair] tensor zero-padded to 128 channels; so is the result."""
+        p = self.packed()
+        return ops.triangle_multiplication(
+            pair128, mask, 0 if self._outgoing else 1, p["ln_in_w"], p["ln_in_b"], p["w_proj_gate"],
+            p["ln_c_w"], p["ln_c_b"], p["w_out"], p["w_gl"], residual=residual, valid_channels=self.c_pair)
+
     def run(self, pair: torch.Tensor, mask, residual: bool):
+        if self.padded:
+            res = self.run_padded(pad_channels(pair), mask, residual)[..., :self.c_pair]
+            if residual:
+                pair.copy_(res)
+                return pair
+            return res.contiguous()
         if self.c_pair != 128:
             return self._run_other_width(pair, mask, residual)
         p = self.packed()

@@ -78,9 +78,10 @@ def _mask_f32(mask: Optional[torch.Tensor], shape, name: str):
 # --------------------------------------------------------------------------
 def triangle_multiplication(act, mask, equation_flag, left_norm_input_weight, left_norm_input_bias,
                             w_proj_gate, center_norm_weight, center_norm_bias,
-                            w_output_projection, w_gating_linear, residual=False, out=None):
+                            w_output_projection, w_gating_linear, residual=False, out=None, valid_channels=128):
     """traingle_multiplication_forward (csrc/Alpha_Attention.cpp:148-169); returns
-    the update, or act + update written in place when residual=True."""
+    the update, or act + update written in place when residual=True.
+    `valid_channels` < 128: tensor and weights are zero-padded to 128 channels."""
     lib = _L.load()
     _gpu(act, "act")
     if act.dim() != 3 or act.shape[0] != act.shape[1] or act.shape[2] != 128:
@@ -100,6 +101,14 @@ def triangle_multiplication(act, mask, equation_flag, left_norm_input_weight, le
         _gpu(out, "out", act.dtype, act.shape)
     nbytes = lib.af3_triangle_multiplication_workspace_bytes(n)
     ws = _ws(nbytes, act.device)
+    if valid_channels != 128:
+        rc = lib.af3_triangle_multiplication_forward_padded(
+            _p(act), io, _p(maskf), int(equation_flag), _p(left_norm_input_weight), _p(left_norm_input_bias),
+            _p(w_proj_gate), _p(center_norm_weight), _p(center_norm_bias), _p(w_output_projection),
+            _p(w_gating_linear), _p(out), int(bool(residual)), n, int(valid_channels), _p(ws), ws.numel(),
+            _stream(act.device))
+        _L.check(rc, "af3_triangle_multiplication_forward_padded")
+        return out
     rc = lib.af3_triangle_multiplication_forward(
         _p(act), io, _p(maskf), int(equation_flag), _p(left_norm_input_weight), _p(left_norm_input_bias),
         _p(w_proj_gate), _p(center_norm_weight), _p(center_norm_bias), _p(w_output_projection),
@@ -109,9 +118,10 @@ def triangle_multiplication(act, mask, equation_flag, left_norm_input_weight, le
 
 
 def grid_self_attn(pair, mask, transpose, act_norm_weight, act_norm_bias, w_pair_bias, nonbatched_bias,
-                   w_qkvg, w_output, num_head, residual=False, out=None):
+                   w_qkvg, w_output, num_head, residual=False, out=None, valid_channels=128):
     """grid_self_attn_forward (csrc/Alpha_Attention.cpp:50-70) fused with the steps
-    of DistributeGridSelfAttention.xsmm_forward (nn/d_attention.py:58-85)."""
+    of DistributeGridSelfAttention.xsmm_forward (nn/d_attention.py:58-85).
+    `valid_channels` < 128: tensor and weights are zero-padded to 128 channels."""
     lib = _L.load()
     _gpu(pair, "pair")
     if pair.dim() != 3 or pair.shape[0] != pair.shape[1] or pair.shape[2] != 128:
@@ -137,6 +147,13 @@ def grid_self_attn(pair, mask, transpose, act_norm_weight, act_norm_bias, w_pair
         _gpu(out, "out", pair.dtype, pair.shape)
     nbytes = lib.af3_grid_self_attn_workspace_bytes(n, num_head)
     ws = _ws(nbytes, pair.device)
+    if valid_channels != 128:
+        rc = lib.af3_grid_self_attn_forward_padded(
+            _p(pair), io, _p(maskf), int(bool(transpose)), _p(act_norm_weight), _p(act_norm_bias),
+            _p(w_pair_bias), _p(nonbatched_bias), _p(w_qkvg), _p(w_output), int(num_head),
+            _p(out), int(bool(residual)), n, int(valid_channels), _p(ws), ws.numel(), _stream(pair.device))
+        _L.check(rc, "af3_grid_self_attn_forward_padded")
+        return out
     rc = lib.af3_grid_self_attn_forward(
         _p(pair), io, _p(maskf), int(bool(transpose)), _p(act_norm_weight), _p(act_norm_bias),
         _p(w_pair_bias), _p(nonbatched_bias), _p(w_qkvg), _p(w_output), int(num_head),
@@ -145,8 +162,9 @@ def grid_self_attn(pair, mask, transpose, act_norm_weight, act_norm_bias, w_pair
     return out
 
 
-def transition128(act, layernorm_weight, layernorm_bias, w1_packed, w2, residual=False, out=None):
-    """transition_forward (csrc/Alpha_Attention.cpp:116-125) for 128-channel rows."""
+def transition128(act, layernorm_weight, layernorm_bias, w1_packed, w2, residual=False, out=None, valid_channels=128):
+    """transition_forward (csrc/Alpha_Attention.cpp:116-125) for 128-channel rows.
+    `valid_channels` < 128: rows and weights are zero-padded to 128 channels."""
     lib = _L.load()
     _gpu(act, "act")
     if act.shape[-1] != 128:
@@ -162,6 +180,12 @@ def transition128(act, layernorm_weight, layernorm_bias, w1_packed, w2, residual
         out = act if residual else torch.empty_like(act)
     else:
         _gpu(out, "out", act.dtype, act.shape)
+    if valid_channels != 128:
+        rc = lib.af3_transition_forward_padded(_p(act), io, _p(layernorm_weight), _p(layernorm_bias), _p(w1_packed),
+                                               _p(w2), int(hidden), _p(out), int(bool(residual)), rows,
+                                               int(valid_channels), _stream(act.device))
+        _L.check(rc, "af3_transition_forward_padded")
+        return out
     rc = lib.af3_transition_forward(_p(act), io, _p(layernorm_weight), _p(layernorm_bias), _p(w1_packed),
                                     _p(w2), int(hidden), _p(out), int(bool(residual)), rows,
                                     _stream(act.device))

@@ -119,6 +119,43 @@ int af3_transition_forward(
     void* out, int residual, int64_t rows, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * The three pair operators above on FEWER than 128 pair channels: the Pairformer
+ * blocks of the template embedding run on 64 (nn/d_template.py:198-201:
+ * PairformerBlock(c_pair=64, num_intermediate_factor=2, with_single=False)),
+ * through the same reference operators as the 128-channel trunk.  The caller
+ * zero-pads the channel axis: the tensor is [N,N,128] with channels
+ * valid_channels..127 zero, LayerNorm weights and biases are zero there, and
+ * every weight matrix has zero rows / columns for the padded channels (for the
+ * attention each head's valid_channels/num_head dimensions sit at the front of
+ * a 32-wide slot).  The kernels are the 128-channel ones; valid_channels only
+ * tells the LayerNorms how many channels their statistics cover and the
+ * attention what head dimension scales its logits.  The padded output channels
+ * come out zero, so a residual stream stays padded.  Same arguments, workspace
+ * sizes and error codes as the un-suffixed entry points otherwise; with
+ * valid_channels = 128 the results are the same bits.
+ */
+int af3_triangle_multiplication_forward_padded(
+    const void* act, int io_dtype, const float* mask, int equation_flag,
+    const float* left_norm_input_weight, const float* left_norm_input_bias,
+    const uint16_t* w_proj_gate,
+    const float* center_norm_weight, const float* center_norm_bias,
+    const uint16_t* w_output_projection, const uint16_t* w_gating_linear,
+    void* out, int residual, int64_t n_token, int valid_channels,
+    void* workspace, size_t workspace_bytes, af3_stream_t stream);
+int af3_grid_self_attn_forward_padded(
+    const void* pair, int io_dtype, const float* mask, int transpose,
+    const float* act_norm_weight, const float* act_norm_bias,
+    const uint16_t* w_pair_bias, const float* nonbatched_bias,
+    const uint16_t* w_qkvg, const uint16_t* w_output, int num_head,
+    void* out, int residual, int64_t n_token, int valid_channels,
+    void* workspace, size_t workspace_bytes, af3_stream_t stream);
+int af3_transition_forward_padded(
+    const void* act, int io_dtype,
+    const float* layernorm_weight, const float* layernorm_bias,
+    const uint16_t* w1_packed, const uint16_t* w2, int hidden,
+    void* out, int residual, int64_t rows, int valid_channels, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Pair-biased gated self-attention without output projection.  Replaces
  *   torch.ops._alpha_attention.batch_diffusion_self_attention_forward
  *   (csrc/Alpha_Attention.cpp:72-92, schema :191-194; bodies
