@@ -241,6 +241,22 @@ def evoformer_block_ms(pkg, n, dev, rows=1024, iters=10):
             "outer_product_mean_tflops": round(flops_opm / ms_opm / 1e9, 1), "msa_attention_ms": round(ms_att, 3)}
 
 
+def template_block_ms(pkg, n, dev, iters=10):
+    """The Pairformer block of the template embedding (nn/d_template.py:198-201): 64 pair channels, transition
+    factor 2, no single track.  It runs on the 128-channel kernels over zero-padded operands."""
+    import torch
+    g = torch.Generator().manual_seed(5)
+    blk = random_init_(pkg.nn.PairformerBlock(c_pair=64, num_intermediate_factor=2, with_single=False), g).to(dev)
+    blk.load_hip_params()
+    pair = torch.randn(n, n, 64, generator=g).to(dev).bfloat16()
+    seq = (torch.arange(n) < int(0.9 * n)).float().to(dev)
+    pm = (seq[:, None] * seq[None, :]).contiguous()
+    ms = gpu_time_ms(lambda: blk(pair, pm), iters, warm_ms=40.0)
+    return {"workload": f"one Pairformer block on 64 pair channels (template embedding), N_token={n}, bf16, "
+                        "10% trailing tokens masked, padded to the 128-channel kernels",
+            "ms_per_block": round(ms, 3)}
+
+
 def trunk_recycle_ms(pkg, n, dev, rows=1024, iters=3):
     """One recycling pass of the Evoformer trunk: input embeddings, 4 Evoformer
     (MSA) blocks, 48 Pairformer blocks (no template embedding), bf16 streams."""
@@ -300,7 +316,8 @@ def main():
     ap.add_argument("--io", choices=["bf16", "f32"], default="bf16", help="dtype of the residual stream")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-trunk", action="store_true", help="skip the 48-block N=1536 trunk timing")
-    ap.add_argument("--no-diffusion", action="store_true", help="skip the diffusion-head and Evoformer-block timings")
+    ap.add_argument("--no-diffusion", action="store_true",
+                    help="skip the diffusion-head, Evoformer-block and 64-channel-block timings")
     ap.add_argument("--only", choices=["diffusion-head", "evoformer-block", "trunk-recycle"],
                     help="run that leg alone and print its object (for profiler runs)")
     ap.add_argument("--calibrate", action="store_true",
@@ -442,6 +459,7 @@ def main():
     if not args.no_diffusion:
         diffusion = diffusion_step(pkg, n, dev)
     evo = None if args.no_diffusion else evoformer_block_ms(pkg, n, dev)
+    template = None if args.no_diffusion else template_block_ms(pkg, n, dev)
 
     if args.calibrate:
         cx = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device=dev)   # 256 MiB in, 256 MiB out
@@ -481,6 +499,8 @@ def main():
         out["trunk_n1536"] = trunk
     if diffusion is not None:
         out["diffusion_head"] = diffusion
+    if template is not None:
+        out["template_block_c64"] = template
     if evo is not None:
         out["evoformer_block"] = evo
     if not args.no_cpu_baseline:
