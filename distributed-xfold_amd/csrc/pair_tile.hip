@@ -19,6 +19,8 @@
 // out^T[ch][px] with the weight rows as A (a lane owns one pixel and groups of
 // 4 consecutive channels).  D form feeds channel-major stores, T form feeds
 // pixel-major stores; the fragments are the same registers in both.
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 #include "tile_common.h"
@@ -30,11 +32,21 @@ namespace {
 // ============================================================================
 template <typename TIO>
 __global__ __launch_bounds__(256, 3) void trimul_prologue_kernel(TriMulArgs a) {
-  // 34.8 KB + 17.4 KB + 0.5 KB of LDS and at most 168 registers: three workgroups per CU.  The kernel is
-  // a chain of short dependent phases (load, LayerNorm, MFMA, stage, store), so what it needs is company.
-  __shared__ __attribute__((aligned(16))) bf16_t sX[TM * LDX];  // LN tile, then the [32 ch][px] staging tile
-  __shared__ __attribute__((aligned(16))) bf16_t sW[64 * LDX];  // 32 projection rows | the 32 matching gate rows
+  // 34.8 KB + 17.4 KB + 0.5 KB of LDS and at most 168 registers: three workgroups per CU.
+  //
+  // Eight steps of 64 weight rows (32 projection rows and the 32 matching gate rows) per tile.  A wave
+  // runs them as a software pipeline: the 16 MFMAs of step s are issued one by one with, behind each, the
+  // gating arithmetic (mask * proj * sigmoid(gate), packing, staging) of one register pair of step s - 1.
+  // Inside one wave the matrix unit works while the wave goes on issuing vector instructions; between
+  // waves of a SIMD it does not, so phases run back to back cost the sum of the two.  One barrier per step:
+  // the weights and the staged results are double-buffered.
+  __shared__ __attribute__((aligned(16))) bf16_t sX[TM * LDX];  // LN tile; then [S0 | S1 | W odd steps]
+  __shared__ __attribute__((aligned(16))) bf16_t sW0[64 * LDX];  // weights of the even steps
   __shared__ float sMask[TM];
+  static_assert(2 * 32 * LDX + 64 * LDX <= TM * LDX, "staging buffers and the second weight buffer fit the LN tile");
+  bf16_t* const sS0 = sX;
+  bf16_t* const sS1 = sX + 32 * LDX;
+  bf16_t* const sW1 = sX + 64 * LDX;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // outgoing: tiles run along k for fixed i (a[c][i][k]); incoming: along k for
   // fixed j, i.e. a column segment of the pair tensor (a'[c][j][k] = a[k][j][c]).
@@ -53,11 +65,11 @@ __global__ __launch_bounds__(256, 3) void trimul_prologue_kernel(TriMulArgs a) {
       wr[i] = *reinterpret_cast<const u32x4*>(base + ((row & 31) + (row >> 5) * 64) * C + (idx & 15) * 8);
     }
   };
-  auto wstore = [&]() {
+  auto wstore = [&](bf16_t* dst) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int idx = tid + 256 * i;
-      *reinterpret_cast<u32x4*>(sW + (idx >> 4) * LDX + (idx & 15) * 8) = wr[i];
+      *reinterpret_cast<u32x4*>(dst + (idx >> 4) * LDX + (idx & 15) * 8) = wr[i];
     }
   };
   const float mk = tid < TM && t.valid(tid) ? (a.mask ? a.mask[t.pix(tid)] : 1.f) : 0.f;
@@ -72,51 +84,132 @@ __global__ __launch_bounds__(256, 3) void trimul_prologue_kernel(TriMulArgs a) {
     }
     return;
   }
+#ifdef AF3_PROF
+  long long stamps[14];
+  int n_stamp = 0;
+#define PSTAMP() do { stamps[n_stamp++] = __builtin_readcyclecounter(); } while (0)
+#else
+#define PSTAMP() do {} while (0)
+#endif
+  PSTAMP();
   wload(0);
   if (tid < TM) sMask[tid] = mk;
   load_ln_tile<TIO>(x, t, a.ln_in_w, a.ln_in_b, sX, tid, false, a.lw.inv_c, a.lw.pad);
-  wstore();
+  PSTAMP();
+  wstore(sW0);
+  wload(1);
   lds_barrier();
+  PSTAMP();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
   lds_barrier();  // sX is free from here on
+  wstore(sW1);    // W_1
+  wload(2);
 
-#pragma unroll 1
-  for (int s = 0; s < 8; ++s) {
-    // request the next weights before this step's stores go out (vector
-    // memory operations retire in order)
-    if (s < 7) wload(s + 1);
-    f32x16 acc[2];
-    mfma_chunk<false, 2>(xf, sW, lane, acc);
-    // D form: lane owns channel (lane & 31) of tile 0 (P) and tile 1 (G)
-    {
-      const int ch = lane & 31;
+  f32x16 zero16;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int p0 = wave * 32 + 8 * g + 4 * (lane >> 5);
-        float v[4];
+  for (int r = 0; r < 16; ++r) zero16[r] = 0.f;
+  f32x16 accA[2], accB[2];  // [0] projection, [1] gate; A: even steps, B: odd steps
+  const int ch = lane & 31;
+
+  // Step S (0..8): the MFMAs of step S (S < 8) into `cur`, the gating of step S - 1 (S > 0) out of `prev`.
+  auto step = [&](auto step_c, f32x16* cur, f32x16* prev) {
+    constexpr int S = decltype(step_c)::value;
+    const bf16_t* w = (S & 1) ? sW1 : sW0;                    // W_S
+    bf16_t* stage = ((S - 1) & 1) ? sS1 : sS0;                // staging of step S - 1
+    // results of step S - 2, complete since the last barrier: 32 channels x 128 positions, two 16-byte
+    // pieces per thread, requested from LDS now and sent out further down
+    u32x4 outv[2];
+    if (S >= 2) {
+      const bf16_t* done = ((S - 2) & 1) ? sS1 : sS0;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc[0][4 * g + e] * sMask[p0 + e] * sigmoidf_(acc[1][4 * g + e]);
-        u32x2 pk;
-        pk.x = pack2bf(v[0], v[1]);
-        pk.y = pack2bf(v[2], v[3]);
-        *reinterpret_cast<u32x2*>(sX + ch * LDX + p0) = pk;
+      for (int i = 0; i < 2; ++i) {
+        const int idx = tid + 256 * i;
+        outv[i] = *reinterpret_cast<const u32x4*>(done + (idx >> 4) * LDX + (idx & 15) * 8);
       }
     }
-    lds_barrier();  // staging visible; every wave is done with sW
-    if (s < 7) wstore();
-    // 32 channels x 128 positions: two 16-byte pieces per thread
-    bf16_t* dst = (s < 4 ? a.a_buf : a.b_buf) + ((int64_t)(((s >> 1) & 1) * 64 + (s & 1) * 32) * a.N + t.o) * a.Np;
+    bf16x8 wf[3];  // weight fragments, read two MFMAs ahead
+    auto frag = [&](int m) { return lds_frag(w, LDX, (m & 1) * 32, (m >> 1) * 16, lane); };  // MFMA m: k-step m / 2, tile m % 2
+    if (S < 8) {
+      wf[0] = frag(0);
+      wf[1] = frag(1);
+    }
+    f32x4 m4 = {0.f, 0.f, 0.f, 0.f};
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int idx = tid + 256 * i, ch = idx >> 4, pc = idx & 15;
-      const int r = t.r0 + pc * 8;
-      if (r < a.Np)
-        *reinterpret_cast<u32x4*>(dst + (int64_t)ch * a.N * a.Np + r) =
-            *reinterpret_cast<const u32x4*>(sX + ch * LDX + pc * 8);
+    for (int m = 0; m < 16; ++m) {
+      if (S > 0 && (m & 3) == 0)  // the masks of pixels p0 .. p0 + 3, p0 = wave * 32 + 8 (m >> 2) + 4 hh
+        m4 = *reinterpret_cast<const f32x4*>(sMask + wave * 32 + 2 * m + 4 * (lane >> 5));
+      if (S < 8) {
+        if (m + 2 < 16) wf[(m + 2) % 3] = frag(m + 2);
+        cur[m & 1] = mfma32(xf[m >> 1], wf[m % 3], m < 2 ? zero16 : cur[m & 1]);
+      }
+      if (S > 0) {
+        // register m of the previous step: pixel p0 + (m & 3), p0 = wave * 32 + 8 (m >> 2) + 4 hh
+        float v = prev[0][m] * m4[m & 3] * sigmoidf_(prev[1][m]);
+        asm volatile("" : "+v"(v));  // keeps the arithmetic in this group
+        prev[0][m] = v;
+        if ((m & 3) == 3) {
+          const int g = m >> 2;
+          const int p0 = wave * 32 + 8 * g + 4 * (lane >> 5);
+          u32x2 pk;
+          pk.x = pack2bf(prev[0][4 * g], prev[0][4 * g + 1]);
+          pk.y = pack2bf(prev[0][4 * g + 2], prev[0][4 * g + 3]);
+          *reinterpret_cast<u32x2*>(stage + ch * LDX + p0) = pk;
+        }
+      }
+      if (m == 7) {
+        // half way: the next weights go to LDS (the buffer of step S + 1 was last read in step S - 1), the
+        // ones after them are requested, and step S - 2's results leave
+        if (S >= 1 && S + 1 < 8) {
+          wstore((S + 1) & 1 ? sW1 : sW0);
+          if (S + 2 < 8) wload(S + 2);
+        }
+        if (S >= 2) {
+          constexpr int SO = S >= 2 ? S - 2 : 0;
+          bf16_t* dst = (SO < 4 ? a.a_buf : a.b_buf) + ((int64_t)(((SO >> 1) & 1) * 64 + (SO & 1) * 32) * a.N + t.o) * a.Np;
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const int idx = tid + 256 * i, c2 = idx >> 4, pc = idx & 15;
+            const int r = t.r0 + pc * 8;
+            if (r < a.Np) *reinterpret_cast<u32x4*>(dst + (int64_t)c2 * a.N * a.Np + r) = outv[i];
+          }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
     lds_barrier();
+    PSTAMP();
+  };
+  PSTAMP();
+  step(std::integral_constant<int, 0>{}, accA, accB);
+  step(std::integral_constant<int, 1>{}, accB, accA);
+  step(std::integral_constant<int, 2>{}, accA, accB);
+  step(std::integral_constant<int, 3>{}, accB, accA);
+  step(std::integral_constant<int, 4>{}, accA, accB);
+  step(std::integral_constant<int, 5>{}, accB, accA);
+  step(std::integral_constant<int, 6>{}, accA, accB);
+  step(std::integral_constant<int, 7>{}, accB, accA);
+  step(std::integral_constant<int, 8>{}, accA, accB);  // gating of step 7, results of step 6
+  {
+    // results of step 7
+    bf16_t* dst = a.b_buf + ((int64_t)(64 + 32) * a.N + t.o) * a.Np;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int idx = tid + 256 * i, c2 = idx >> 4, pc = idx & 15;
+      const int r = t.r0 + pc * 8;
+      if (r < a.Np)
+        *reinterpret_cast<u32x4*>(dst + (int64_t)c2 * a.N * a.Np + r) =
+            *reinterpret_cast<const u32x4*>(sS1 + c2 * LDX + pc * 8);
+    }
   }
+#ifdef AF3_PROF
+  PSTAMP();
+  if (tid == 0) {
+    long long* dst = reinterpret_cast<long long*>(a.a_buf + ((int64_t)0 * a.N + t.o) * a.Np + t.r0);
+    for (int i = 0; i < 14; ++i) dst[i] = stamps[i];
+  }
+#endif
 }
 
 // ============================================================================

@@ -56,16 +56,28 @@ __device__ __forceinline__ void load_param8(const float* p, float fill, float* o
 // unconditional (an out-of-range pixel re-reads the tile's first one) and all
 // issued before any value is converted: a load under a lane mask, or one whose
 // value is touched at once, costs a full memory round trip per pixel.
+//
+// This phase is vector arithmetic per element and a large share of every tile
+// kernel's instructions, so the bf16 stream takes the short form: sum and sum of
+// squares in one pass (variance = E[x^2] - mean^2 in fp32: the error relative to
+// the variance is 1e-7 (1 + mean^2 / variance), and a bf16 tensor cannot hold a
+// mean of more than ~2^8 standard deviations to begin with), normalisation as two
+// FMAs per element (x * rstd - mean * rstd, then * w + b), and no per-element
+// select when every pixel of the tile is in range.  The fp32 stream keeps the
+// two-pass form.  Zero-padded channels (fewer than 128 real ones) add nothing to
+// either sum; the two-pass form takes their pad * mean^2 out again.
 template <typename TIO>
 __device__ __forceinline__ void load_ln_tile(const TIO* x, const Tile& t, const float* lnw,
                                              const float* lnb, bf16_t* sX, int tid, bool skip_ln = false,
                                              float inv_c = 1.f / C, float pad = 0.f) {
   using E = Elem<TIO>;
   constexpr int NB = E::kBatch;
+  constexpr bool ONE_PASS = sizeof(TIO) == 2;
   const int chunk = tid & 15, prow = tid >> 4;
   float w[8], b[8];
   load_param8(lnw ? lnw + chunk * 8 : nullptr, 1.f, w);
   load_param8(lnb ? lnb + chunk * 8 : nullptr, 0.f, b);
+  const bool full = t.r0 + TM <= t.N;  // every pixel of the tile is in range (uniform over the workgroup)
 #pragma unroll
   for (int base = 0; base < 8; base += NB) {
     typename E::Raw raw[NB];
@@ -77,22 +89,35 @@ __device__ __forceinline__ void load_ln_tile(const TIO* x, const Tile& t, const 
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
       const int p = (base + i) * 16 + prow;
-      float v[8];
+      float v[8], o[8];
       E::unpack_raw(raw[i], v);
-      float s = 0.f;
+      if (ONE_PASS) {
+        float s = 0.f, q = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) s += v[e];
-      const float mean = group16_sum(s) * inv_c;
-      float q = 0.f;
+        for (int e = 0; e < 8; ++e) { s += v[e]; q = fmaf(v[e], v[e], q); }
+        const float mean = group16_sum(s) * inv_c;
+        const float var = fmaxf(fmaf(group16_sum(q), inv_c, -mean * mean), 0.f);
+        // (an already normalised input comes with w = 1, b = 0: scale 1 and shift 0 pass it through unchanged)
+        const float rstd = skip_ln ? 1.f : rsqrtf(var + LN_EPS);
+        const float shift = skip_ln ? 0.f : -mean * rstd;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) { const float d = v[e] - mean; q += d * d; }
-      // (zero-padded channels, if any, each put mean^2 into the sum)
-      const float rstd = rsqrtf((group16_sum(q) - pad * mean * mean) * inv_c + LN_EPS);
-      float o[8];
-      const bool ok = t.valid(p);
+        for (int e = 0; e < 8; ++e) o[e] = fmaf(fmaf(v[e], rstd, shift), w[e], b[e]);
+      } else {
+        float s = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] = ok ? (skip_ln ? v[e] : (v[e] - mean) * rstd * w[e] + b[e]) : 0.f;
-      *reinterpret_cast<u32x4*>(sX + p * LDX + chunk * 8) = pack8(o);
+        for (int e = 0; e < 8; ++e) s += v[e];
+        const float mean = group16_sum(s) * inv_c;
+        float q = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { const float d = v[e] - mean; q += d * d; }
+        // (zero-padded channels, if any, each put mean^2 into the sum)
+        const float rstd = rsqrtf((group16_sum(q) - pad * mean * mean) * inv_c + LN_EPS);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = skip_ln ? v[e] : (v[e] - mean) * rstd * w[e] + b[e];
+      }
+      u32x4 pk = pack8(o);
+      if (!full && !t.valid(p)) pk = u32x4{0u, 0u, 0u, 0u};
+      *reinterpret_cast<u32x4*>(sX + p * LDX + chunk * 8) = pk;
     }
   }
 }
