@@ -439,128 +439,190 @@ __global__ __launch_bounds__(256) void attn_out_kernel(AttnOutArgs a) {
 // ============================================================================
 // SwiGLU transition, c = 128, hidden = 128 * factor, all in one kernel
 // ============================================================================
-constexpr int LDW2 = 68;  // LDS row stride (bf16) of a [128 out][64 hidden] W2 slab: 136 B = 34 dwords, so
-                          // the 32 rows of an 8-byte fragment read fall on 32 different bank pairs
+// Weight slabs go from global memory straight into LDS (global_load_lds_dwordx4: no staging
+// registers, no LDS stores in the instruction stream).  Such a load puts lane l's 16 bytes at
+// base + 16 l, so rows cannot be padded; their 16-byte chunks are XOR-permuted instead, on the
+// global side, where a lane is free to fetch any chunk.
+template <int OFF>
+__device__ __forceinline__ void lds_dma16(const char* gbase, uint32_t voff, const char* dst) {
+  const uint32_t lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)dst;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
+               :: "s"(lds), "v"(voff), "s"(gbase), "n"(OFF) : "memory");
+}
+// workgroup barrier that also waits for this wave's loads into LDS
+__device__ __forceinline__ void dma_lds_barrier() {
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+constexpr int W1_SLAB = 64 * 256;  // 32 "a" rows + 32 "b" rows of 128 bf16: 16 KB
+constexpr int W2_SLAB = 128 * 64;  // 128 output rows x 32 hidden units: 8 KB
 
 template <typename TIO>
 __global__ __launch_bounds__(256, 2) void transition_kernel(TransitionArgs a) {
-  __shared__ __attribute__((aligned(16))) bf16_t smem[2 * TM * LDX];
-  bf16_t* sX = smem;              // phase 0: LN tile;   later: W1 slab [128][LDX]
-  bf16_t* sW1 = smem;
-  bf16_t* sW2 = smem + TM * LDX;  // W2 slab [128][LDW2]
+  // The hidden layer is walked in slabs of 32 units.  Per slab a wave issues 16 MFMAs of GEMM1 (T form:
+  // a^T and b^T, 32 hidden x 32 pixels each), 32 SiLU-gate evaluations per lane pair of registers and 8
+  // MFMAs of GEMM2 into the four output tiles; h^T = silu(a) * b in registers 8s..8s+7 is, as it stands,
+  // the B fragment of k-step s of GEMM2 when row rho of the slab holds hidden unit swap23(rho) (bits 2
+  // and 3 exchanged): the lane-half's eight registers are then eight consecutive units, one 16-byte
+  // fragment of W2's natural order.
+  //
+  // The slabs run as a software pipeline inside each wave: the MFMAs of GEMM1 of slab h are issued one by
+  // one with the gating of slab h - 1 between them, and the MFMAs of GEMM2 of slab h - 1 follow as their
+  // fragments become complete.  Phases run back to back would cost the sum of the matrix unit's and the
+  // vector unit's time (the two do not overlap between the waves of a SIMD).  W1 slabs are double-
+  // buffered, W2 slabs triple-buffered (a W2 slab is used one iteration after its W1 slab); one barrier
+  // per slab.
+  __shared__ __attribute__((aligned(1024))) char smem[2 * TM * LDX * 2];  // 69.6 KB
+  // layout: [0, 34816) LN tile, later W1 buffer 1 (16 KB) and W2 buffers 1, 2 (8 KB each);
+  //         [34816, 34816 + 24 KB) W1 buffer 0 and W2 buffer 0, loaded while the LN tile is being made
+  static_assert(TM * LDX * 2 >= W1_SLAB + 2 * W2_SLAB, "buffers 1, 2 fit the LN tile");
+  static_assert(TM * LDX * 2 + W1_SLAB + W2_SLAB <= (int)sizeof(smem), "buffers 0 fit behind it");
+  static_assert(TM * LDS_F * 4 <= (int)sizeof(smem), "staging tile must fit");
+  bf16_t* sX = reinterpret_cast<bf16_t*>(smem);
   float* sS = reinterpret_cast<float*>(smem);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  char* const w1buf0 = smem + TM * LDX * 2;
+  char* const w1buf1 = smem;
+  char* const w2buf0 = smem + TM * LDX * 2 + W1_SLAB;
+  char* const w2buf1 = smem + W1_SLAB;
+  char* const w2buf2 = smem + W1_SLAB + W2_SLAB;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int j = lane & 31, hh = lane >> 5;
   const Tile t = make_tile(a.N, false);
   const TIO* x = reinterpret_cast<const TIO*>(a.x);
+  const int n_slabs = a.hidden / 32;
+
+  // ---- loads into LDS: per-lane global offsets, wave-uniform LDS destinations ----
+  // W1 slab h: rows of the host-packed [hidden/64][64 a | 64 b][128] array; LDS row rho (0..31 a, 32..63 b)
+  // holds unit swap23(rho % 32); chunk c of a row at position c ^ (rho & 15).  Load i of 4 covers rows
+  // 16 i + lane / 16 (of this wave's quarter: rows 16 i + 4 wave + ...), one 16-byte chunk per lane.
+  const char* w1g = reinterpret_cast<const char*>(a.w1);
+  const char* w2g = reinterpret_cast<const char*>(a.w2);
+  uint32_t w1off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int rho = 16 * i + 4 * wave + (lane >> 4);              // 0..63
+    const int u = rho & 31;
+    const int unit = (u & ~12) | ((u & 4) << 1) | ((u & 8) >> 1);  // swap23
+    const int chunk = (lane & 15) ^ (rho & 15);
+    w1off[i] = (uint32_t)((((rho >> 5) * 64 + unit) * C + chunk * 8) * 2);  // + slab base (below)
+  }
+  // W2 slab h: rows o = 0..127 of w2[128][hidden], columns 32 h .. + 31 (four 16-byte chunks); chunk c of
+  // row o at position c ^ ((o >> 2) & 3).  Load i of 2 covers rows 64 i + 16 wave + lane / 4.
+  uint32_t w2off[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int o = 64 * i + 16 * wave + (lane >> 2);
+    const int chunk = (lane & 3) ^ ((o >> 2) & 3);
+    w2off[i] = (uint32_t)((o * a.hidden + chunk * 8) * 2);
+  }
+  auto load_slab = [&](int h, char* w1dst, char* w2dst) {
+    // slab h = half (h & 1) of the 64-unit block h / 2: a rows 32 (h & 1) .., b rows 64 + 32 (h & 1) ..
+    const uint32_t base1 = (uint32_t)(((h >> 1) * 128 + (h & 1) * 32) * C * 2);
+    const uint32_t base2 = (uint32_t)(h * 32 * 2);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lds_dma16<0>(w1g, w1off[i] + base1, w1dst + (16 * i + 4 * wave) * 256);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) lds_dma16<0>(w2g, w2off[i] + base2, w2dst + (64 * i + 16 * wave) * 64);
+  };
+  load_slab(0, w1buf0, w2buf0);
+
   load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, false, a.lw.inv_c, a.lw.pad);
   lds_barrier();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
-  lds_barrier();
+  dma_lds_barrier();  // sX is free from here on; slab 0 has landed
+  if (n_slabs > 1) load_slab(1, w1buf1, w2buf1);
 
-  f32x16 out[4];
+  f32x16 out[4], zero16;
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt)
+  for (int r = 0; r < 16; ++r) zero16[r] = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) out[nt][r] = 0.f;
+  for (int nt = 0; nt < 4; ++nt) out[nt] = zero16;
 
-  const int n_slabs = a.hidden / 64;
-  // Slab hs of W1 (64 "a" rows then the 64 matching "b" rows, host-packed, K = 128)
-  // and of W2 (all 128 output rows, hidden columns 64 hs .. +63) are fetched
-  // into registers one slab ahead, so their latency hides behind the MFMAs.
-  WChunkRegs w1r;
-  u32x4 w2r[4];
-  auto fetch = [&](int hs) {
-    w1r.load(a.w1 + (int64_t)hs * 128 * C, tid);
+  // fragment addresses: W1 row (32 tile + j), chunk 2 ks + hh; W2 row (32 ot + j), chunk 2 s + hh
+  const int w1frag = j * 256, w1sw = j & 15;
+  const int w2frag = j * 64, w2sw = (j >> 2) & 3;
+  auto w1_frag = [&](const char* buf, int tile, int ks) {
+    return as_frag(*reinterpret_cast<const u32x4*>(buf + tile * (32 * 256) + w1frag + (((2 * ks + hh) ^ w1sw) << 4)));
+  };
+  auto w2_frag = [&](const char* buf, int ot, int s) {
+    return as_frag(*reinterpret_cast<const u32x4*>(buf + ot * (32 * 64) + w2frag + (((2 * s + hh) ^ w2sw) << 4)));
+  };
+
+  f32x16 abA[2], abB[2];  // [0] a^T, [1] b^T of a slab; A: even slabs, B: odd slabs
+  // One iteration: GEMM1 of slab h into `cur` (h < n_slabs) out of W1 buffer `w1`; gating of slab h - 1 out
+  // of `prev` and its GEMM2 out of W2 buffer `w2p` (h > 0).
+  auto iteration = [&](auto g1_c, auto g2_c, const char* w1, const char* w2p, f32x16* cur, f32x16* prev) {
+    constexpr bool gemm1 = decltype(g1_c)::value, gemm2 = decltype(g2_c)::value;
+    bf16x8 wf[3];
+    if (gemm1) {
+      wf[0] = w1_frag(w1, 0, 0);
+      wf[1] = w1_frag(w1, 1, 0);
+    }
+    bf16x8 w2f[4];
+    u32x4 hfrag[2];
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int idx = tid + 256 * i;
-      w2r[i] = *reinterpret_cast<const u32x4*>(a.w2 + (int64_t)(idx >> 3) * a.hidden + hs * 64 + (idx & 7) * 8);
+    for (int m = 0; m < 16; ++m) {
+      // MFMA m of GEMM1: k-step m / 2, tile m % 2 (a, b)
+      if (gemm1) {
+        if (m + 2 < 16) wf[(m + 2) % 3] = w1_frag(w1, (m + 2) & 1, (m + 2) >> 1);
+        cur[m & 1] = mfma32(wf[m % 3], xf[m >> 1], m < 2 ? zero16 : cur[m & 1]);
+      }
+      if (gemm2) {
+        // register m of the previous slab: h = silu(a) * b
+        const float av = prev[0][m], bv = prev[1][m];
+        float hv = av * sigmoidf_(av) * bv;
+        asm volatile("" : "+v"(hv));  // keeps the arithmetic in this group
+        prev[0][m] = hv;
+        if (m == 3 || m == 12) {
+          // the W2 fragments of k-step 0 (used behind groups 8..11) and, once those are through, of k-step 1
+#pragma unroll
+          for (int ot = 0; ot < 4; ++ot) w2f[ot] = w2_frag(w2p, ot, m == 3 ? 0 : 1);
+        }
+        if ((m & 7) == 7) {
+          const int s8 = m & 8;
+          float f8[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) f8[e] = prev[0][s8 + e];
+          hfrag[m >> 3] = pack8(f8);
+        }
+        // GEMM2 of k-step 0 behind groups 8..11
+        if (m >= 8 && m < 12) out[m - 8] = mfma32(w2f[m - 8], as_frag(hfrag[0]), out[m - 8]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (gemm2) {
+      // (k-step 0's fragments were consumed behind groups 8..11; k-step 1's were read in group 12)
+#pragma unroll
+      for (int ot = 0; ot < 4; ++ot) out[ot] = mfma32(w2f[ot], as_frag(hfrag[1]), out[ot]);
     }
   };
-  auto commit = [&]() {
-    w1r.store(sW1, tid);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int idx = tid + 256 * i;
-      // rows are 8-byte aligned only: two 8-byte stores
-      u32x2* dst = reinterpret_cast<u32x2*>(sW2 + (idx >> 3) * LDW2 + (idx & 7) * 8);
-      dst[0] = u32x2{w2r[i].x, w2r[i].y};
-      dst[1] = u32x2{w2r[i].z, w2r[i].w};
-    }
-  };
-  fetch(0);
-  commit();
-  lds_barrier();
+
+  // slab h: W1 buffer h % 2, W2 buffer h % 3; the loads of slab h + 1 are issued at the top of iteration h
+  // (its W1 buffer was last read in iteration h - 1, its W2 buffer in iteration h - 1 as slab h - 2's)
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+  auto w2buf = [&](int h) -> char* { return h % 3 == 0 ? w2buf0 : (h % 3 == 1 ? w2buf1 : w2buf2); };
+  // slab 0: GEMM1 only
+  iteration(T_{}, F_{}, w1buf0, w2buf0, abA, abB);
+  dma_lds_barrier();
 #pragma unroll 1
-  for (int hs = 0; hs < n_slabs; ++hs) {
-    if (hs + 1 < n_slabs) fetch(hs + 1);
-    // GEMM1, T form, one 32-unit half of the slab at a time (32 live
-    // accumulators instead of 64): ab[0] = a^T (32 hidden x 32 px), ab[1] = b^T.
-    // h^T = silu(a) * b; registers 8s..8s+7 are, as they stand, the B fragment of
-    // k-step s of GEMM2 provided W2's k index is permuted alike: element e of
-    // lane-half hh is hidden unit 32*nt + 16*s + 8*(e >> 2) + 4*hh + (e & 3).
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-      f32x16 ab[2];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) ab[0][r] = ab[1][r] = 0.f;
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        ab[0] = mfma32(lds_frag(sW1, LDX, nt * 32, ks * 16, lane), xf[ks], ab[0]);
-        ab[1] = mfma32(lds_frag(sW1, LDX, 64 + nt * 32, ks * 16, lane), xf[ks], ab[1]);
-      }
-      // fragment reads four ahead of the MFMAs that use them (left to itself the
-      // compiler reads each one right in front of its MFMA and waits for it)
-      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-      for (int i = 0; i < 12; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      // GEMM2: the W2 fragments of a step are requested before its silu, not
-      // in front of each MFMA
-      auto w2_frags = [&](int s, u32x4* wv) {
-        const int kbase = 32 * nt + 16 * s + 4 * (lane >> 5);
-#pragma unroll
-        for (int ot = 0; ot < 4; ++ot) {
-          const bf16_t* wp = sW2 + (ot * 32 + (lane & 31)) * LDW2 + kbase;
-          const u32x2 lo = *reinterpret_cast<const u32x2*>(wp);
-          const u32x2 hi = *reinterpret_cast<const u32x2*>(wp + 8);
-          wv[ot].x = lo.x; wv[ot].y = lo.y; wv[ot].z = hi.x; wv[ot].w = hi.y;
-        }
-      };
-      auto silu_frag = [&](int s) {
-        float hv[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float av = ab[0][8 * s + e], bv = ab[1][8 * s + e];
-          hv[e] = av * sigmoidf_(av) * bv;
-        }
-        return as_frag(pack8(hv));
-      };
-      u32x4 wv0[4], wv1[4];
-      w2_frags(0, wv0);
-      __builtin_amdgcn_sched_barrier(0);
-      const bf16x8 hf0 = silu_frag(0);
-      __builtin_amdgcn_sched_barrier(0);
-      w2_frags(1, wv1);
-#pragma unroll
-      for (int ot = 0; ot < 4; ++ot) out[ot] = mfma32(as_frag(wv0[ot]), hf0, out[ot]);
-      const bf16x8 hf1 = silu_frag(1);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int ot = 0; ot < 4; ++ot) out[ot] = mfma32(as_frag(wv1[ot]), hf1, out[ot]);
-    }
-    lds_barrier();  // every wave is done with this slab
-    if (hs + 1 < n_slabs) {
-      commit();
-      lds_barrier();
+  for (int h = 1; h < n_slabs; h += 2) {
+    // odd slab h, then even slab h + 1 (n_slabs is even: the last odd slab has no successor)
+    if (h + 1 < n_slabs) load_slab(h + 1, w1buf0, w2buf(h + 1));
+    iteration(T_{}, T_{}, w1buf1, w2buf(h - 1), abB, abA);
+    dma_lds_barrier();
+    if (h + 1 < n_slabs) {
+      if (h + 2 < n_slabs) load_slab(h + 2, w1buf1, w2buf(h + 2));
+      iteration(T_{}, T_{}, w1buf0, w2buf(h), abA, abB);
+      dma_lds_barrier();
     }
   }
+  // gating and GEMM2 of the last slab (odd: in abB)
+  iteration(F_{}, T_{}, w1buf0, w2buf(n_slabs - 1), abA, abB);
+  dma_lds_barrier();
   stage_t_f32(out, sS, wave, lane);
   lds_barrier();
   store_tile_f32<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), a.residual ? x : nullptr, tid);
