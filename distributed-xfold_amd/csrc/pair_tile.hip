@@ -553,18 +553,22 @@ __global__ __launch_bounds__(256, 2) void transition_kernel(TransitionArgs a) {
   f32x16 abA[2], abB[2];  // [0] a^T, [1] b^T of a slab; A: even slabs, B: odd slabs
   // One iteration: GEMM1 of slab h into `cur` (h < n_slabs) out of W1 buffer `w1`; gating of slab h - 1 out
   // of `prev` and its GEMM2 out of W2 buffer `w2p` (h > 0).
-  auto iteration = [&](auto g1_c, auto g2_c, const char* w1, const char* w2p, f32x16* cur, f32x16* prev) {
-    constexpr bool gemm1 = decltype(g1_c)::value, gemm2 = decltype(g2_c)::value;
+  // (the second k-step of a slab's GEMM2 is issued behind the first groups of the NEXT iteration: its
+  // fragments are complete only when the last group of this one is through)
+  bf16x8 w2f[4];
+  u32x4 hfrag[2];
+  auto iteration = [&](auto g1_c, auto g2_c, auto carry_c, const char* w1, const char* w2p, f32x16* cur, f32x16* prev) {
+    constexpr bool gemm1 = decltype(g1_c)::value, gemm2 = decltype(g2_c)::value, carry = decltype(carry_c)::value;
     bf16x8 wf[3];
     if (gemm1) {
       wf[0] = w1_frag(w1, 0, 0);
       wf[1] = w1_frag(w1, 1, 0);
     }
-    bf16x8 w2f[4];
-    u32x4 hfrag[2];
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < 16; ++m) {
+      // GEMM2, k-step 1 of the slab gated in the previous iteration
+      if (carry && m < 4) out[m] = mfma32(w2f[m], as_frag(hfrag[1]), out[m]);
       // MFMA m of GEMM1: k-step m / 2, tile m % 2 (a, b)
       if (gemm1) {
         if (m + 2 < 16) wf[(m + 2) % 3] = w1_frag(w1, (m + 2) & 1, (m + 2) >> 1);
@@ -593,11 +597,6 @@ __global__ __launch_bounds__(256, 2) void transition_kernel(TransitionArgs a) {
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (gemm2) {
-      // (k-step 0's fragments were consumed behind groups 8..11; k-step 1's were read in group 12)
-#pragma unroll
-      for (int ot = 0; ot < 4; ++ot) out[ot] = mfma32(w2f[ot], as_frag(hfrag[1]), out[ot]);
-    }
   };
 
   // slab h: W1 buffer h % 2, W2 buffer h % 3; the loads of slab h + 1 are issued at the top of iteration h
@@ -606,22 +605,26 @@ __global__ __launch_bounds__(256, 2) void transition_kernel(TransitionArgs a) {
   using F_ = std::false_type;
   auto w2buf = [&](int h) -> char* { return h % 3 == 0 ? w2buf0 : (h % 3 == 1 ? w2buf1 : w2buf2); };
   // slab 0: GEMM1 only
-  iteration(T_{}, F_{}, w1buf0, w2buf0, abA, abB);
+  iteration(T_{}, F_{}, F_{}, w1buf0, w2buf0, abA, abB);
+  dma_lds_barrier();
+  // slab 1 (gating of slab 0: nothing carried over yet)
+  if (n_slabs > 2) load_slab(2, w1buf0, w2buf(2));
+  iteration(T_{}, T_{}, F_{}, w1buf1, w2buf(0), abB, abA);
   dma_lds_barrier();
 #pragma unroll 1
-  for (int h = 1; h < n_slabs; h += 2) {
-    // odd slab h, then even slab h + 1 (n_slabs is even: the last odd slab has no successor)
-    if (h + 1 < n_slabs) load_slab(h + 1, w1buf0, w2buf(h + 1));
-    iteration(T_{}, T_{}, w1buf1, w2buf(h - 1), abB, abA);
+  for (int h = 2; h < n_slabs; h += 2) {
+    // even slab h, then odd slab h + 1 (n_slabs is even)
+    load_slab(h + 1, w1buf1, w2buf(h + 1));
+    iteration(T_{}, T_{}, T_{}, w1buf0, w2buf(h - 1), abA, abB);
     dma_lds_barrier();
-    if (h + 1 < n_slabs) {
-      if (h + 2 < n_slabs) load_slab(h + 2, w1buf1, w2buf(h + 2));
-      iteration(T_{}, T_{}, w1buf0, w2buf(h), abA, abB);
-      dma_lds_barrier();
-    }
+    if (h + 2 < n_slabs) load_slab(h + 2, w1buf0, w2buf(h + 2));
+    iteration(T_{}, T_{}, T_{}, w1buf1, w2buf(h), abB, abA);
+    dma_lds_barrier();
   }
-  // gating and GEMM2 of the last slab (odd: in abB)
-  iteration(F_{}, T_{}, w1buf0, w2buf(n_slabs - 1), abA, abB);
+  // gating and GEMM2 of the last slab (odd: in abB), then its second k-step
+  iteration(F_{}, T_{}, T_{}, w1buf0, w2buf(n_slabs - 1), abA, abB);
+#pragma unroll
+  for (int ot = 0; ot < 4; ++ot) out[ot] = mfma32(w2f[ot], as_frag(hfrag[1]), out[ot]);
   dma_lds_barrier();
   stage_t_f32(out, sS, wave, lane);
   lds_barrier();
