@@ -3,7 +3,8 @@ kernel (at least 120 such tiles, in one round of the 256 CUs or more): plain / b
 regrouped store and the segmented q-k-v-gate projection of the diffusion
 self-attention, against float64 products of the same bf16 operands.  Ragged
 M (not a multiple of 256), N (a partial last tile) and K (not a multiple of
-the 32-deep slab) are part of every case."""
+the 32-deep slab) are part of every case; the cases of more than 256 tiles make
+some of the kernel's persistent workgroups walk on to a second tile."""
 
 import pytest
 import torch
@@ -60,10 +61,10 @@ def test_linear_swiglu(gpu_pkg, m, k, hidden):
     within_bf16_ulp("swiglu", h, torch.nn.functional.silu(y[:, :hidden]) * y[:, hidden:])
 
 
-def test_linear_regrouped_store(gpu_pkg):
-    print("test_linear_regrouped_store (large tile)", flush=True)
+@pytest.mark.parametrize("m,n,k", [(3872, 2720, 136), (6400, 3072, 40)])   # 176 tiles; 300: some workgroups take two
+def test_linear_regrouped_store(gpu_pkg, m, n, k):
+    print(f"test_linear_regrouped_store (large tile) m={m} n={n} k={k}", flush=True)
     g = gen(12)
-    m, n, k = 3872, 2720, 136
     x, w = O.round_bf16(torch.randn(m, k, generator=g)), O.round_bf16(torch.randn(n, k, generator=g) * 0.1)
     got = gpu_pkg.ops.linear(x.to(dev()).bfloat16(), w.to(dev()).bfloat16(), mode=gpu_pkg.lib.LINEAR_REGROUP32)
     y = x.double() @ w.double().T

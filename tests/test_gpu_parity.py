@@ -416,6 +416,28 @@ def test_kernel_level_contraction(gpu_pkg, n):
     assert_within_bf16_ulp("contraction", t[:, :, :n].cpu(), want.cpu(), ulps=1.01, atol=1e-3)
 
 
+@pytest.mark.parametrize("batch,m,n,k", [
+    (8, 2048, 1792, 16),      # less than one 32-deep slab of k, 448 tiles: several per workgroup
+    (3, 2300, 1100, 40),      # partial tiles on both edges and a k tail
+    (600, 130, 264, 72),      # many small products, one or two tiles each
+    (1, 8192, 4096, 64),      # one large product: the rectangle-per-XCD order, two tiles per workgroup
+    (2, 256, 256, 2048),      # two tiles in all: most workgroups have nothing to do
+])
+def test_kernel_level_batched_product_tile_walk(gpu_pkg, batch, m, n, k):
+    """The large-tile kernel's workgroups are persistent and run their slab pipeline across
+    tile boundaries (a tile's first slabs are fetched while the previous one finishes): shapes
+    where a workgroup gets several tiles, with short k, k tails and partial edge tiles."""
+    note(f"test_kernel_level_batched_product_tile_walk {batch} {m} {n} {k}")
+    g = gen(batch + m + n + k)
+    a = rb(torch.randn(batch, m, k, generator=g)).to(dev())
+    b = rb(torch.randn(batch, n, k, generator=g)).to(dev())
+    t = gpu_pkg.ops.batched_nt_product(a.bfloat16(), b.bfloat16())
+    step = max(1, (1 << 24) // (m * n))
+    for c0 in range(0, batch, step):                                 # float64 on the GPU, a few products at a time
+        want = torch.bmm(a[c0:c0 + step].double(), b[c0:c0 + step].double().transpose(1, 2))
+        assert_within_bf16_ulp("product", t[c0:c0 + step].cpu(), want.cpu(), ulps=1.01, atol=1e-3)
+
+
 def _attention_core_case(gpu_pkg, n, tiles, scale=0.7, bias_shift=0.0, seed=None, dense=False):
     g = gen(n + tiles if seed is None else seed)
     log2e = 1.4426950408889634
