@@ -178,23 +178,70 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
   if (tid < R * 5) sLive[tid] = 0u;
   if (tid == 0) sRedo = 0u;
   lds_barrier();
+  // A wave takes every fourth key tile; the mask values of eight of its tiles and all rows are
+  // requested together (one trip per 32 key tiles, not one per tile and row).  The mask is small
+  // and comes out of L2; Q and the output gates come from memory and are requested right behind
+  // the first batch of mask values: loads return in order, so the mask pass does not wait for
+  // them, and they travel while it, the barriers and the first tiles' loads are under way.
+  bf16x8 qf[R][2];
+  u32x2 gw[R][4];  // output gates: used at the very end
+  // What a wave finds out about its tiles stays in scalar registers (the ballots are uniform)
+  // and reaches the workgroup's words in LDS once, at the end.
+  uint64_t my_live[R], my_plain[R];
+  bool my_any[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const float* mrow = a.mask ? a.mask + (int64_t)brow[r] * N : nullptr;
-    for (int t0 = 0; t0 < nkt; t0 += 4) {
-      const int tile = t0 + wave;
-      if (tile < nkt) {
-        const int key = tile * KT + lane;
-        const float mv = mrow ? mrow[min(key, N - 1)] : 1.f;
-        const bool on = key < N && mv != 0.f;
-        sCode[r * nk64 + key] = (uint16_t)(key >= N ? BF16_NEG_INF : (mv == 0.f ? BF16_NEG_1E9 : 0u));
-        const uint64_t on_lanes = __ballot(on);
-        if (on_lanes != 0ull && lane == 0) {
-          if (tile < 64) atomicOr(&sLive[r * 5 + (tile >> 5)], 1u << (tile & 31));
-          atomicOr(&sLive[r * 5 + 2], 1u);
-          if (tile < 64 && on_lanes == ~0ull) atomicOr(&sLive[r * 5 + 3 + (tile >> 5)], 1u << (tile & 31));
+    my_live[r] = my_plain[r] = 0ull;
+    my_any[r] = false;
+  }
+  for (int t0 = 0; t0 < nkt; t0 += 32) {
+    float mv[R][8];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        mv[r][u] = a.mask ? a.mask[(int64_t)brow[r] * N + min((t0 + 4 * u + wave) * KT + lane, N - 1)] : 1.f;
+    if (t0 == 0) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int64_t row = ((int64_t)brow[r] * H + h) * N + qi;
+        const bf16_t* qp = a.q + row * D + 8 * hh;
+        qf[r][0] = as_frag(*reinterpret_cast<const u32x4*>(qp));
+        qf[r][1] = as_frag(*reinterpret_cast<const u32x4*>(qp + 16));
+        const bf16_t* gp = a.g + row * D + 4 * hh;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) gw[r][g] = *reinterpret_cast<const u32x2*>(gp + 8 * g);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int tile = t0 + 4 * u + wave;
+        if (tile < nkt) {
+          const int key = tile * KT + lane;
+          const bool on = key < N && mv[r][u] != 0.f;
+          sCode[r * nk64 + key] = (uint16_t)(key >= N ? BF16_NEG_INF : (mv[r][u] == 0.f ? BF16_NEG_1E9 : 0u));
+          const uint64_t on_lanes = __ballot(on);
+          my_any[r] = my_any[r] || on_lanes != 0ull;
+          if (tile < 64) {
+            my_live[r] |= (uint64_t)(on_lanes != 0ull) << tile;
+            my_plain[r] |= (uint64_t)(on_lanes == ~0ull) << tile;
+          }
         }
       }
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (!my_any[r]) continue;
+      atomicOr(&sLive[r * 5], (uint32_t)my_live[r]);
+      atomicOr(&sLive[r * 5 + 1], (uint32_t)(my_live[r] >> 32));
+      atomicOr(&sLive[r * 5 + 2], 1u);
+      atomicOr(&sLive[r * 5 + 3], (uint32_t)my_plain[r]);
+      atomicOr(&sLive[r * 5 + 4], (uint32_t)(my_plain[r] >> 32));
     }
   }
   lds_barrier();
@@ -235,16 +282,12 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
 
   if (!all_dead) {
     // ---- per-lane constants ----
-    bf16x8 qf[R][2];
     u32x4 qm[R];  // Q side of the mask k-step: slot 0 = 1.0 (times the key's code), slot 1 = -base
     const char* kglob[R];
     const char* vglob[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int64_t bh = (int64_t)brow[r] * H + h;
-      const bf16_t* qp = a.q + (bh * N + qi) * D + 8 * hh;
-      qf[r][0] = as_frag(*reinterpret_cast<const u32x4*>(qp));
-      qf[r][1] = as_frag(*reinterpret_cast<const u32x4*>(qp + 16));
       qm[r] = u32x4{hh == 0 ? (BF16_ONE | 0x80000000u) : 0u, 0u, 0u, 0u};  // -0.0 in slot 1
       kglob[r] = reinterpret_cast<const char*>(a.k + bh * N * D);
       vglob[r] = reinterpret_cast<const char*>(a.vt + bh * D * a.ldn);
@@ -498,6 +541,15 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
     int t_cur = pop(), t_n1 = pop(), t_n2 = pop();
     // the buffer the first virtual tile reads its "previous" V^T from must hold finite data
     *reinterpret_cast<u32x4*>(VBUF(1, R - 1) + tid * 16) = u32x4{0u, 0u, 0u, 0u};
+    // the first tiles' loads into LDS and the first bias tile's ordinary loads travel together
+    dma_bias(t_n1, sBias1);
+    dma_k(t_cur, 0, KBUF(0, 0));
+    if (R == 2) {
+      dma_k(t_cur, 1, KBUF(0, 1));
+      dma_k(t_n1, 0, KBUF(1, 0));
+      dma_v(t_cur, 0, VBUF(0, 0));
+      dma_v(t_cur, 1, VBUF(0, 1));
+    }
     if (HAS_BIAS) {
       const char* p = bbase + (size_t)t_cur * 4096u + (j * 32 + hh * 16);
       u32x4 f[4];
@@ -506,13 +558,7 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       bt[0] = mfma32_f16(idf[1], as_frag_f16(f[1]), mfma32_f16(idf[0], as_frag_f16(f[0]), zero16));
       bt[1] = mfma32_f16(idf[1], as_frag_f16(f[3]), mfma32_f16(idf[0], as_frag_f16(f[2]), zero16));
     }
-    dma_bias(t_n1, sBias1);
-    dma_k(t_cur, 0, KBUF(0, 0));
     if (R == 2) {
-      dma_k(t_cur, 1, KBUF(0, 1));
-      dma_k(t_n1, 0, KBUF(1, 0));
-      dma_v(t_cur, 0, VBUF(0, 0));
-      dma_v(t_cur, 1, VBUF(0, 1));
       dma_barrier();
       kpre[0] = lds16(KBUF(0, 0) + ka0);
       kpre[1] = lds16(KBUF(0, 0) + ka1);
@@ -627,17 +673,12 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
   for (int r = 0; r < R; ++r) {
     if (!bvalid[r]) continue;
     const float inv = 1.f / lrun[r];  // the sum over both half-waves' keys
-    const int64_t bh = (int64_t)brow[r] * H + h;
-    const bf16_t* gp = a.g + (bh * N + qw) * D + 4 * hh;
     bf16_t* op = a.og + ((int64_t)brow[r] * N + qw) * 128 + h * D + 4 * hh;
-    u32x2 gw[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) gw[g] = *reinterpret_cast<const u32x2*>(gp + 8 * g);
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       u32x2 w;
-      w.x = pack2bf(o[r][4 * g] * inv * bflo(gw[g].x), o[r][4 * g + 1] * inv * bfhi(gw[g].x));
-      w.y = pack2bf(o[r][4 * g + 2] * inv * bflo(gw[g].y), o[r][4 * g + 3] * inv * bfhi(gw[g].y));
+      w.x = pack2bf(o[r][4 * g] * inv * bflo(gw[r][g].x), o[r][4 * g + 1] * inv * bfhi(gw[r][g].x));
+      w.y = pack2bf(o[r][4 * g + 2] * inv * bflo(gw[r][g].y), o[r][4 * g + 3] * inv * bfhi(gw[r][g].y));
       *reinterpret_cast<u32x2*>(op + 8 * g) = w;
     }
   }
