@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from rocprofv3 counters (FETCH_SIZE x 2.000 +
 # WRITE_SIZE x 1.000, scaled by a plain elementwise kernel of known size in the same run, see
 # --calibrate); measured offline, per N_token: profiles/pairformer_block_n768_bf16_hbm_traffic.txt
-MEASURED_TRAFFIC_BYTES = {("triattn_flash_kernel", 768): 810.3e6, ("contract_kernel", 768): 508.6e6}
+MEASURED_TRAFFIC_BYTES = {("triattn_flash_kernel", 768): 839.9e6, ("contract_kernel", 768): 508.5e6}
 
 
 def flops_trimul(n):      # one direction
