@@ -135,7 +135,8 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
   __shared__ __attribute__((aligned(1024))) char sV11[R > 1 ? TILE_BYTES : 16];
   __shared__ __attribute__((aligned(1024))) char sBias0[HAS_BIAS ? 4 * 4096 : 16];  // a bias tile per wave, by key tile parity
   __shared__ __attribute__((aligned(1024))) char sBias1[HAS_BIAS ? 4 * 4096 : 16];
-  __shared__ uint32_t sLive[R * 5];  // per row: live tiles (2 words), any live key, wholly unmasked tiles (2 words)
+  __shared__ uint32_t sLive[R];      // per row: some key is unmasked
+  __shared__ uint8_t sFlag[R * 64];  // per row and key tile (the first 64): 1 = some key unmasked, 3 = all 64 of them
   __shared__ float sMean[D];
   __shared__ uint32_t sRedo;  // a wave's unmasked-tile shortcut went wrong: the workgroup repeats its rows without it
   extern __shared__ __attribute__((aligned(16))) uint16_t sCode[];  // [R][nkt * 64] mask code per key
@@ -175,7 +176,8 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
   }
 
   // ---- mask pass: per-key codes for the mask k-step, live key tiles, dead rows ----
-  if (tid < R * 5) sLive[tid] = 0u;
+  if (tid < R) sLive[tid] = 0u;
+  if (tid < R * 16) reinterpret_cast<uint32_t*>(sFlag)[tid] = 0u;
   if (tid == 0) sRedo = 0u;
   lds_barrier();
   // A wave takes every fourth key tile; the mask values of eight of its tiles and all rows are
@@ -185,15 +187,11 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
   // them, and they travel while it, the barriers and the first tiles' loads are under way.
   bf16x8 qf[R][2];
   u32x2 gw[R][4];  // output gates: used at the very end
-  // What a wave finds out about its tiles stays in scalar registers (the ballots are uniform)
-  // and reaches the workgroup's words in LDS once, at the end.
-  uint64_t my_live[R], my_plain[R];
+  // What a wave finds out about a tile is one byte in LDS, written by all its lanes alike; the
+  // workgroup's bit masks of live and of wholly unmasked tiles are ballots over those bytes.
   bool my_any[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    my_live[r] = my_plain[r] = 0ull;
-    my_any[r] = false;
-  }
+  for (int r = 0; r < R; ++r) my_any[r] = false;
   for (int t0 = 0; t0 < nkt; t0 += 32) {
     float mv[R][8];
 #pragma unroll
@@ -226,24 +224,13 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
           sCode[r * nk64 + key] = (uint16_t)(key >= N ? BF16_NEG_INF : (mv[r][u] == 0.f ? BF16_NEG_1E9 : 0u));
           const uint64_t on_lanes = __ballot(on);
           my_any[r] = my_any[r] || on_lanes != 0ull;
-          if (tile < 64) {
-            my_live[r] |= (uint64_t)(on_lanes != 0ull) << tile;
-            my_plain[r] |= (uint64_t)(on_lanes == ~0ull) << tile;
-          }
+          if (tile < 64) sFlag[r * 64 + tile] = (uint8_t)((on_lanes != 0ull ? 1 : 0) | (on_lanes == ~0ull ? 2 : 0));
         }
       }
   }
-  if (lane == 0) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      if (!my_any[r]) continue;
-      atomicOr(&sLive[r * 5], (uint32_t)my_live[r]);
-      atomicOr(&sLive[r * 5 + 1], (uint32_t)(my_live[r] >> 32));
-      atomicOr(&sLive[r * 5 + 2], 1u);
-      atomicOr(&sLive[r * 5 + 3], (uint32_t)my_plain[r]);
-      atomicOr(&sLive[r * 5 + 4], (uint32_t)(my_plain[r] >> 32));
-    }
-  }
+  for (int r = 0; r < R; ++r)
+    if (my_any[r]) sLive[r] = 1u;
   lds_barrier();
   bool dead[R];
   uint64_t live = 0ull;
@@ -251,12 +238,11 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
   bool all_dead = true;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    dead[r] = __builtin_amdgcn_readfirstlane(sLive[r * 5 + 2]) == 0u;
+    dead[r] = __builtin_amdgcn_readfirstlane(sLive[r]) == 0u;
+    const uint32_t flag = lane < nkt ? sFlag[r * 64 + lane] : 0u;
     all_dead = all_dead && dead[r];
-    live |= (uint64_t)__builtin_amdgcn_readfirstlane(sLive[r * 5]) |
-            ((uint64_t)__builtin_amdgcn_readfirstlane(sLive[r * 5 + 1]) << 32);
-    plain[r] = (uint64_t)__builtin_amdgcn_readfirstlane(sLive[r * 5 + 3]) |
-               ((uint64_t)__builtin_amdgcn_readfirstlane(sLive[r * 5 + 4]) << 32);
+    live |= __ballot((flag & 1u) != 0u);
+    plain[r] = __ballot((flag & 2u) != 0u);
   }
   // next live tile, or nkt when none is left; more than 64 tiles are simply taken in order
   uint64_t rest = live;
