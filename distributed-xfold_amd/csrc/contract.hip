@@ -79,6 +79,15 @@ __device__ __forceinline__ T* uniform_ptr(T* p) {
   return reinterpret_cast<T*>(((uint64_t)hi << 32) | lo);
 }
 
+// One accumulator value, read where the source says: left to itself the register allocator,
+// faced with an epilogue of many basic blocks, copies most of the 256 accumulators out of their
+// accumulation registers up front, which costs as many vector registers (and spills).
+__device__ __forceinline__ float acc_read(float a) {
+  float v;
+  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+  return v;
+}
+
 // s_waitcnt with vmcnt = n, lgkmcnt = 0 (expcnt left alone)
 template <int N>
 __device__ __forceinline__ void wait_loads_but() {
@@ -321,73 +330,91 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
     const int col_end = MODE == BIG_SWIGLU ? g.N / 2 : MODE == BIG_PLAIN ? g.ldc : g.N;
     const __amdgpu_buffer_rsrc_t whole =
         __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(C), 0, MODE == BIG_COLUMN_OPS && g.regroup32 ? g.M * g.N * 2 : 0, RSRC_RAW);
+    // Pass n = (it, p): 32 rows x 64 output columns.  convert: accumulators -> eight packed 8-byte
+    // pieces per lane; write: those into the staging area; read_store: 16 bytes per lane back out
+    // of it and to memory.  The passes are software-pipelined in the source (write n, convert
+    // n + 1, read_store n): the conversions of the next pass fill the LDS round trip of this one.
+    constexpr int NP = IT * PASSES;
+    auto convert = [&](int n, u32x2* out) {
+      const int it = n / PASSES, p = n % PASSES;
 #pragma unroll
-    for (int it = 0; it < IT; ++it) {
+      for (int jj = 0; jj < 2; ++jj) {
+        const int jt = MODE == BIG_SWIGLU ? 2 * jj : 2 * p + jj;
+        // column ops: a 32-column block never straddles segments (seg_len % 32 == 0)
+        bool affine = false, sig = false;
+        float alpha = 1.f;
+        const int nb = t.n0 + wn + 32 * jt;
+        if constexpr (MODE == BIG_COLUMN_OPS) {
+          int op = SEG_BIAS_SCALE;
+          sig = g.act_sigmoid != 0;
+          if (g.epi == EPI_SEGMENTED) {
+            op = (g.seg_ops >> (4 * (min(nb, g.N - 1) / g.seg_len))) & 15;
+            sig = op == SEG_SIGMOID;
+          }
+          affine = op == SEG_BIAS_SCALE;
+          if (affine) alpha = g.alpha;
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float o[4];
+          f32x4 bb = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (MODE == BIG_COLUMN_OPS) {
+            if (affine && g.bias) bb = *reinterpret_cast<const f32x4*>(g.bias + min(nb + 8 * q + 4 * hh, g.N - 4));
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float v = acc_read(acc[jt][it][4 * q + e]);
+            if constexpr (MODE == BIG_COLUMN_OPS) {
+              v = (v + bb[e]) * alpha;
+              if (sig) v = sigmoidf_(v);
+            }
+            if constexpr (MODE == BIG_SWIGLU) v = v * sigmoidf_(v) * acc_read(acc[jt + 1][it][4 * q + e]);
+            o[e] = v;
+          }
+          out[4 * jj + q].x = pack2bf(o[0], o[1]);
+          out[4 * jj + q].y = pack2bf(o[2], o[3]);
+        }
+      }
+    };
+    auto write = [&](const u32x2* in) {
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<u32x2*>(sE + l31 * LDE + 32 * jj + 8 * q + 4 * hh) = in[4 * jj + q];
+    };
+    // Bounds are enforced by the memory pipeline, not by branches (which would cut the
+    // epilogue into many basic blocks): a buffer descriptor that ends with the last valid row
+    // of this 32-row block drops rows past M, and lanes whose columns lie past the end
+    // get an offset beyond any descriptor.  Every wave issues all its stores.
+    auto read_store = [&](int n) {
+      const int it = n / PASSES, p = n % PASSES;
       const int row0 = t.m0 + wm + 32 * it;
       const __amdgpu_buffer_rsrc_t rows32 = __builtin_amdgcn_make_buffer_rsrc(
           uniform_ptr(C + (int64_t)row0 * g.ldc), 0,
           __builtin_amdgcn_readfirstlane(max(0, min(32, g.M - row0)) * g.ldc * 2), RSRC_RAW);
+      const int col0 = MODE == BIG_SWIGLU ? (t.n0 + wn) / 2 : t.n0 + wn + 64 * p;
+      const uint32_t voff = c8 * 8 < col_end - col0 ? lane_off + (uint32_t)col0 * 2u : 0x80000000u;
 #pragma unroll
-      for (int p = 0; p < PASSES; ++p) {
-#pragma unroll
-        for (int jj = 0; jj < 2; ++jj) {
-          const int jt = MODE == BIG_SWIGLU ? 2 * jj : 2 * p + jj;
-          // column ops: a 32-column block never straddles segments (seg_len % 32 == 0)
-          bool affine = false, sig = false;
-          float alpha = 1.f;
-          const int nb = t.n0 + wn + 32 * jt;
-          if constexpr (MODE == BIG_COLUMN_OPS) {
-            int op = SEG_BIAS_SCALE;
-            sig = g.act_sigmoid != 0;
-            if (g.epi == EPI_SEGMENTED) {
-              op = (g.seg_ops >> (4 * (min(nb, g.N - 1) / g.seg_len))) & 15;
-              sig = op == SEG_SIGMOID;
-            }
-            affine = op == SEG_BIAS_SCALE;
-            if (affine) alpha = g.alpha;
-          }
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            float o[4];
-            f32x4 bb = {0.f, 0.f, 0.f, 0.f};
-            if constexpr (MODE == BIG_COLUMN_OPS) {
-              if (affine && g.bias) bb = *reinterpret_cast<const f32x4*>(g.bias + min(nb + 8 * q + 4 * hh, g.N - 4));
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              float v = acc[jt][it][4 * q + e];
-              if constexpr (MODE == BIG_COLUMN_OPS) {
-                v = (v + bb[e]) * alpha;
-                if (sig) v = sigmoidf_(v);
-              }
-              if constexpr (MODE == BIG_SWIGLU) v = v * sigmoidf_(v) * acc[jt + 1][it][4 * q + e];
-              o[e] = v;
-            }
-            u32x2 v2;
-            v2.x = pack2bf(o[0], o[1]);
-            v2.y = pack2bf(o[2], o[3]);
-            *reinterpret_cast<u32x2*>(sE + l31 * LDE + 32 * jj + 8 * q + 4 * hh) = v2;
-          }
-        }
-        // Bounds are enforced by the memory pipeline, not by branches (which would cut the
-        // epilogue into many basic blocks): a buffer descriptor that ends with the last valid row
-        // of this 32-row block drops rows past M, and lanes whose columns lie past the end
-        // get an offset beyond any descriptor.  Every wave issues all its stores.
-        const int col0 = MODE == BIG_SWIGLU ? (t.n0 + wn) / 2 : t.n0 + wn + 64 * p;
-        const uint32_t voff = c8 * 8 < col_end - col0 ? lane_off + (uint32_t)col0 * 2u : 0x80000000u;
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          const int r = 8 * s + rsub;
-          const u32x4 v = *reinterpret_cast<const u32x4*>(sE + r * LDE + c8 * 8);
-          if (MODE == BIG_COLUMN_OPS && g.regroup32) {
-            const int row = row0 + r, col = col0 + c8 * 8;
-            const uint32_t off = ((((uint32_t)(row >> 5) * (uint32_t)(g.N >> 5) + (col >> 5)) * 32 + (row & 31)) * 32 + (col & 31)) * 2u;
-            __builtin_amdgcn_raw_buffer_store_b128(v, whole, row < g.M && col < g.N ? off : 0x80000000u, 0, 0);
-          } else {
-            __builtin_amdgcn_raw_buffer_store_b128(v, rows32, voff + (uint32_t)(8 * s * g.ldc) * 2u, 0, 0);
-          }
+      for (int s = 0; s < 4; ++s) {
+        const int r = 8 * s + rsub;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(sE + r * LDE + c8 * 8);
+        if (MODE == BIG_COLUMN_OPS && g.regroup32) {
+          const int row = row0 + r, col = col0 + c8 * 8;
+          const uint32_t off = ((((uint32_t)(row >> 5) * (uint32_t)(g.N >> 5) + (col >> 5)) * 32 + (row & 31)) * 32 + (col & 31)) * 2u;
+          __builtin_amdgcn_raw_buffer_store_b128(v, whole, row < g.M && col < g.N ? off : 0x80000000u, 0, 0);
+        } else {
+          __builtin_amdgcn_raw_buffer_store_b128(v, rows32, voff + (uint32_t)(8 * s * g.ldc) * 2u, 0, 0);
         }
       }
+    };
+    u32x2 vals[2][8];
+    convert(0, vals[0]);
+#pragma unroll
+    for (int n = 0; n < NP; ++n) {
+      write(vals[n & 1]);
+      if (n + 1 < NP) convert(n + 1, vals[(n + 1) & 1]);
+      read_store(n);
     }
   };
 
