@@ -422,17 +422,17 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   while (true) {
     const bool has_next = tile_at(slot + slot_step, next_t);
     if (!has_next) next_t = cur_t;  // the loads past the tile's end then re-read its first slabs, unused
-#pragma unroll
-    for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-      for (int it = 0; it < IT; ++it)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[jt][it][r] = 0.f;
-    for (int kt = 0; kt < nk4; kt += 4) {
+    // the tile's first four stages apart: its very first k-step starts the accumulators from the
+    // constant zero (no 256 moves to clear them), and a branch on "first" inside the loop would
+    // have the accumulators meet at its join
+    stage(0, std::integral_constant<int, 0>{}, std::true_type{}, nk4 == 4, stored);
+    stage(1, std::integral_constant<int, 1>{}, std::false_type{}, nk4 == 4, stored);
+    stage(2, std::integral_constant<int, 2>{}, std::false_type{}, nk4 == 4, false);
+    stage(3, std::integral_constant<int, 3>{}, std::false_type{}, nk4 == 4, false);
+    for (int kt = 4; kt < nk4; kt += 4) {
       const bool last = kt + 4 == nk4;
-      const bool behind_stores = kt == 0 && stored;
-      stage(kt, std::integral_constant<int, 0>{}, std::false_type{}, last, behind_stores);
-      stage(kt + 1, std::integral_constant<int, 1>{}, std::false_type{}, last, behind_stores);
+      stage(kt, std::integral_constant<int, 0>{}, std::false_type{}, last, false);
+      stage(kt + 1, std::integral_constant<int, 1>{}, std::false_type{}, last, false);
       stage(kt + 2, std::integral_constant<int, 2>{}, std::false_type{}, last, false);
       stage(kt + 3, std::integral_constant<int, 3>{}, std::false_type{}, last, false);
     }
