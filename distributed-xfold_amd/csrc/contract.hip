@@ -116,6 +116,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   __shared__ __attribute__((aligned(1024))) char sb2[SLAB];
   __shared__ __attribute__((aligned(1024))) char sb3[SLAB];
   __shared__ __attribute__((aligned(16))) char sOut[4 * EPI_BYTES];
+  __shared__ __attribute__((aligned(16))) float sColBias[MODE == BIG_COLUMN_OPS ? 4 * 128 : 4];  // a wave's 128 bias values
   auto buf = [&](int i) -> char* { return (i & 3) == 0 ? sb0 : (i & 3) == 1 ? sb1 : (i & 3) == 2 ? sb2 : sb3; };
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -335,6 +336,20 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
     // of it and to memory.  The passes are software-pipelined in the source (write n, convert
     // n + 1, read_store n): the conversions of the next pass fill the LDS round trip of this one.
     constexpr int NP = IT * PASSES;
+    // The bias of the wave's 128 columns goes through LDS once per tile, requested before the
+    // tile's first store: a load from memory issued between the stores would wait for them all
+    // (vector memory operations retire in order).
+    float* sBiasW = sColBias + (MODE == BIG_COLUMN_OPS ? wave * 128 : 0);
+    if constexpr (MODE == BIG_COLUMN_OPS) {
+      // the bias array only covers the segments that use it
+      const int colb = t.n0 + wn + 4 * lane;
+      bool uses_bias = g.bias != nullptr && lane < 32;
+      if (g.epi == EPI_SEGMENTED)
+        uses_bias = uses_bias && ((g.seg_ops >> (4 * (min(colb, g.N - 1) / g.seg_len))) & 15) == SEG_BIAS_SCALE;
+      f32x4 b4 = {0.f, 0.f, 0.f, 0.f};
+      if (uses_bias) b4 = *reinterpret_cast<const f32x4*>(g.bias + min(colb, g.N - 4));
+      if (lane < 32) *reinterpret_cast<f32x4*>(sBiasW + 4 * lane) = b4;
+    }
     auto convert = [&](int n, u32x2* out) {
       const int it = n / PASSES, p = n % PASSES;
 #pragma unroll
@@ -359,7 +374,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
           float o[4];
           f32x4 bb = {0.f, 0.f, 0.f, 0.f};
           if constexpr (MODE == BIG_COLUMN_OPS) {
-            if (affine && g.bias) bb = *reinterpret_cast<const f32x4*>(g.bias + min(nb + 8 * q + 4 * hh, g.N - 4));
+            if (affine && g.bias) bb = *reinterpret_cast<const f32x4*>(sBiasW + 32 * jt + 8 * q + 4 * hh);
           }
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
