@@ -324,8 +324,9 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
   bf16_t* sE = reinterpret_cast<bf16_t*>(sOut + wave * EPI_BYTES);
   auto store_tile = [&](const Tile& t) {
     bf16_t* C = reinterpret_cast<bf16_t*>(g.C) + (int64_t)t.bz * g.sC;
-    constexpr int JSTEP = MODE == BIG_SWIGLU ? 2 : 1;  // SwiGLU: tiles (0,1) and (2,3) give 32 output columns each
-    constexpr int PASSES = MODE == BIG_SWIGLU ? 1 : 2;  // 64 output columns per pass
+    // SwiGLU: accumulator tiles (0,1) and (2,3) give 32 output columns each, one pass per 32 rows;
+    // otherwise two passes of 64 output columns
+    constexpr int PASSES = MODE == BIG_SWIGLU ? 1 : 2;
     const int c8 = lane & 7, rsub = lane >> 3;  // 8 chunks of 8 output columns per row, 8 rows per instruction
     const uint32_t lane_off = (uint32_t)(rsub * g.ldc + c8 * 8) * 2u;
     const int col_end = MODE == BIG_SWIGLU ? g.N / 2 : MODE == BIG_PLAIN ? g.ldc : g.N;
