@@ -412,14 +412,14 @@ def main():
     a[:, :, n:] = 0
     b[:, :, n:] = 0
     t_buf = torch.empty_like(a)
-    q_, k_, g_ = ((torch.randn(n, 4, n, 32, generator=g) * 0.5).to(dev).bfloat16() for _ in range(3))
+    q_, k_ = ((torch.randn(n, 4, n, 32, generator=g) * 0.5).to(dev).bfloat16() for _ in range(2))
     vt_ = pkg.ops.pack_vt((torch.randn(n, 4, 32, n, generator=g) * 0.5).to(dev).bfloat16())
     nb = pkg.ops.pack_pair_bias(torch.randn(4, n, n, generator=g).to(dev))
     og = torch.empty((n * n, 128), dtype=torch.bfloat16, device=dev)
     # (the operands above are generated on the host, during which the GPU idles and its clock drops)
     ms_contract = gpu_time_ms(lambda: pkg.ops.triangle_contraction(a, b, t_buf), 30, warm_ms=40.0)
-    ms_attn = gpu_time_ms(lambda: pkg.ops.grid_attention_core(q_, k_, vt_, g_, nb, pair_mask, og), 30, warm_ms=40.0)
-    ms_attn_un = gpu_time_ms(lambda: pkg.ops.grid_attention_core(q_, k_, vt_, g_, nb, pair_ones, og), 30,
+    ms_attn = gpu_time_ms(lambda: pkg.ops.grid_attention_core(q_, k_, vt_, nb, pair_mask, og), 30, warm_ms=40.0)
+    ms_attn_un = gpu_time_ms(lambda: pkg.ops.grid_attention_core(q_, k_, vt_, nb, pair_ones, og), 30,
                              warm_ms=40.0)
     # FLOPs the attention core executes under the trailing padding: a row without a live key takes the uniform
     # shortcut (no products), a live row visits only the 64-key tiles that hold a live key, all N queries each
@@ -449,7 +449,7 @@ def main():
 
     roofline = roofline_of(ms_contract, ms_attn, executed_attn)
     roofline_un = roofline_of(ms_contract, ms_attn_un, flops_attention_core(n))
-    del a, b, t_buf, q_, k_, g_, vt_, nb, og
+    del a, b, t_buf, q_, k_, vt_, nb, og
 
     # ---- the target run: the 48-block trunk at 1536 tokens, whole pair tensor resident ----
     trunk = None if args.no_trunk else trunk_n1536(pkg, dev)

@@ -68,7 +68,7 @@ void* static_scratch_ptr() {
 
 extern "C" {
 
-int af3_abi_version(void) { return 1; }
+int af3_abi_version(void) { return AF3_ABI_VERSION; }
 
 const char* af3_error_string(int code) {
   switch (code) {
@@ -144,12 +144,12 @@ static int triangle_multiplication_impl(
 size_t af3_grid_self_attn_workspace_bytes(int64_t n, int num_head) {
   if (n <= 0 || num_head <= 0) return 0;
   const size_t e = sizeof(bf16_t), ldn = (size_t)tri_ldn(n);
-  // fast path: q, k, g planes, vt, og, fp16 bias
-  const size_t fast = 3 * align_up((size_t)n * n * C_PAIR * e, 256) + align_up((size_t)n * C_PAIR * ldn * e, 256) +
+  // fast path: q, k planes, vt, og, fp16 bias
+  const size_t fast = 2 * align_up((size_t)n * n * C_PAIR * e, 256) + align_up((size_t)n * C_PAIR * ldn * e, 256) +
                       align_up((size_t)n * n * C_PAIR * e, 256) +
                       align_up((size_t)tri_bias_elems(n, num_head) * sizeof(uint16_t), 256);
-  // general path (external fp32 bias): qkvg + og
-  const size_t general = align_up((size_t)n * n * 4 * C_PAIR * e, 256) + align_up((size_t)n * n * C_PAIR * e, 256);
+  // general path (external fp32 bias): qkv + og
+  const size_t general = align_up((size_t)n * n * 3 * C_PAIR * e, 256) + align_up((size_t)n * n * C_PAIR * e, 256);
   return fast > general ? fast : general;
 }
 
@@ -181,7 +181,6 @@ static int grid_self_attn_impl(
     const int64_t ldn = tri_ldn(n);
     bf16_t* q = ws.take<bf16_t>((size_t)n * n * C_PAIR);
     bf16_t* k = ws.take<bf16_t>((size_t)n * n * C_PAIR);
-    bf16_t* g = ws.take<bf16_t>((size_t)n * n * C_PAIR);
     bf16_t* vt = ws.take<bf16_t>((size_t)n * C_PAIR * ldn);
     og = ws.take<bf16_t>((size_t)n * n * C_PAIR);
     uint16_t* bias = ws.take<uint16_t>((size_t)tri_bias_elems(n, num_head));
@@ -192,33 +191,33 @@ static int grid_self_attn_impl(
     p.skip_ln = ln_w == nullptr; p.ln_w = ln_w; p.ln_b = ln_b;
     p.w_qkvg = w_qkvg; p.w_bias = w_pair_bias; p.n_bias = w_pair_bias ? num_head : 0;
     p.q_scale = LOG2E / sqrtf(d_valid); p.bias_scale = LOG2E;
-    p.q = q; p.k = k; p.vt = vt; p.g = g; p.bias = bias; p.ldn = ldn;
+    p.q = q; p.k = k; p.vt = vt; p.bias = bias; p.ldn = ldn;
     rc = launch_triattn_proj(p, s);
     if (rc) return rc;
     TriAttnArgs t;
-    t.q = q; t.k = k; t.vt = vt; t.g = g; t.bias = w_pair_bias ? bias : nullptr;
+    t.q = q; t.k = k; t.vt = vt; t.bias = w_pair_bias ? bias : nullptr;
     t.mask = mask; t.og = og; t.N = (int)n; t.ldn = ldn;
     rc = launch_triattn_flash(t, s);
     if (rc) return rc;
   } else {
     // General path: an external fp32 bias [H][N][N] (operator-level contract).
-    bf16_t* qkvg = ws.take<bf16_t>((size_t)n * n * 4 * C_PAIR);
+    bf16_t* qkv = ws.take<bf16_t>((size_t)n * n * 3 * C_PAIR);
     og = ws.take<bf16_t>((size_t)n * n * C_PAIR);
     if (!ws.ok) return AF3_ERR_WORKSPACE;
     AttnProjArgs p;
     p.lw = ln_width(valid_channels);
     p.pair = pair; p.io_f32 = io_dtype == AF3_F32; p.N = (int)n; p.transpose = transpose != 0;
     p.ln_w = ln_w; p.ln_b = ln_b; p.skip_ln = ln_w == nullptr;
-    p.w_main = w_qkvg; p.n_chunks = 4;
-    p.chunk_ops = SEG_BIAS_SCALE | (SEG_PLAIN << 4) | (SEG_PLAIN << 8) | (SEG_SIGMOID << 12);
+    p.w_main = w_qkvg; p.n_chunks = 3;  // the gate chunk is applied by attn_out
+    p.chunk_ops = SEG_BIAS_SCALE | (SEG_PLAIN << 4) | (SEG_PLAIN << 8);
     p.q_scale = 1.0f / sqrtf(d_valid);
-    p.out_main = qkvg; p.ld_main = 4 * C_PAIR;
+    p.out_main = qkv; p.ld_main = 3 * C_PAIR;
     rc = launch_attn_proj(p, s);
     if (rc) return rc;
     FlashArgs f;
-    f.q = qkvg; f.k = qkvg + C_PAIR; f.v = qkvg + 2 * C_PAIR; f.g = qkvg + 3 * C_PAIR;
-    f.q_ss = f.k_ss = f.v_ss = f.g_ss = 4 * C_PAIR;
-    f.q_sb = f.k_sb = f.v_sb = f.g_sb = n * 4 * C_PAIR;
+    f.q = qkv; f.k = qkv + C_PAIR; f.v = qkv + 2 * C_PAIR;
+    f.q_ss = f.k_ss = f.v_ss = 3 * C_PAIR;
+    f.q_sb = f.k_sb = f.v_sb = n * 3 * C_PAIR;
     f.out = og; f.out_f32 = 0; f.o_ss = C_PAIR; f.o_sb = n * C_PAIR;
     f.B = (int)n; f.H = num_head; f.Sq = f.Sk = (int)n; f.d = d;
     f.bias = nonbatched_bias; f.bias_sb = 0; f.bias_sh = n * n; f.bias_sq = n;
@@ -228,7 +227,9 @@ static int grid_self_attn_impl(
   }
 
   AttnOutArgs o;
-  o.og = og; o.ld_og = C_PAIR; o.w_out = w_output; o.pair = pair; o.out = out;
+  o.lw = ln_width(valid_channels);
+  o.og = og; o.ld_og = C_PAIR; o.w_gate = w_qkvg + 3 * C_PAIR * C_PAIR; o.w_out = w_output; o.pair = pair; o.out = out;
+  o.skip_ln = ln_w == nullptr; o.ln_w = ln_w; o.ln_b = ln_b;
   o.io_f32 = io_dtype == AF3_F32; o.N = (int)n; o.transpose = transpose != 0; o.residual = residual != 0;
   return launch_attn_out(o, s);
 }
@@ -623,11 +624,11 @@ int af3_triangle_contraction_forward(
 }
 
 int af3_grid_attention_core_forward(
-    const uint16_t* q, const uint16_t* k, const uint16_t* vt, const uint16_t* g,
+    const uint16_t* q, const uint16_t* k, const uint16_t* vt,
     const uint16_t* pair_bias, const float* mask, uint16_t* og, int64_t n, af3_stream_t stream) {
   if (n <= 0 || n > 8192) return AF3_ERR_BAD_ARG;
   TriAttnArgs t;
-  t.q = q; t.k = k; t.vt = vt; t.g = g; t.bias = pair_bias; t.mask = mask; t.og = og;
+  t.q = q; t.k = k; t.vt = vt; t.bias = pair_bias; t.mask = mask; t.og = og;
   t.N = (int)n; t.ldn = tri_ldn(n);
   return launch_triattn_flash(t, static_cast<hipStream_t>(stream));
 }

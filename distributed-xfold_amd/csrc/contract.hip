@@ -68,7 +68,7 @@ constexpr int RSRC_RAW = 0x00020000;     // last word of a raw (unstructured, ra
 // explicit wait and barrier that follow the load's issue.
 __device__ __forceinline__ void load_to_lds(const char* base, uint32_t off, const char* dst) {
   const uint32_t lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)dst;
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(off), "s"(base));
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(off), "s"(base) : "m0");
 }
 
 // a pointer the compiler cannot prove wave-uniform, moved to scalar registers

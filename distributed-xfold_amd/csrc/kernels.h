@@ -129,10 +129,14 @@ struct AttnProjArgs {
 int launch_attn_proj(const AttnProjArgs& a, hipStream_t s);
 
 struct AttnOutArgs {
-  const bf16_t* og = nullptr;  // [(b*N + s)][ld_og] gated attention output
+  LnWidth lw;
+  const bf16_t* og = nullptr;  // [(b*N + s)][ld_og] attention output, normalised, not yet gated
   int64_t ld_og = 0;
-  const bf16_t* w_out = nullptr;  // [128][128]
-  const void* pair = nullptr;     // residual source
+  const bf16_t* w_gate = nullptr;  // [128][128] gating_query: the gate is sigmoid(LN(pair) w_gate^T)
+  const bf16_t* w_out = nullptr;   // [128][128]
+  const void* pair = nullptr;      // gate input and residual source
+  int skip_ln = 0;                 // pair is already normalised
+  const float *ln_w = nullptr, *ln_b = nullptr;
   void* out = nullptr;
   int io_f32 = 0, N = 0, transpose = 0, residual = 0;
 };
@@ -180,7 +184,7 @@ int launch_flash_attention(const FlashArgs& a, hipStream_t stream);
 // ------------------------------------------- triattn.hip, triattn_core.hip
 // Scratch of the triangle-attention fast path, in the frame of the (possibly
 // transposed) operator, rows b:
-//   q, k, g  bf16 [b][h][s][32]   (q times log2(e)/sqrt(32); g = sigmoid gate)
+//   q, k     bf16 [b][h][s][32]   (q times log2(e)/sqrt(32))
 //   vt       bf16 [b][h][32][ldn] V transposed, ldn = N rounded up to 16, columns >= N zero,
 //            key k of a row stored at column tri_vt_pos(k): inside every aligned group of 16
 //            keys the two middle quads are swapped, which makes the 8 keys one lane feeds to
@@ -210,21 +214,21 @@ struct TriAttnProjArgs {
   const void* pair = nullptr;  // [N][N][128]
   int io_f32 = 0, N = 0, transpose = 0, skip_ln = 0;
   const float *ln_w = nullptr, *ln_b = nullptr;
-  const bf16_t* w_qkvg = nullptr;  // [4][128][128]
+  const bf16_t* w_qkvg = nullptr;  // [4][128][128]: q, k, v chunks are used here (the gate chunk by attn_out)
   const bf16_t* w_bias = nullptr;  // [32][128], rows >= 4 zero
   int n_bias = 0;                  // 0 or 4
   float q_scale = 1.f, bias_scale = 1.f;
-  bf16_t *q = nullptr, *k = nullptr, *vt = nullptr, *g = nullptr;
+  bf16_t *q = nullptr, *k = nullptr, *vt = nullptr;
   uint16_t* bias = nullptr;  // fp16 bits, fragment order, tri_bias_elems(N, 4) elements
   int64_t ldn = 0;        // tri_ldn(N)
 };
 int launch_triattn_proj(const TriAttnProjArgs& a, hipStream_t stream);
 
 struct TriAttnArgs {
-  const bf16_t *q = nullptr, *k = nullptr, *vt = nullptr, *g = nullptr;
+  const bf16_t *q = nullptr, *k = nullptr, *vt = nullptr;
   const uint16_t* bias = nullptr;  // fp16 bits, fragment order (tri_bias_offset), or null
   const float* mask = nullptr;   // [N][N] 0/1 or null
-  bf16_t* og = nullptr;          // [(b*N + s)][128]
+  bf16_t* og = nullptr;          // [(b*N + s)][128] normalised attention output (the gate is applied by attn_out)
   int N = 0;
   int64_t ldn = 0;
 };

@@ -11,7 +11,7 @@
 //   trimul_epilogue  channel-major contraction result -> LN -> out-proj ->
 //                    * sigmoid(LN(x) Wgl^T) -> (+ residual)
 //   attn_proj        LN -> q (scaled), k, v, sigmoid gate, + pair-bias heads
-//   attn_out         gated attention output -> out-proj -> (+ residual)
+//   attn_out         attention output * sigmoid(LN(x) Wg^T) -> out-proj -> (+ residual)
 //   transition       LN -> W1 -> silu(a) * b -> W2 -> (+ residual), hidden in registers
 //
 // MFMA orientation: "D form" computes out[px][ch] with the pixel fragments as
@@ -84,22 +84,12 @@ __global__ __launch_bounds__(256, 3) void trimul_prologue_kernel(TriMulArgs a) {
     }
     return;
   }
-#ifdef AF3_PROF
-  long long stamps[14];
-  int n_stamp = 0;
-#define PSTAMP() do { stamps[n_stamp++] = __builtin_readcyclecounter(); } while (0)
-#else
-#define PSTAMP() do {} while (0)
-#endif
-  PSTAMP();
   wload(0);
   if (tid < TM) sMask[tid] = mk;
   load_ln_tile<TIO>(x, t, a.ln_in_w, a.ln_in_b, sX, tid, false, a.lw.inv_c, a.lw.pad);
-  PSTAMP();
   wstore(sW0);
   wload(1);
   lds_barrier();
-  PSTAMP();
   bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
   lds_barrier();  // sX is free from here on
@@ -179,9 +169,7 @@ __global__ __launch_bounds__(256, 3) void trimul_prologue_kernel(TriMulArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     }
     lds_barrier();
-    PSTAMP();
   };
-  PSTAMP();
   step(std::integral_constant<int, 0>{}, accA, accB);
   step(std::integral_constant<int, 1>{}, accB, accA);
   step(std::integral_constant<int, 2>{}, accA, accB);
@@ -203,13 +191,6 @@ __global__ __launch_bounds__(256, 3) void trimul_prologue_kernel(TriMulArgs a) {
             *reinterpret_cast<const u32x4*>(sS1 + c2 * LDX + pc * 8);
     }
   }
-#ifdef AF3_PROF
-  PSTAMP();
-  if (tid == 0) {
-    long long* dst = reinterpret_cast<long long*>(a.a_buf + ((int64_t)0 * a.N + t.o) * a.Np + t.r0);
-    for (int i = 0; i < 14; ++i) dst[i] = stamps[i];
-  }
-#endif
 }
 
 // ============================================================================
@@ -393,31 +374,61 @@ __global__ __launch_bounds__(256, 2) void attn_proj_kernel(AttnProjArgs a) {
 }
 
 // ============================================================================
-// triangle attention: output projection
+// triangle attention: output gate and output projection
 // ============================================================================
+// The attention core leaves the normalised, ungated output.  The gate sigmoid(LN(x) Wg^T) belongs to the
+// same pixel of the pair tensor that this kernel reads anyway for the residual, so it is computed here
+// (one LayerNorm and one 128 x 128 product per pixel) instead of making a round trip through memory as a
+// fourth projection plane.  The gate comes out of its MFMAs in T form (a lane owns a pixel and, per
+// register quad, 4 consecutive weight rows); with the weight rows permuted on their way into LDS (row rho
+// holds channel swap23(rho): bits 2 and 3 exchanged) a lane-half's registers 8 a .. 8 a + 7 of tile nt are
+// the eight consecutive channels 32 nt + 16 a + 8 hh .. of its pixel: exactly the B fragment of k-step
+// 2 nt + a of the output projection, so gate and attention output meet register by register.
 template <typename TIO>
-__global__ __launch_bounds__(256) void attn_out_kernel(AttnOutArgs a) {
+__global__ __launch_bounds__(256, 2) void attn_out_kernel(AttnOutArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t smem[2 * TM * LDX];
   bf16_t* sX = smem;
   bf16_t* sW = smem + TM * LDX;
   float* sS = reinterpret_cast<float*>(smem);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const Tile t = make_tile(a.N, a.transpose != 0);  // where the result lands in the pair tensor
-  // Everything the tile needs is requested up front, unconditionally (rows past
-  // the end re-read a valid one and are zeroed / skipped later): the gated
-  // attention output, the output weights and the residual rows.
+  // Loads are unconditional (rows past the end re-read a valid one and are zeroed /
+  // skipped later).  Up front: the pair rows (gate input and residual) and the gate
+  // weights; the attention output follows once the gate's MFMAs are issued (its 32
+  // registers would not fit beside them).  The bf16 stream keeps its pair rows in
+  // registers for the residual; the fp32 stream (twice the registers) reads them a
+  // second time at the end.
+#ifndef X_KEEP_ROWS
+#define X_KEEP_ROWS false
+#endif
+  constexpr bool KEEP_ROWS = X_KEEP_ROWS;
+  const TIO* x = reinterpret_cast<const TIO*>(a.pair);
   const int ck = tid & 15, prow = tid >> 4;
+  typename Elem<TIO>::Raw res[KEEP_ROWS ? 8 : 1];
+  if (KEEP_ROWS) prefetch_tile_rows<TIO>(x, t, tid, res);
+  WChunkRegs wr;
+  wr.load<true>(a.w_gate, tid);
+  if (KEEP_ROWS) ln_tile_from_rows<TIO>(res, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0, a.lw.inv_c, a.lw.pad);
+  else load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0, a.lw.inv_c, a.lw.pad);
+  wr.store(sW, tid);
+  lds_barrier();
+  bf16x8 xf[8];
+  load_x_frags(sX, wave, lane, xf);
+  f32x16 gate[4];
+  mfma_chunk<true, 4>(xf, sW, lane, gate);
+  // the attention output and the output weights travel while the sigmoids are taken
   u32x4 og[8];
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
     const int p = it * 16 + prow;
     og[it] = *reinterpret_cast<const u32x4*>(a.og + ((int64_t)t.o * a.N + t.r0 + (t.valid(p) ? p : 0)) * a.ld_og + ck * 8);
   }
-  WChunkRegs wr;
-  wr.load(a.w_out, tid);
-  const bool add = a.residual != 0;
-  typename Elem<TIO>::Raw res[8];
-  prefetch_tile_rows<TIO>(reinterpret_cast<const TIO*>(add ? a.pair : a.out), t, tid, res);
+  wr.load<false>(a.w_out, tid);
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) gate[nt][r] = sigmoidf_(gate[nt][r]);
+  lds_barrier();  // every wave is done with the LayerNorm tile and the gate weights
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
     const int p = it * 16 + prow;
@@ -426,14 +437,22 @@ __global__ __launch_bounds__(256) void attn_out_kernel(AttnOutArgs a) {
   }
   wr.store(sW, tid);
   lds_barrier();
-  bf16x8 xf[8];
   load_x_frags(sX, wave, lane, xf);
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    float f[8];
+    unpack8(__builtin_bit_cast(u32x4, xf[ks]), f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] *= gate[ks >> 1][8 * (ks & 1) + e];
+    xf[ks] = as_frag(pack8(f));
+  }
   f32x16 acc[4];
   mfma_chunk<true, 4>(xf, sW, lane, acc);
   lds_barrier();
   stage_t_f32(acc, sS, wave, lane);
   lds_barrier();
-  store_tile_f32_pre<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), res, add, tid);
+  if (KEEP_ROWS) store_tile_f32_pre<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), res, a.residual != 0, tid);
+  else store_tile_f32<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), a.residual ? x : nullptr, tid);
 }
 
 // ============================================================================
@@ -447,7 +466,7 @@ template <int OFF>
 __device__ __forceinline__ void lds_dma16(const char* gbase, uint32_t voff, const char* dst) {
   const uint32_t lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)dst;
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
-               :: "s"(lds), "v"(voff), "s"(gbase), "n"(OFF) : "memory");
+               :: "s"(lds), "v"(voff), "s"(gbase), "n"(OFF) : "memory", "m0");
 }
 // workgroup barrier that also waits for this wave's loads into LDS
 __device__ __forceinline__ void dma_lds_barrier() {
@@ -668,8 +687,10 @@ int launch_attn_proj(const AttnProjArgs& a, hipStream_t s) {
                   : launch_tiles(attn_proj_kernel<bf16_t>, a, a.N, a.N, s);
 }
 int launch_attn_out(const AttnOutArgs& a, hipStream_t s) {
-  if (a.N <= 0 || !a.og || !a.w_out || !a.out || (a.ld_og & 7) || (a.residual && !a.pair)) return AF3_ERR_BAD_ARG;
-  if (!aligned16(a.og) || !aligned16(a.w_out) || !aligned16(a.out) || !aligned16(a.pair)) return AF3_ERR_BAD_ARG;
+  if (a.N <= 0 || !a.og || !a.w_out || !a.w_gate || !a.out || (a.ld_og & 7) || !a.pair) return AF3_ERR_BAD_ARG;
+  if ((a.ln_w == nullptr) != (a.ln_b == nullptr) || (a.skip_ln == 0) != (a.ln_w != nullptr)) return AF3_ERR_BAD_ARG;
+  if (!aligned16(a.og) || !aligned16(a.w_out) || !aligned16(a.w_gate) || !aligned16(a.out) || !aligned16(a.pair))
+    return AF3_ERR_BAD_ARG;
   return a.io_f32 ? launch_tiles(attn_out_kernel<float>, a, a.N, a.N, s)
                   : launch_tiles(attn_out_kernel<bf16_t>, a, a.N, a.N, s);
 }

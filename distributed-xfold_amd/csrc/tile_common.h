@@ -49,13 +49,8 @@ __device__ __forceinline__ void load_param8(const float* p, float fill, float* o
   }
 }
 
-// LayerNorm of a tile of pixels from global memory into sX[p][c] (bf16).
-// Thread (prow = tid / 16, chunk = tid % 16) handles channels 8*chunk..+7 of
-// pixels prow, prow + 16, ...; 16 lanes cooperate on one pixel's statistics.
-// Out-of-range pixels become zero rows.  The loads of a batch of pixels are
-// unconditional (an out-of-range pixel re-reads the tile's first one) and all
-// issued before any value is converted: a load under a lane mask, or one whose
-// value is touched at once, costs a full memory round trip per pixel.
+// LayerNorm of one pixel's eight channels (the thread's share: 16 lanes cooperate on the
+// pixel's statistics) -> packed bf16.
 //
 // This phase is vector arithmetic per element and a large share of every tile
 // kernel's instructions, so the bf16 stream takes the short form: sum and sum of
@@ -67,12 +62,52 @@ __device__ __forceinline__ void load_param8(const float* p, float fill, float* o
 // two-pass form.  Zero-padded channels (fewer than 128 real ones) add nothing to
 // either sum; the two-pass form takes their pad * mean^2 out again.
 template <typename TIO>
+__device__ __forceinline__ u32x4 ln_pixel8(const typename Elem<TIO>::Raw& raw, const float* w, const float* b,
+                                           bool skip_ln, float inv_c, float pad) {
+  using E = Elem<TIO>;
+  constexpr bool ONE_PASS = sizeof(TIO) == 2;
+  float v[8], o[8];
+  E::unpack_raw(raw, v);
+  if (ONE_PASS) {
+    float s = 0.f, q = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { s += v[e]; q = fmaf(v[e], v[e], q); }
+    const float mean = group16_sum(s) * inv_c;
+    const float var = fmaxf(fmaf(group16_sum(q), inv_c, -mean * mean), 0.f);
+    // (an already normalised input comes with w = 1, b = 0: scale 1 and shift 0 pass it through unchanged)
+    const float rstd = skip_ln ? 1.f : rsqrtf(var + LN_EPS);
+    const float shift = skip_ln ? 0.f : -mean * rstd;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = fmaf(fmaf(v[e], rstd, shift), w[e], b[e]);
+  } else {
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += v[e];
+    const float mean = group16_sum(s) * inv_c;
+    float q = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { const float d = v[e] - mean; q += d * d; }
+    // (zero-padded channels, if any, each put mean^2 into the sum)
+    const float rstd = rsqrtf((group16_sum(q) - pad * mean * mean) * inv_c + LN_EPS);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = skip_ln ? v[e] : (v[e] - mean) * rstd * w[e] + b[e];
+  }
+  return pack8(o);
+}
+
+// LayerNorm of a tile of pixels from global memory into sX[p][c] (bf16).
+// Thread (prow = tid / 16, chunk = tid % 16) handles channels 8*chunk..+7 of
+// pixels prow, prow + 16, ...; 16 lanes cooperate on one pixel's statistics.
+// Out-of-range pixels become zero rows.  The loads of a batch of pixels are
+// unconditional (an out-of-range pixel re-reads the tile's first one) and all
+// issued before any value is converted: a load under a lane mask, or one whose
+// value is touched at once, costs a full memory round trip per pixel.
+template <typename TIO>
 __device__ __forceinline__ void load_ln_tile(const TIO* x, const Tile& t, const float* lnw,
                                              const float* lnb, bf16_t* sX, int tid, bool skip_ln = false,
                                              float inv_c = 1.f / C, float pad = 0.f) {
   using E = Elem<TIO>;
   constexpr int NB = E::kBatch;
-  constexpr bool ONE_PASS = sizeof(TIO) == 2;
   const int chunk = tid & 15, prow = tid >> 4;
   float w[8], b[8];
   load_param8(lnw ? lnw + chunk * 8 : nullptr, 1.f, w);
@@ -89,36 +124,29 @@ __device__ __forceinline__ void load_ln_tile(const TIO* x, const Tile& t, const 
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
       const int p = (base + i) * 16 + prow;
-      float v[8], o[8];
-      E::unpack_raw(raw[i], v);
-      if (ONE_PASS) {
-        float s = 0.f, q = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { s += v[e]; q = fmaf(v[e], v[e], q); }
-        const float mean = group16_sum(s) * inv_c;
-        const float var = fmaxf(fmaf(group16_sum(q), inv_c, -mean * mean), 0.f);
-        // (an already normalised input comes with w = 1, b = 0: scale 1 and shift 0 pass it through unchanged)
-        const float rstd = skip_ln ? 1.f : rsqrtf(var + LN_EPS);
-        const float shift = skip_ln ? 0.f : -mean * rstd;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = fmaf(fmaf(v[e], rstd, shift), w[e], b[e]);
-      } else {
-        float s = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s += v[e];
-        const float mean = group16_sum(s) * inv_c;
-        float q = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { const float d = v[e] - mean; q += d * d; }
-        // (zero-padded channels, if any, each put mean^2 into the sum)
-        const float rstd = rsqrtf((group16_sum(q) - pad * mean * mean) * inv_c + LN_EPS);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = skip_ln ? v[e] : (v[e] - mean) * rstd * w[e] + b[e];
-      }
-      u32x4 pk = pack8(o);
+      u32x4 pk = ln_pixel8<TIO>(raw[i], w, b, skip_ln, inv_c, pad);
       if (!full && !t.valid(p)) pk = u32x4{0u, 0u, 0u, 0u};
       *reinterpret_cast<u32x4*>(sX + p * LDX + chunk * 8) = pk;
     }
+  }
+}
+
+// The same from rows already in registers (prefetch_tile_rows), which stay intact for a later use.
+template <typename TIO>
+__device__ __forceinline__ void ln_tile_from_rows(const typename Elem<TIO>::Raw* raw, const Tile& t, const float* lnw,
+                                                  const float* lnb, bf16_t* sX, int tid, bool skip_ln, float inv_c,
+                                                  float pad) {
+  const int chunk = tid & 15, prow = tid >> 4;
+  float w[8], b[8];
+  load_param8(lnw ? lnw + chunk * 8 : nullptr, 1.f, w);
+  load_param8(lnb ? lnb + chunk * 8 : nullptr, 0.f, b);
+  const bool full = t.r0 + TM <= t.N;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int p = i * 16 + prow;
+    u32x4 pk = ln_pixel8<TIO>(raw[i], w, b, skip_ln, inv_c, pad);
+    if (!full && !t.valid(p)) pk = u32x4{0u, 0u, 0u, 0u};
+    *reinterpret_cast<u32x4*>(sX + p * LDX + chunk * 8) = pk;
   }
 }
 
@@ -290,11 +318,14 @@ __device__ __forceinline__ void store_tile_f32_pre(const float* sS, const Tile& 
 // LDS store, so the load overlaps the MFMA work on the previous chunk.
 struct WChunkRegs {
   u32x4 r[8];
+  // SWAP23: register row rho receives weight row swap23(rho) (bits 2 and 3 exchanged)
+  template <bool SWAP23 = false>
   __device__ __forceinline__ void load(const bf16_t* gW, int tid) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int idx = tid + 256 * i;
-      r[i] = *reinterpret_cast<const u32x4*>(gW + (idx >> 4) * C + (idx & 15) * 8);
+      const int idx = tid + 256 * i, rho = idx >> 4;
+      const int row = SWAP23 ? ((rho & ~12) | ((rho & 4) << 1) | ((rho & 8) >> 1)) : rho;
+      r[i] = *reinterpret_cast<const u32x4*>(gW + row * C + (idx & 15) * 8);
     }
   }
   __device__ __forceinline__ void store(bf16_t* sW, int tid) const {

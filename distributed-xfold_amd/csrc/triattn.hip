@@ -1,8 +1,9 @@
 // Triangle attention, the fast path: the projection kernel.  It produces, in one
 // pass over the pair tensor, everything the attention core (triattn_core.hip)
-// reads, in the layouts it wants (described in kernels.h): head-major q (scaled),
-// k and sigmoid gate, V transposed with the key order the core's MFMA fragments
-// use, and the fp16 pair bias in the order of the core's MFMA fragments.
+// reads, in the layouts it wants (described in kernels.h): head-major q (scaled)
+// and k, V transposed with the key order the core's MFMA fragments use, and the
+// fp16 pair bias in the order of the core's MFMA fragments.  (The output gate is
+// computed where it is used, by attn_out_kernel.)
 #include "common.h"
 #include "kernels.h"
 #include <type_traits>
@@ -14,8 +15,8 @@ namespace {
 constexpr int H = 4, D = 32;
 
 // ============================================================================
-// projections: LN -> q (scaled), k, sigmoid gate (position-major) and v
-// (channel-major), + pair-bias heads
+// projections: LN -> q (scaled), k (position-major) and v (channel-major),
+// + pair-bias heads
 // ============================================================================
 template <typename TIO>
 __global__ __launch_bounds__(256, 3) void triattn_proj_kernel(TriAttnProjArgs a) {
@@ -30,8 +31,8 @@ __global__ __launch_bounds__(256, 3) void triattn_proj_kernel(TriAttnProjArgs a)
   // which is then the freshest part of q / k / v (measured: 1.4 % of the block)
   const Tile t = make_tile(a.N, a.transpose != 0, true);
   const TIO* x = reinterpret_cast<const TIO*>(a.pair);
-  // Step s = 2 * chunk + half: weight rows 64 half .. + 63 of chunk s / 2 (chunks q, k, v, g as packed in
-  // w_qkvg), four 16-byte pieces per thread; the 32 (padded) pair-bias rows ride in the same registers.
+  // Step s = 2 * chunk + half: weight rows 64 half .. + 63 of chunk s / 2 (chunks q, k, v of w_qkvg),
+  // four 16-byte pieces per thread; the 32 (padded) pair-bias rows ride in the same registers.
   u32x4 wr[4];
   auto wload = [&](int s) {
     const bf16_t* base = a.w_qkvg + (int64_t)s * 64 * C;
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(256, 3) void triattn_proj_kernel(TriAttnProjArgs a)
     // The next weights are requested BEFORE this chunk's results are stored:
     // vector memory operations retire in order, so a load issued behind the
     // stores would make its consumer wait for the stores' round trip to HBM.
-    if (step < 7) wload(step + 1);
+    if (step < 5) wload(step + 1);
     else if (a.n_bias > 0) wload_bias();
     {
       f32x16 acc[2];
@@ -101,7 +102,7 @@ __global__ __launch_bounds__(256, 3) void triattn_proj_kernel(TriAttnProjArgs a)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const float y = acc[nt][4 * g + e];
-              v[e] = chunk == 0 ? y * a.q_scale : (chunk == 3 ? sigmoidf_(y) : y);
+              v[e] = chunk == 0 ? y * a.q_scale : y;
             }
             const int ch = (pairt * 2 + nt) * 32 + 8 * g + 4 * (lane >> 5);
             u32x2 pk;
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(256, 3) void triattn_proj_kernel(TriAttnProjArgs a)
       }
     }
     lds_barrier();  // staging visible; every wave is done with sW
-    if (step < 7) wstore(4);
+    if (step < 5) wstore(4);
     else if (a.n_bias > 0) wstore(2);
     if (pairt == 1) {
       // both halves of the chunk are staged: 128 channels per position go out
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(256, 3) void triattn_proj_kernel(TriAttnProjArgs a)
                 *reinterpret_cast<const u32x4*>(sX + ch * LDX + pc * 8);
         }
       } else {
-        bf16_t* plane = chunk == 0 ? a.q : (chunk == 1 ? a.k : a.g);
+        bf16_t* plane = chunk == 0 ? a.q : a.k;
         const int ck = tid & 15, prow = tid >> 4;
         const int h = ck >> 2, part = ck & 3;
 #pragma unroll
@@ -148,8 +149,6 @@ __global__ __launch_bounds__(256, 3) void triattn_proj_kernel(TriAttnProjArgs a)
   do_step(std::integral_constant<int, 3>{});
   do_step(std::integral_constant<int, 4>{});
   do_step(std::integral_constant<int, 5>{});
-  do_step(std::integral_constant<int, 6>{});
-  do_step(std::integral_constant<int, 7>{});
 
   // pair-bias heads (T form: lane = pixel, rows = heads): bias[h][q][k] with
   // (q, k) the pixel's own (row, col) in the un-transposed pair tensor
@@ -185,11 +184,11 @@ bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 }  // namespace
 
 int launch_triattn_proj(const TriAttnProjArgs& a, hipStream_t stream) {
-  if (a.N <= 0 || !a.pair || !a.w_qkvg || !a.q || !a.k || !a.vt || !a.g) return AF3_ERR_BAD_ARG;
+  if (a.N <= 0 || !a.pair || !a.w_qkvg || !a.q || !a.k || !a.vt) return AF3_ERR_BAD_ARG;
   if (a.ldn < a.N || (a.ldn & 15)) return AF3_ERR_BAD_ARG;
   if (a.n_bias != 0 && (a.n_bias != H || !a.w_bias || !a.bias)) return AF3_ERR_BAD_ARG;
   if (!al16(a.pair) || !al16(a.w_qkvg) || !al16(a.w_bias) || !al16(a.q) || !al16(a.k) || !al16(a.vt) ||
-      !al16(a.g) || !al16(a.bias))
+      !al16(a.bias))
     return AF3_ERR_BAD_ARG;
   const int64_t tiles = (int64_t)a.N * ((a.N + TM - 1) / TM);
   if (tiles > 0x7fffffff) return AF3_ERR_BAD_ARG;

@@ -1,7 +1,7 @@
 // Triangle attention, the flash-attention core (4 heads of 32 channels).
 //
 // Operands (all produced by triattn_proj_kernel, see kernels.h):
-//   Q, K, G : bf16 [b][h][s][32]  (Q pre-multiplied by log2(e)/sqrt(32), G = sigmoid gate)
+//   Q, K    : bf16 [b][h][s][32]  (Q pre-multiplied by log2(e)/sqrt(32))
 //   Vt      : bf16 [b][h][32][ldn], V transposed, ldn = N rounded up to 16, columns
 //             permuted inside every aligned group of 16 (tri_vt_pos) so that the 8 keys one
 //             lane feeds to a P.V MFMA are 16 contiguous bytes
@@ -46,15 +46,6 @@
 #include "common.h"
 #include "kernels.h"
 
-#ifdef AF3_PROF
-#define STAMP(i) do { const long long now_ = __builtin_readcyclecounter(); prof[i] += now_ - tlast; tlast = now_; } while (0)
-#else
-#define STAMP(i) do {} while (0)
-#endif
-#ifndef AF3_WPE
-#define AF3_WPE 2
-#endif
-
 namespace {
 
 constexpr int H = 4, D = 32;
@@ -77,7 +68,7 @@ template <int OFF>
 __device__ __forceinline__ void dma16(const char* gbase, uint32_t voff, const char* dst) {
   const uint32_t lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)dst;
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
-               :: "s"(lds), "v"(voff), "s"(gbase), "n"(OFF) : "memory");
+               :: "s"(lds), "v"(voff), "s"(gbase), "n"(OFF) : "memory", "m0");
 }
 __device__ __forceinline__ bf16x8 lds16(const char* p) { return as_frag(*reinterpret_cast<const u32x4*>(p)); }
 
@@ -122,7 +113,7 @@ __device__ __forceinline__ void scale_in_place(f32x16& o, float f) {
 }
 
 template <int R, bool HAS_BIAS>
-__global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs a) {
+__global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
   // [buffer][row] as separate arrays: a load in flight to one of them provably does not alias
   // a fragment read from another
   __shared__ __attribute__((aligned(1024))) char sK00[TILE_BYTES];
@@ -182,11 +173,10 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
   lds_barrier();
   // A wave takes every fourth key tile; the mask values of eight of its tiles and all rows are
   // requested together (one trip per 32 key tiles, not one per tile and row).  The mask is small
-  // and comes out of L2; Q and the output gates come from memory and are requested right behind
-  // the first batch of mask values: loads return in order, so the mask pass does not wait for
-  // them, and they travel while it, the barriers and the first tiles' loads are under way.
+  // and comes out of L2; Q comes from memory and is requested right behind the first batch of
+  // mask values: loads return in order, so the mask pass does not wait for it, and it travels
+  // while the mask pass, the barriers and the first tiles' loads are under way.
   bf16x8 qf[R][2];
-  u32x2 gw[R][4];  // output gates: used at the very end
   // What a wave finds out about a tile is one byte in LDS, written by all its lanes alike; the
   // workgroup's bit masks of live and of wholly unmasked tiles are ballots over those bytes.
   bool my_any[R];
@@ -207,9 +197,6 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
         const bf16_t* qp = a.q + row * D + 8 * hh;
         qf[r][0] = as_frag(*reinterpret_cast<const u32x4*>(qp));
         qf[r][1] = as_frag(*reinterpret_cast<const u32x4*>(qp + 16));
-        const bf16_t* gp = a.g + row * D + 4 * hh;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) gw[r][g] = *reinterpret_cast<const u32x2*>(gp + 8 * g);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -355,11 +342,6 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
     // the careful route.
     bool allow_fast = true;
     uint64_t bad = 0ull;
-#ifdef AF3_PROF
-    long long prof[6] = {0, 0, 0, 0, 0, 0};
-    long long tlast = __builtin_readcyclecounter();
-    const long long tstart = tlast;
-#endif
     bf16x8 kpre[4];  // R == 2: row 0's K fragments of the next key tile
     u32x4 pp[4];  // probabilities of the previous virtual tile (bf16 B fragments), zero before the first
 
@@ -385,7 +367,6 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       const bf16x8 k10 = pre ? kpre[2] : lds16(kb + 2048 + ka0), k11 = pre ? kpre[3] : lds16(kb + 2048 + ka1);
       bf16x8 af0, af1;
       f32x16 s0, s1;
-      STAMP(4);
       scores(k00, k01, k10, k11, qf[RR], s0, s1);
       if (step3) {
         const uint16_t* mc = sCode + RR * nk64 + tile * KT;
@@ -399,7 +380,6 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       if (!fast) {
       float mx = max32(s0, s1);
       mx = fmaxf(mx, half_swap(xaddr, mx));
-      STAMP(5);
       const float mnew = fmaxf(mrel[RR], mx);
       // (lanes of queries past the end have no say: in a partly filled block they see bias values nobody wrote)
       const bool want = qw < N && (mx > T_HI || (mnew < T_LO && mnew > LIVE_MIN));
@@ -439,7 +419,6 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       }
       }
       float linc = 0.f;
-      STAMP(2);
       // From here to the end: one basic block in a fixed order.  Each of the four P.V MFMAs of the
       // previous virtual tile is issued in front of eight exponentials of this one (the matrix
       // unit works while the wave goes on issuing vector instructions; another wave's would not
@@ -495,7 +474,6 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
         // running maximum, the same in both half-waves, all the careful route's lower guard needs
         mrel[RR] = fmaxf(mrel[RR], -42.f);
       }
-      STAMP(3);
     };
     // the tail of the pipeline: the last virtual tile's probabilities
     auto drain = [&](const char* vb) {
@@ -564,9 +542,7 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
       using P0 = std::integral_constant<int, PH>;
       if (R == 2) {
         iter(P0{}, std::integral_constant<int, 0>{}, t_cur);
-        STAMP(0);
         dma_barrier();
-        STAMP(1);
         dma_bias(t_n2, PH == 0 ? sBias0 : sBias1);
         dma_k(t_n1, 1, KBUF(PH ^ 1, 1));
         dma_k(t_n2, 0, KBUF(PH, 0));
@@ -574,9 +550,7 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
         dma_v(t_n1, 1, VBUF(PH ^ 1, 1));
         iter(P0{}, std::integral_constant<int, R - 1>{}, t_cur);
       } else {
-        STAMP(0);
         dma_barrier();
-        STAMP(1);
         dma_bias(t_n2, PH == 0 ? sBias0 : sBias1);
         dma_k(t_n1, 0, KBUF(PH ^ 1, 0));
         dma_v(t_cur, 0, VBUF(PH, 0));
@@ -602,14 +576,6 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
     lds_barrier();  // also: every wave is done with the K / V^T tiles before a second pass loads over them
     if (__builtin_amdgcn_readfirstlane(sRedo) == 0u) break;
     }
-#ifdef AF3_PROF
-    if (lane == 0) {
-      long long* dst = reinterpret_cast<long long*>(a.og + ((int64_t)brow[0] * N + q0 + wave * 32) * 128 + h * D);
-      dst[0] = prof[0]; dst[1] = prof[1]; dst[2] = prof[2]; dst[3] = prof[3];
-      dst[4] = __builtin_readcyclecounter() - tstart; dst[5] = prof[4]; dst[6] = prof[5];
-    }
-    return;
-#endif
   }
 
   // a query's keys are split over the two half-waves
@@ -663,8 +629,8 @@ __global__ __launch_bounds__(256, AF3_WPE) void triattn_flash_kernel(TriAttnArgs
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       u32x2 w;
-      w.x = pack2bf(o[r][4 * g] * inv * bflo(gw[r][g].x), o[r][4 * g + 1] * inv * bfhi(gw[r][g].x));
-      w.y = pack2bf(o[r][4 * g + 2] * inv * bflo(gw[r][g].y), o[r][4 * g + 3] * inv * bfhi(gw[r][g].y));
+      w.x = pack2bf(o[r][4 * g] * inv, o[r][4 * g + 1] * inv);
+      w.y = pack2bf(o[r][4 * g + 2] * inv, o[r][4 * g + 3] * inv);
       *reinterpret_cast<u32x2*>(op + 8 * g) = w;
     }
   }
@@ -677,9 +643,9 @@ bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 }  // namespace
 
 int launch_triattn_flash(const TriAttnArgs& a, hipStream_t stream) {
-  if (!a.q || !a.k || !a.vt || !a.g || !a.og || a.N <= 0 || a.N > 8192) return AF3_ERR_BAD_ARG;
+  if (!a.q || !a.k || !a.vt || !a.og || a.N <= 0 || a.N > 8192) return AF3_ERR_BAD_ARG;
   if (a.ldn < a.N || (a.ldn & 15)) return AF3_ERR_BAD_ARG;
-  if (!al16(a.q) || !al16(a.k) || !al16(a.vt) || !al16(a.g) || !al16(a.og) || !al16(a.bias)) return AF3_ERR_BAD_ARG;
+  if (!al16(a.q) || !al16(a.k) || !al16(a.vt) || !al16(a.og) || !al16(a.bias)) return AF3_ERR_BAD_ARG;
   const int QT = (a.N + QW - 1) / QW;
   const int nkt = (a.N + KT - 1) / KT;
   // Two rows per wave once that still leaves every CU several workgroups, one row below that

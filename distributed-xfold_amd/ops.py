@@ -617,11 +617,12 @@ def pack_vt(vt):
     return full.view(n, 4, 32, ld // 16, 4, 4)[..., [0, 2, 1, 3], :].reshape(n, 4, 32, ld).contiguous()
 
 
-def grid_attention_core(q, k, vt, g, pair_bias, mask, out=None):
+def grid_attention_core(q, k, vt, pair_bias, mask, out=None):
     """The flash-attention stage of the triangle attention on projected, head-major
-    operands in base-2 form: q, k, g bf16 [N, 4, N, 32] (q and the bias
-    pre-multiplied by log2(e); g = sigmoid gate), vt from pack_vt(), pair_bias
-    from pack_pair_bias() or None.  Returns the gated output [N*N, 128] bf16."""
+    operands in base-2 form: q, k bf16 [N, 4, N, 32] (q and the bias
+    pre-multiplied by log2(e)), vt from pack_vt(), pair_bias from
+    pack_pair_bias() or None.  Returns softmax(q k^T + bias) v as [N*N, 128]
+    bf16 (the output gate belongs to the operator's last kernel)."""
     lib = _L.load()
     _gpu(q, "q", torch.bfloat16)
     if q.dim() != 4 or q.shape[1] != 4 or q.shape[3] != 32 or q.shape[0] != q.shape[2]:
@@ -629,14 +630,13 @@ def grid_attention_core(q, k, vt, g, pair_bias, mask, out=None):
     n = q.shape[0]
     ld = (n + 15) // 16 * 16
     _gpu(k, "k", torch.bfloat16, q.shape)
-    _gpu(g, "g", torch.bfloat16, q.shape)
     _gpu(vt, "vt", torch.bfloat16, (n, 4, 32, ld))
     if pair_bias is not None:
         _gpu(pair_bias, "pair_bias", torch.float16, (4, (n + 31) // 32, (n + 63) // 64, 4, 32, 16))
     maskf = _mask_f32(mask, (n, n), "mask")
     if out is None:
         out = torch.empty((n * n, 128), dtype=torch.bfloat16, device=q.device)
-    rc = lib.af3_grid_attention_core_forward(_p(q), _p(k), _p(vt), _p(g), _p(pair_bias), _p(maskf), _p(out), n,
+    rc = lib.af3_grid_attention_core_forward(_p(q), _p(k), _p(vt), _p(pair_bias), _p(maskf), _p(out), n,
                                              _stream(q.device))
     _L.check(rc, "af3_grid_attention_core_forward")
     return out

@@ -43,6 +43,13 @@ extern "C" {
 
 typedef void* af3_stream_t; /* a hipStream_t */
 
+/* Version of this interface; af3_abi_version() returns the value the library
+ * was built with.  It changes whenever the meaning or layout of an argument of
+ * an existing entry point changes, so a caller that packed operands for another
+ * version can tell.  2: af3_grid_attention_core_forward takes no gate and
+ * leaves the normalised, ungated output; its pair bias is fp16 in fragment
+ * order and vt has its quads swapped (version 1 took a bf16 bias and a gate). */
+#define AF3_ABI_VERSION 2
 int af3_abi_version(void);
 const char* af3_error_string(int code);
 
@@ -411,7 +418,7 @@ int af3_linear_forward(
  *   attention (csrc/grid_self_attention_bf16.h:226-481) on already projected
  *   operands, head-major, in base-2 form (4 heads of 32, ld = n_token rounded
  *   up to 16):
- *     q  bf16 [b][h][s][32] = query * log2(e)/sqrt(32);  k, g bf16 [b][h][s][32] (g = sigmoid gate);
+ *     q  bf16 [b][h][s][32] = query * log2(e)/sqrt(32);  k bf16 [b][h][s][32];
  *     vt bf16 [b][h][32][ld] = value transposed, key k of a row stored at column
  *       (k & ~12) | ((k & 8) >> 1) | ((k & 4) << 1) (inside every aligned group of 16 keys
  *       the two middle quads are swapped), columns of keys >= n_token zero;
@@ -421,12 +428,13 @@ int af3_linear_forward(
  *       (per head, 32-query block and 64-key tile: four contiguous 1 KB runs, each
  *       the B operand of one identity-matrix MFMA that adds the bias to the logits);
  *   key mask [N][N] fp32 0/1 or NULL;
- *   og [(b*N + s)][128] = gate * softmax(q k^T + bias) v.
+ *   og [(b*N + s)][128] = softmax(q k^T + bias) v  (the output gate, sigmoid(LN(x) Wg^T), is
+ *   applied by the operator's last kernel together with the output projection).
  */
 int af3_triangle_contraction_forward(
     const uint16_t* a, const uint16_t* b, uint16_t* t, int64_t n_token, af3_stream_t stream);
 int af3_grid_attention_core_forward(
-    const uint16_t* q, const uint16_t* k, const uint16_t* vt, const uint16_t* g,
+    const uint16_t* q, const uint16_t* k, const uint16_t* vt,
     const uint16_t* pair_bias, const float* mask, uint16_t* og, int64_t n_token, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------

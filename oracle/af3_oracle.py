@@ -252,7 +252,8 @@ def grid_self_attention(pair, mask, p: Params, num_head: int, transpose: bool,
     key_mask = mask.to(torch.bool)[:, None, None, :]
     avg = dot_product_attention(q, k, v, mask=key_mask, bias=nb[None])
     avg = avg.permute(0, 2, 1, 3).reshape(n_row, n_key, c)
-    avg = _r(avg * _r(torch.sigmoid(linear(x, p["gating_query.weight"]))))
+    # (emulation: the attention output is stored in bf16, the gate meets it in fp32)
+    avg = _r(_r(avg) * torch.sigmoid(linear(x, p["gating_query.weight"])))
     out = linear(avg, p["output_projection.weight"])
     if transpose:
         out = out.permute(1, 0, 2)

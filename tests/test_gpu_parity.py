@@ -444,7 +444,6 @@ def _attention_core_case(gpu_pkg, n, tiles, scale=0.7, bias_shift=0.0, seed=None
     d = dev()
     qkvg = rb(torch.randn(n, n, 4, 4, 32, generator=g) * scale)     # [b, s, (q k v g), h, d]
     qkvg[:, :, 2] = rb(qkvg[:, :, 2] * (0.7 / scale))
-    qkvg[:, :, 3] = torch.sigmoid(qkvg[:, :, 3] * (0.7 / scale)).bfloat16().float()
     # the kernel-level entry point takes the bias in fp16: the reference sees the same values
     bias = (rb(torch.randn(4, n, n, generator=g)) + bias_shift).half().float()
     mask = (torch.rand(n, n, generator=g) > 0.2).float()
@@ -468,23 +467,23 @@ def _attention_core_case(gpu_pkg, n, tiles, scale=0.7, bias_shift=0.0, seed=None
     hm = lambda i: qkvg[:, :, i].permute(0, 2, 1, 3).contiguous()       # [b, h, s, d]
     t = lambda x: x.to(d).bfloat16()
     og = gpu_pkg.ops.grid_attention_core(t(hm(0)), t(hm(1)), gpu_pkg.ops.pack_vt(t(hm(2).transpose(-1, -2))),
-                                         t(hm(3)), gpu_pkg.ops.pack_pair_bias(bias.to(d)), mask.to(d))
+                                         gpu_pkg.ops.pack_pair_bias(bias.to(d)), mask.to(d))
     og = og.view(n, n, 4, 32).float()
     # the reference on the GPU in float64, a block of rows at a time
-    q, k, v, gt = (qkvg[:, :, i].permute(0, 2, 1, 3).to(d).double() for i in range(4))   # [b, h, s, d]
+    q, k, v = (qkvg[:, :, i].permute(0, 2, 1, 3).to(d).double() for i in range(3))   # [b, h, s, d]
     bd, md = bias.to(d).double(), mask.to(d)
     want = torch.empty(n, n, 4, 32, dtype=torch.float64, device=d)
     for b0 in range(0, n, 32):
         sl = slice(b0, min(n, b0 + 32))
         logits = (q[sl] @ k[sl].transpose(-1, -2) + bd[None]) / log2e
         logits = logits.masked_fill(md[sl][:, None, None, :] == 0, -1e9)
-        want[sl] = ((torch.softmax(logits, -1) @ v[sl]) * gt[sl]).permute(0, 2, 1, 3)
+        want[sl] = (torch.softmax(logits, -1) @ v[sl]).permute(0, 2, 1, 3)
     return og, want
 
 
 @pytest.mark.parametrize("n,tiles", [(40, False), (200, False), (200, True), (330, True), (515, True), (576, False)])
 def test_kernel_level_attention_core(gpu_pkg, n, tiles):
-    """Base-2 operands in, gate * softmax(q k^T + bias, masked) v out.  `tiles`:
+    """Base-2 operands in, softmax(q k^T + bias, masked) v out.  `tiles`:
     whole 64-key tiles masked (the kernel leaves such tiles out for rows that
     have an unmasked key elsewhere, which must not change a bit of the result).
     From 512 tokens on a wave takes two rows at a time (515: the last row has no partner)."""
