@@ -193,8 +193,8 @@ int launch_flash_attention(const FlashArgs& a, hipStream_t stream);
 //            the attention core adds it to the scores on the matrix unit, S^T += I * bias^T with an
 //            fp16 identity, and wants per (head, 32-query block, 64-key tile) the four B fragments
 //            of that product as four contiguous 1 KB runs: run (k % 64) / 16, then [q % 32][k % 16].
-//            fp16 rather than fp32: at 8 MFMAs per key tile the kernel is paced by the bytes the
-//            CU's vector memory path can take, and the bias is most of them; fp16's 11 significant
+//            fp16 rather than fp32: the bias is half of what the attention core pulls in from L2
+//            per key tile, and that traffic is a sixth of its run time; fp16's 11 significant
 //            bits put its rounding (2^-12 of a logit) below that of the bf16 probabilities (2^-9).
 //            Entries whose key is >= N are zero; query rows >= N of the last block are unused.
 __host__ __device__ inline int64_t tri_ldn(int64_t n) { return (n + 15) / 16 * 16; }

@@ -392,24 +392,16 @@ __global__ __launch_bounds__(256, 2) void attn_out_kernel(AttnOutArgs a) {
   float* sS = reinterpret_cast<float*>(smem);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const Tile t = make_tile(a.N, a.transpose != 0);  // where the result lands in the pair tensor
-  // Loads are unconditional (rows past the end re-read a valid one and are zeroed /
-  // skipped later).  Up front: the pair rows (gate input and residual) and the gate
-  // weights; the attention output follows once the gate's MFMAs are issued (its 32
-  // registers would not fit beside them).  The bf16 stream keeps its pair rows in
-  // registers for the residual; the fp32 stream (twice the registers) reads them a
-  // second time at the end.
-#ifndef X_KEEP_ROWS
-#define X_KEEP_ROWS false
-#endif
-  constexpr bool KEEP_ROWS = X_KEEP_ROWS;
+  // Loads are unconditional (rows past the end re-read a valid one and are zeroed / skipped later).
+  // The attention output is requested once the gate's MFMAs are issued (its 32 registers would not
+  // fit beside them), and the pair rows are read a second time, out of the cache, for the residual:
+  // keeping them in registers from the LayerNorm on costs more (spills, or a bf16-rounded gate)
+  // than the second read (measured).
   const TIO* x = reinterpret_cast<const TIO*>(a.pair);
   const int ck = tid & 15, prow = tid >> 4;
-  typename Elem<TIO>::Raw res[KEEP_ROWS ? 8 : 1];
-  if (KEEP_ROWS) prefetch_tile_rows<TIO>(x, t, tid, res);
   WChunkRegs wr;
   wr.load<true>(a.w_gate, tid);
-  if (KEEP_ROWS) ln_tile_from_rows<TIO>(res, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0, a.lw.inv_c, a.lw.pad);
-  else load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0, a.lw.inv_c, a.lw.pad);
+  load_ln_tile<TIO>(x, t, a.ln_w, a.ln_b, sX, tid, a.skip_ln != 0, a.lw.inv_c, a.lw.pad);
   wr.store(sW, tid);
   lds_barrier();
   bf16x8 xf[8];
@@ -451,8 +443,7 @@ __global__ __launch_bounds__(256, 2) void attn_out_kernel(AttnOutArgs a) {
   lds_barrier();
   stage_t_f32(acc, sS, wave, lane);
   lds_barrier();
-  if (KEEP_ROWS) store_tile_f32_pre<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), res, a.residual != 0, tid);
-  else store_tile_f32<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), a.residual ? x : nullptr, tid);
+  store_tile_f32<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), a.residual ? x : nullptr, tid);
 }
 
 // ============================================================================

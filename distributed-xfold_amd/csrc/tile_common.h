@@ -131,25 +131,6 @@ __device__ __forceinline__ void load_ln_tile(const TIO* x, const Tile& t, const 
   }
 }
 
-// The same from rows already in registers (prefetch_tile_rows), which stay intact for a later use.
-template <typename TIO>
-__device__ __forceinline__ void ln_tile_from_rows(const typename Elem<TIO>::Raw* raw, const Tile& t, const float* lnw,
-                                                  const float* lnb, bf16_t* sX, int tid, bool skip_ln, float inv_c,
-                                                  float pad) {
-  const int chunk = tid & 15, prow = tid >> 4;
-  float w[8], b[8];
-  load_param8(lnw ? lnw + chunk * 8 : nullptr, 1.f, w);
-  load_param8(lnb ? lnb + chunk * 8 : nullptr, 0.f, b);
-  const bool full = t.r0 + TM <= t.N;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int p = i * 16 + prow;
-    u32x4 pk = ln_pixel8<TIO>(raw[i], w, b, skip_ln, inv_c, pad);
-    if (!full && !t.valid(p)) pk = u32x4{0u, 0u, 0u, 0u};
-    *reinterpret_cast<u32x4*>(sX + p * LDX + chunk * 8) = pk;
-  }
-}
-
 // In-place LayerNorm of the rows of sX (bf16 in LDS), same thread mapping.
 __device__ __forceinline__ void ln_inplace_tile(bf16_t* sX, const float* lnw, const float* lnb, int tid) {
   const int chunk = tid & 15, prow = tid >> 4;
@@ -284,35 +265,6 @@ __device__ __forceinline__ void store_tile_f32(const float* sS, const Tile& t, T
   }
 }
 
-
-// The same with the residual rows fetched by the caller ahead of time
-// (prefetch_tile_rows at kernel entry, so their latency hides behind the MFMAs).
-template <typename TIO>
-__device__ __forceinline__ void prefetch_tile_rows(const TIO* src, const Tile& t, int tid, typename Elem<TIO>::Raw* raw) {
-  const int chunk = tid & 15, prow = tid >> 4;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int p = i * 16 + prow;
-    raw[i] = Elem<TIO>::load_raw(src + t.pix(t.valid(p) ? p : 0) * C + chunk * 8);
-  }
-}
-template <typename TIO>
-__device__ __forceinline__ void store_tile_f32_pre(const float* sS, const Tile& t, TIO* out,
-                                                   const typename Elem<TIO>::Raw* raw, bool add, int tid) {
-  const int chunk = tid & 15, prow = tid >> 4;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int p = i * 16 + prow;
-    float v[8], rr[8];
-    const f32x4 a = *reinterpret_cast<const f32x4*>(sS + p * LDS_F + chunk * 8);
-    const f32x4 b = *reinterpret_cast<const f32x4*>(sS + p * LDS_F + chunk * 8 + 4);
-    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-    Elem<TIO>::unpack_raw(raw[i], rr);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] += add ? rr[e] : 0.f;
-    if (t.valid(p)) Elem<TIO>::store8(out + t.pix(p) * C + chunk * 8, v);
-  }
-}
 
 // 128 x 128 bf16 weight chunk held in registers between a global load and the
 // LDS store, so the load overlaps the MFMA work on the previous chunk.

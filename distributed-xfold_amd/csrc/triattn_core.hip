@@ -12,13 +12,18 @@
 // for 8 cycles, any other vector instruction for 4-5, a 32x32x16 MFMA for about 16 of the 32
 // cycles it takes in the matrix unit - and vector work of OTHER waves does not issue while a
 // wave has an MFMA waiting for the unit.  So vector and matrix work overlap only inside one
-// wave's own instruction stream, and the kernel is built around that:
+// wave's own instruction stream.  The other cost is what a workgroup pulls in from L2 per key
+// tile: with every load taken out of the key-tile loop (operands reused, results wrong) the
+// kernel runs 30 % faster, 17 % of which remain when the same loads all hit the CU's own
+// cache, i.e. are the loads into LDS as such, the rest is the L2 traffic (8 KB of K / V^T per
+// row and 4 KB of bias per wave and key tile: 28 GB per launch at 1536 tokens).  The kernel
+// is built around both:
 //   * one wave = 32 queries of R rows b; lane = one query; S^T = K Q^T so that the softmax
 //     reductions are per lane.  The pair bias enters on the matrix unit as well, S^T += I *
 //     bias^T with an fp16 identity; its fragments do not depend on the row, so the R rows of a
-//     wave share one load of them.  (With the fp32 bias as the accumulators' initial value the
-//     kernel ran 35 % slower than without any bias: at this rate the bytes the bias brings
-//     through the CU's vector memory path are what paces it; hence fp16 and two rows per wave.)
+//     wave share one load of them, straight into registers.  (With the fp32 bias as the
+//     accumulators' initial value the kernel ran 35 % slower than without any bias: the bytes
+//     the bias brings in from L2 are half of all it loads; hence fp16 and two rows per wave.)
 //   * the key mask rides in the product as a third k-step (K side 0 / -1e9 / -inf, Q side 1.0),
 //     and so does the softmax's running base: the Q side of the next slot holds -base, so the
 //     accumulator comes out as s - base and exp2 takes it as it is.  `base` only moves when a
@@ -33,10 +38,10 @@
 //     V^T fragment read from LDS one group ahead.  Row sums are taken from the bf16
 //     probabilities by v_dot2c_f32_bf16 against a pair of ones (per lane, i.e. per half of the
 //     keys; the halves are added once at the end).
-//   * K and V^T tiles, and the bias tile of the wave, go from global memory straight into LDS
-//     (global_load_lds_dwordx4: no staging registers, no LDS store instructions), K / V^T
-//     double-buffered per row with one barrier per key tile, the bias one key tile ahead;
-//     unpadded rows with XOR-permuted 16-byte chunks keep the fragment reads conflict-free.
+//   * K and V^T tiles go from global memory straight into LDS (global_load_lds_dwordx4: no
+//     staging registers, no LDS store instructions), double-buffered per row with one barrier
+//     per key tile; unpadded rows with XOR-permuted 16-byte chunks keep the fragment reads
+//     conflict-free.
 // Key tiles whose 64 keys are masked in every row of the wave are left out (their
 // probabilities are exactly zero); a row whose keys are ALL masked gets the reference's exact
 // answer, the mean of V, directly.
@@ -72,9 +77,14 @@ __device__ __forceinline__ void dma16(const char* gbase, uint32_t voff, const ch
 }
 __device__ __forceinline__ bf16x8 lds16(const char* p) { return as_frag(*reinterpret_cast<const u32x4*>(p)); }
 
-// workgroup barrier that also waits for this wave's loads into LDS
+// Workgroup barrier that also waits for this wave's loads, those into LDS and the ordinary ones
+// (the bias registers).  The wait is a builtin so that the compiler sees it: it then knows the
+// registers have landed and puts no wait of its own in front of their use, where it would also
+// wait for the loads into LDS issued since.
 __device__ __forceinline__ void dma_barrier() {
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
 }
 
 __device__ __forceinline__ float max32(const f32x16& a, const f32x16& b) {
@@ -124,8 +134,6 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
   __shared__ __attribute__((aligned(1024))) char sV01[R > 1 ? TILE_BYTES : 16];
   __shared__ __attribute__((aligned(1024))) char sV10[TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) char sV11[R > 1 ? TILE_BYTES : 16];
-  __shared__ __attribute__((aligned(1024))) char sBias0[HAS_BIAS ? 4 * 4096 : 16];  // a bias tile per wave, by key tile parity
-  __shared__ __attribute__((aligned(1024))) char sBias1[HAS_BIAS ? 4 * 4096 : 16];
   __shared__ uint32_t sLive[R];      // per row: some key is unmasked
   __shared__ uint8_t sFlag[R * 64];  // per row and key tile (the first 64): 1 = some key unmasked, 3 = all 64 of them
   __shared__ float sMean[D];
@@ -285,29 +293,28 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
       const int col = min(tile, nkt - 1) * KT + dv_col;  // columns past ldn: any finite data will do (P is zero there)
       dma16<0>(vglob[r], (uint32_t)(dv_row * ldn + (col < ldn ? col : 0)) * 2u, buf + wave * 1024);
     };
-    // bias tile of this wave's 32-query block: eight 1 KB runs, lane l takes bytes 16 l of each
+    // bias tiles of this wave's 32-query block: 4 KB per key tile
     const int wave_blk = q0 + wave * 32 < N ? (q0 >> 5) + wave : 0;
     const char* bbase =
         HAS_BIAS ? reinterpret_cast<const char*>(a.bias + tri_bias_offset(N, h, wave_blk * 32, 0)) : nullptr;
-    // The bias tile (four 1 KB fp16 fragments) of key tile t + 2 is fetched into the wave's own
-    // 4 KB of LDS (one of two buffers, by key tile parity) right after tile t's barrier, with the
-    // K / V^T tiles: two rows' worth of time for the load to land.  While the last row of tile
-    // t computes its exponentials, tile t + 1's fragments are read from LDS and turned into fp32
-    // on the matrix unit, bt = I * bias^T with an fp16 identity: the initial value of the score
-    // accumulators of every row of tile t + 1 (four MFMAs per key tile, each issued between two
-    // groups of exponentials).
+    // The bias tile of key tile t + 1 (four 1 KB fp16 fragments; fragment i = 2 u + st: keys
+    // 32 u + 16 st + 8 hh .. + 8 of this lane's query, bytes 32 j + 16 hh of run i) is only ever
+    // read by this wave, so it goes from memory straight into registers, requested when tile t
+    // begins.  The wait that the barrier in the middle of tile t needs anyway covers it.  While
+    // the last row of tile t computes its exponentials the fragments are turned into fp32 on
+    // the matrix unit, bt = I * bias^T with an fp16 identity: the initial value of the score
+    // accumulators of every row of tile t + 1 (four MFMAs per key tile, each issued between
+    // two groups of exponentials).  (Staged through LDS like K and V^T, by loads into LDS two
+    // tiles ahead, the same kernel ran 3.5 % slower: a load into LDS costs the wave more than
+    // a load into registers, and the fragments cost an LDS read each on top.)
     f32x16 bt[2];
-    auto dma_bias = [&](int tile, char* buf) {
+    u32x4 bnext[4];
+    auto load_bias = [&](int tile) {
       if (!HAS_BIAS) return;
-      const char* p = bbase + (size_t)min(tile, nkt - 1) * 4096u;
-      char* dst = buf + wave * 4096;
-      dma16<0>(p, lane * 16u, dst);
-      dma16<1024>(p, lane * 16u, dst);
-      dma16<2048>(p, lane * 16u, dst);
-      dma16<3072>(p, lane * 16u, dst);
+      const char* p = bbase + (size_t)min(tile, nkt - 1) * 4096u + (j * 32 + hh * 16);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bnext[i] = *reinterpret_cast<const u32x4*>(p + 1024 * i);
     };
-    // fragment i = 2 u + st: keys 32 u + 16 st + 8 hh .. + 8 of this lane's query, bytes (32 j + 16 hh) of run i
-    const int boff = wave * 4096 + j * 32 + hh * 16;
     // Identity fragments (fp16): A-fragment of k-step st: lane (row i = j, half hh) holds
     // I[i][16 st + 8 hh + e], e = 0..7: a single 1.0 where 16 st + 8 hh + e == i.
     f16x8 idf[2];
@@ -335,13 +342,16 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
     float pend_alpha = 1.f;  // R == 1: a rescaling of O and l that waits for the tile in flight
     bool pend = false;
     // Tiles of 64 unmasked keys take their exponentials without looking at the tile's maximum
-    // first ("fast").  Every lane of such a tile has 32 live keys, so the sum of what it got says
-    // afterwards where the scores lay: a sum that is not below 2^60 (an overflow included) means
-    // scores far above the base, a row total below 2^-30 scores far below it.  Either is rare,
-    // is only recorded here, and makes the whole workgroup repeat its rows with every tile on
-    // the careful route.
+    // first ("fast").  Every lane of such a tile has 32 live keys, so the sums of what it got say
+    // afterwards where the scores lay: a tile sum that is not below 2^60 (an overflow included)
+    // means scores far above the base, a row total below 2^-30 scores far below it.  Per tile
+    // only the largest tile sum is kept (one instruction); both conditions are looked at once,
+    // when the row is through.  Either is rare and makes the whole workgroup repeat its rows
+    // with every tile on the careful route.
     bool allow_fast = true;
     uint64_t bad = 0ull;
+    float lmax[R];      // largest sum of one fast tile
+    bool used_fast[R];  // this wave took some tile of the row the fast way
     bf16x8 kpre[4];  // R == 2: row 0's K fragments of the next key tile
     u32x4 pp[4];  // probabilities of the previous virtual tile (bf16 B fragments), zero before the first
 
@@ -426,9 +436,8 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
       bf16x8 vf = lds16(vb + va[0]);
       u32x4 bfr[4];  // the next key tile's bias fragments (the last row of this one fetches them)
       if (HAS_BIAS && RR == R - 1) {
-        const char* bsrc = (PH == 0 ? sBias1 : sBias0) + boff;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) bfr[i] = *reinterpret_cast<const u32x4*>(bsrc + 1024 * i);
+        for (int i = 0; i < 4; ++i) bfr[i] = bnext[i];  // (the registers are free for the next request)
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -467,12 +476,12 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
       }
       lrun[RR] += linc;
       if (fast) {
-        // (lanes of queries past the end work on clamped operands and, in a partly filled bias block, on
-        // bias values nobody wrote: they have no say)
-        bad |= __ballot(qw < N && (!(linc < 0x1p60f) || lrun[RR] < 0x1p-30f));
-        // if that was fine, the row total is at least 2^-30 over at most 4096 keys: a lower bound of the
-        // running maximum, the same in both half-waves, all the careful route's lower guard needs
+        lmax[RR] = fmaxf(lmax[RR], linc);
+        // If the row passes its check at the end, its total is at least 2^-30 over at most 4096
+        // keys: a lower bound of the running maximum, all the careful route's lower guard needs
+        // (if it does not, the rows are repeated and what a careful tile decided meanwhile is void).
         mrel[RR] = fmaxf(mrel[RR], -42.f);
+        used_fast[RR] = true;
       }
     };
     // the tail of the pipeline: the last virtual tile's probabilities
@@ -501,12 +510,13 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
       mrel[r] = -__builtin_huge_valf();
       qm[r].x = hh == 0 ? (BF16_ONE | 0x80000000u) : 0u;
       based[r] = false;
+      lmax[r] = 0.f;
+      used_fast[r] = false;
     }
     int t_cur = pop(), t_n1 = pop(), t_n2 = pop();
     // the buffer the first virtual tile reads its "previous" V^T from must hold finite data
     *reinterpret_cast<u32x4*>(VBUF(1, R - 1) + tid * 16) = u32x4{0u, 0u, 0u, 0u};
     // the first tiles' loads into LDS and the first bias tile's ordinary loads travel together
-    dma_bias(t_n1, sBias1);
     dma_k(t_cur, 0, KBUF(0, 0));
     if (R == 2) {
       dma_k(t_cur, 1, KBUF(0, 1));
@@ -541,9 +551,9 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
       constexpr int PH = decltype(PHc)::value;
       using P0 = std::integral_constant<int, PH>;
       if (R == 2) {
+        load_bias(t_n1);
         iter(P0{}, std::integral_constant<int, 0>{}, t_cur);
         dma_barrier();
-        dma_bias(t_n2, PH == 0 ? sBias0 : sBias1);
         dma_k(t_n1, 1, KBUF(PH ^ 1, 1));
         dma_k(t_n2, 0, KBUF(PH, 0));
         dma_v(t_n1, 0, VBUF(PH ^ 1, 0));
@@ -551,7 +561,7 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
         iter(P0{}, std::integral_constant<int, R - 1>{}, t_cur);
       } else {
         dma_barrier();
-        dma_bias(t_n2, PH == 0 ? sBias0 : sBias1);
+        load_bias(t_n1);  // R == 1: requested behind the barrier, used at the end of this virtual tile
         dma_k(t_n1, 0, KBUF(PH ^ 1, 0));
         dma_v(t_cur, 0, VBUF(PH, 0));
         iter(P0{}, std::integral_constant<int, 0>{}, t_cur);
@@ -572,6 +582,14 @@ __global__ __launch_bounds__(256, 2) void triattn_flash_kernel(TriAttnArgs a) {
     dma_barrier();  // every load into LDS has landed (none is in flight when the workgroup ends)
     drain(last_ph == 0 ? VBUF(0, R - 1) : VBUF(1, R - 1));
     if (pass == 1) break;
+    // (lanes of queries past the end work on clamped operands and, in a partly filled bias block, on
+    // bias values nobody wrote: they have no say)
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (!used_fast[r] || dead[r]) continue;
+      const float lt = lrun[r] + half_swap(xaddr, lrun[r]);
+      bad |= __ballot(qw < N && (!(lmax[r] < 0x1p60f) || lt < 0x1p-30f));
+    }
     if (bad != 0ull && lane == 0) sRedo = 1u;
     lds_barrier();  // also: every wave is done with the K / V^T tiles before a second pass loads over them
     if (__builtin_amdgcn_readfirstlane(sRedo) == 0u) break;
@@ -657,16 +675,16 @@ int launch_triattn_flash(const TriAttnArgs& a, hipStream_t stream) {
     return e ? atoi(e) : 0;
   }();
   if (forced == 1 || forced == 2) R = forced;
-  // static LDS: K / V buffers, the staged bias (32 KB), small arrays; dynamic: the mask codes.
-  // Two workgroups must fit a CU's 160 KB.
-  const size_t stat2 = 8 * TILE_BYTES + (a.bias ? 8 * 4096 : 32) + 512;
+  // static LDS: K / V buffers, small arrays; dynamic: the mask codes.  Two workgroups must fit a
+  // CU's 160 KB.
+  const size_t stat2 = 8 * TILE_BYTES + 512;
   if (R == 2 && stat2 + 2 * (size_t)nkt * KT * sizeof(uint16_t) > 80 * 1024) R = 1;
   const int NG = (a.N + R - 1) / R;
   const int64_t blocks = ((int64_t)H * NG + 7) / 8 * 8 * QT;
   if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
   const size_t dyn = (size_t)R * nkt * KT * sizeof(uint16_t);
   const dim3 grid((unsigned)blocks), block(256);
-  const size_t stat = (R == 2 ? 8 : 4) * TILE_BYTES + (a.bias ? 8 * 4096 : 32) + 512;
+  const size_t stat = (R == 2 ? 8 : 4) * TILE_BYTES + 512;
   auto launch = [&](void (*kernel)(TriAttnArgs)) {
     // more than 64 KB of LDS per workgroup in all (static + dynamic) has to be asked for
     // (a per-function, per-device setting of the runtime: no allocation, no synchronisation)
