@@ -9,7 +9,9 @@ last 10% of the tokens masked as padding.  Prints ONE JSON line:
 
   metric / value   Pairformer ms per block (lower is better)
   roofline         the dominant kernel (by time per block) against the MI355X
-                   dense bf16 MFMA peak, its launch timed live with HIP events
+                   dense bf16 MFMA peak, its launch timed live with HIP events on
+                   all-ones masks (nothing skipped); `padded` inside it: the same
+                   launch under the workload's padding
   cpu_baseline     the CPU oracle (eager PyTorch restatement of the reference
                    formulas, fp32) timed on this host's cores on a bounded
                    sample, scaled to the metric's unit
@@ -32,10 +34,41 @@ if ROOT not in sys.path:
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the dominant kernel from rocprofv3 counters (FETCH_SIZE x 2.000 +
-# WRITE_SIZE x 1.000, scaled by a plain elementwise kernel of known size in the same run, see
-# --calibrate); measured offline, per N_token: profiles/pairformer_block_n768_bf16_hbm_traffic.txt
-MEASURED_TRAFFIC_BYTES = {("triattn_flash_kernel", 768): 839.9e6, ("contract_kernel", 768): 508.5e6}
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def measured_traffic_bytes(kernel, n):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 counter summary of this workload
+    (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors from a plain elementwise kernel of known size
+    in the same profiler run, see --calibrate): column `total MB` of
+    profiles/pairformer_block_n<N>_bf16_hbm_traffic.txt.  None when there is no summary for this size."""
+    try:
+        with open(os.path.join(PROFILES, f"pairformer_block_n{n}_bf16_hbm_traffic.txt")) as f:
+            for line in f:
+                cols = line.split()
+                if len(cols) == 7 and cols[0] == kernel:
+                    return float(cols[5]) * 1e6
+    except (OSError, ValueError):
+        pass
+    return None
+
+
+def kernel_time_shares(n, top=6):
+    """Per-kernel share of the GPU time of one block at N_token = n from the committed kernel-trace
+    summary profiles/pairformer_block_n<N>_bf16_kernel_stats.txt: {kernel: [avg us per launch, % of time]}."""
+    shares = {}
+    try:
+        with open(os.path.join(PROFILES, f"pairformer_block_n{n}_bf16_kernel_stats.txt")) as f:
+            for line in f:
+                cols = line.split()
+                if len(cols) >= 6 and "_kernel" in cols[0] and cols[-1].replace(".", "", 1).isdigit():
+                    try:
+                        shares[cols[0].split("<")[0]] = [float(cols[-4]), float(cols[-1])]
+                    except ValueError:
+                        continue
+    except OSError:
+        return None
+    return dict(sorted(shares.items(), key=lambda kv: -kv[1][1])[:top]) or None
 
 
 def flops_trimul(n):      # one direction
@@ -304,6 +337,8 @@ def trunk_n1536(pkg, dev, n=1536, blocks=48, passes=2):
             raise RuntimeError("non-finite pair activations after the trunk")
         res[label] = {"ms_total": round(best, 2), "ms_per_block": round(best / blocks, 3),
                       "tflops": round(blocks * flops_block(n) / best / 1e9, 1)}
+    # where a block's time goes at this size: [avg us per launch, % of GPU time] from the committed summary
+    res["per_kernel_share"] = kernel_time_shares(n)
     return res
 
 
@@ -315,6 +350,8 @@ def main():
     ap.add_argument("--n-token", type=int, default=768)
     ap.add_argument("--io", choices=["bf16", "f32"], default="bf16", help="dtype of the residual stream")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--all-ones", action="store_true",
+                    help="all-ones masks for every leg (no padding), for profiles of the roofline launch")
     ap.add_argument("--no-trunk", action="store_true", help="skip the 48-block N=1536 trunk timing")
     ap.add_argument("--no-diffusion", action="store_true",
                     help="skip the diffusion-head, Evoformer-block and 64-channel-block timings")
@@ -373,6 +410,7 @@ def main():
             raise RuntimeError("non-finite pair activations after the timed steps")
         pair.normal_(generator=None)
         single.normal_(generator=None)
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.steps):
             blk(pair, pm, single, sm)
@@ -382,6 +420,8 @@ def main():
         single.normal_(generator=None)
         return ms, iso
 
+    if args.all_ones:   # (for profiles: every launch of the run then does all of the algorithm's work)
+        seq_mask, pair_mask, live = seq_ones, pair_ones, n
     ms_per_step, ms_isolated = timed(pair_mask, seq_mask)
     # the same block with nothing masked: every kernel leaves out work on padding (fully masked prologue tiles,
     # rows without a live key, key tiles without one), so the padded figure flatters the kernels by that much
@@ -425,30 +465,34 @@ def main():
     # shortcut (no products), a live row visits only the 64-key tiles that hold a live key, all N queries each
     executed_attn = 512.0 * live * n * (64.0 * ((live + 63) // 64))
 
-    def roofline_of(ms_c, ms_a, exec_a):
-        kernels = {
-            "contract_kernel (triangle contraction)": (ms_c, flops_contraction(n), flops_contraction(n)),
-            "triattn_flash_kernel (triangle attention core)": (ms_a, flops_attention_core(n), exec_a),
+    # The roofline object is on the ALL-ONES mask: the kernel then executes exactly the algorithm's FLOPs, so
+    # the fraction is neither flattered by skipped padding nor dependent on how the padding falls on tiles.
+    # `padded` beside it is the same launch under the workload's 10 % padding, on both counts of FLOPs.
+    kernels = {
+        "contract_kernel (triangle contraction)": (ms_contract, flops_contraction(n)),
+        "triattn_flash_kernel (triangle attention core)": (ms_attn_un, flops_attention_core(n)),
+    }
+    dom = max(kernels, key=lambda k: kernels[k][0])      # each runs twice per block
+    dom_ms, dom_flops = kernels[dom]
+    achieved = dom_flops / dom_ms / 1e9
+    roofline = {
+        "kernel": dom, "mask": "all-ones (nothing skipped: algorithmic FLOPs = executed FLOPs)",
+        "bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+        "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
+        "traffic": measured_traffic_bytes(dom.split(" ")[0], n),
+        "launch_ms": round(dom_ms, 4),
+        "others": {k: {"launch_ms": round(v[0], 4), "tflops": round(v[1] / v[0] / 1e9, 2),
+                       "frac": round(v[1] / v[0] / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
+                   for k, v in kernels.items() if k != dom},
+    }
+    if dom.startswith("triattn") and not args.all_ones:
+        roofline["padded"] = {
+            "mask": "10% trailing tokens masked (the workload of `value`)",
+            "launch_ms": round(ms_attn, 4),
+            "frac_algorithmic_flops": round(flops_attention_core(n) / ms_attn / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "frac_executed_flops": round(executed_attn / ms_attn / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "executed_share_of_algorithmic_flops": round(executed_attn / flops_attention_core(n), 4),
         }
-        dom = max(kernels, key=lambda k: kernels[k][0])      # each runs twice per block
-        dom_ms, dom_flops, dom_exec = kernels[dom]
-        achieved = dom_flops / dom_ms / 1e9
-        return {
-            "kernel": dom, "bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
-            "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-            # `achieved` / `frac` count the algorithm's FLOPs at full N; the kernel leaves out the padding's
-            # share, so the fraction of the peak on FLOPs it actually executes is lower:
-            "achieved_executed": round(dom_exec / dom_ms / 1e9, 2),
-            "frac_executed": round(dom_exec / dom_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
-            "executed_share_of_algorithmic_flops": round(dom_exec / dom_flops, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get((dom.split(" ")[0], n)),
-            "launch_ms": round(dom_ms, 4),
-            "others": {k: {"launch_ms": round(v[0], 4), "tflops": round(v[1] / v[0] / 1e9, 2)}
-                       for k, v in kernels.items() if k != dom},
-        }
-
-    roofline = roofline_of(ms_contract, ms_attn, executed_attn)
-    roofline_un = roofline_of(ms_contract, ms_attn_un, flops_attention_core(n))
     del a, b, t_buf, q_, k_, vt_, nb, og
 
     # ---- the target run: the 48-block trunk at 1536 tokens, whole pair tensor resident ----
@@ -492,7 +536,6 @@ def main():
             "block_tflops": round(flops_block(n) / ms_unmasked / 1e9, 2),
             "per_op_ms": {k: round(v, 4) for k, v in per_op_un.items()},
             "tflops_per_op": {k: round(v, 2) for k, v in tflops_per_op_un.items()},
-            "roofline": roofline_un,
         },
     }
     if trunk is not None:

@@ -334,7 +334,7 @@ static int self_attention_run(
   g.epi = EPI_SEGMENTED; g.seg_len = channels;
   g.seg_ops = SEG_BIAS_SCALE | (SEG_PLAIN << 4) | (SEG_PLAIN << 8) | (SEG_SIGMOID << 12);
   g.alpha = 1.0f / sqrtf((float)d);
-  g.bias = query_b;
+  g.bias = query_b; g.bias_len = channels;  // the query segment's columns only
   int rc = launch_gemm_nt(g, s);
   if (rc) return rc;
 
@@ -465,7 +465,7 @@ int af3_batch_diffusion_cross_attention_forward(
   g.epi = EPI_SEGMENTED; g.seg_len = channels;
   g.seg_ops = SEG_BIAS_SCALE | (SEG_SIGMOID << 4);
   g.alpha = 1.0f / sqrtf((float)d);
-  g.bias = query_b;
+  g.bias = query_b; g.bias_len = channels;  // the query segment's columns only
   int rc = launch_gemm_nt(g, s);
   if (rc) return rc;
   GemmArgs g2;
@@ -523,7 +523,7 @@ int af3_gathered_cross_attention_forward(
   g.epi = EPI_SEGMENTED; g.seg_len = channels;
   g.seg_ops = SEG_BIAS_SCALE | (SEG_SIGMOID << 4);
   g.alpha = 1.0f / sqrtf((float)d);
-  g.bias = query_b;
+  g.bias = query_b; g.bias_len = channels;  // the query segment's columns only
   int rc = launch_gemm_nt(g, s);
   if (rc) return rc;
   GemmArgs g2;
@@ -600,7 +600,7 @@ int af3_linear_forward(
   g.lda = k; g.ldb = k;
   g.ldc = mode == AF3_LINEAR_SWIGLU ? n / 2 : n;
   g.out_f32 = y_dtype == AF3_F32;
-  g.epi = mode; g.alpha = alpha; g.bias = bias; g.act_sigmoid = sigmoid;
+  g.epi = mode; g.alpha = alpha; g.bias = bias; g.bias_len = n; g.act_sigmoid = sigmoid;
   g.gate = gate; g.gate_rows = (int)gate_rows; g.ld_gate = gate_ld ? gate_ld : n;
   if (residual) {
     if (res_dtype == AF3_F32) g.res_f32 = static_cast<const float*>(residual);
@@ -608,6 +608,21 @@ int af3_linear_forward(
     g.ld_res = n;
   }
   return launch_gemm_nt(g, static_cast<hipStream_t>(stream));
+}
+
+// ----------------------------------------------------------------- diagnostics
+int af3_linear_bias_span(int64_t m, int n, int k, int seg_len, int seg_ops, int64_t* first, int64_t* last) {
+  if (!first || !last || m <= 0 || m > 0x7fffffff || n <= 0 || k <= 0 || seg_len < 0) return AF3_ERR_BAD_ARG;
+  if (seg_len > 0 && ((seg_len & 7) || n > 8 * seg_len)) return AF3_ERR_BAD_ARG;
+  // the product as af3_linear_forward (seg_len = 0) or the segmented projections (seg_len > 0) describe
+  // it; the operand pointers only have to look aligned, nothing is dereferenced
+  GemmArgs g;
+  g.A = reinterpret_cast<const bf16_t*>(uintptr_t(16)); g.B = g.A; g.C = reinterpret_cast<void*>(uintptr_t(16));
+  g.bias = reinterpret_cast<const float*>(uintptr_t(16));
+  g.M = (int)m; g.N = n; g.K = k; g.lda = g.ldb = k; g.ldc = n;
+  if (seg_len > 0) { g.epi = EPI_SEGMENTED; g.seg_len = seg_len; g.seg_ops = seg_ops; }
+  gemm_bias_span(g, gemm_big_tile_choice(g) >= 0, first, last);
+  return AF3_OK;
 }
 
 // ------------------------------------------------------- kernel-level entry points

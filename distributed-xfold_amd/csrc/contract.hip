@@ -343,12 +343,10 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(GemmArgs g) {
     float* sBiasW = sColBias + (MODE == BIG_COLUMN_OPS ? wave * 128 : 0);
     if constexpr (MODE == BIG_COLUMN_OPS) {
       // the bias array only covers the segments that use it
-      const int colb = t.n0 + wn + 4 * lane;
-      bool uses_bias = g.bias != nullptr && lane < 32;
-      if (g.epi == EPI_SEGMENTED)
-        uses_bias = uses_bias && ((g.seg_ops >> (4 * (min(colb, g.N - 1) / g.seg_len))) & 15) == SEG_BIAS_SCALE;
+      int first;
+      const bool uses_bias = big_tile_bias_quad(g, t.n0 + wn + 4 * lane, &first) && lane < 32;
       f32x4 b4 = {0.f, 0.f, 0.f, 0.f};
-      if (uses_bias) b4 = *reinterpret_cast<const f32x4*>(g.bias + min(colb, g.N - 4));
+      if (uses_bias) b4 = *reinterpret_cast<const f32x4*>(g.bias + first);
       if (lane < 32) *reinterpret_cast<f32x4*>(sBiasW + 4 * lane) = b4;
     }
     auto convert = [&](int n, u32x2* out) {
@@ -495,10 +493,42 @@ int big_tile_mode(const GemmArgs& g) {
   return (g.bias || g.act_sigmoid || g.alpha != 1.f) ? BIG_COLUMN_OPS : BIG_PLAIN;
 }
 
+void gemm_bias_span(const GemmArgs& g, bool big, int64_t* first, int64_t* last) {
+  int64_t lo = INT64_MAX, hi = 0;
+  if (g.bias && g.N > 0 && (g.epi != EPI_SEGMENTED || g.seg_len > 0)) {
+    if (big) {
+      // every (tile column, wave column, lane) of the epilogue's bias fetch
+      for (int n0 = 0; n0 < g.N; n0 += CN)
+        for (int wn = 0; wn < CN; wn += 128)
+          for (int lane = 0; lane < 32; ++lane) {
+            int f;
+            if (!big_tile_bias_quad(g, n0 + wn + 4 * lane, &f)) continue;
+            lo = std::min<int64_t>(lo, f);
+            hi = std::max<int64_t>(hi, (int64_t)f + 4);
+          }
+    } else {
+      // gemm_nt_kernel: chunk of up to 8 columns from every multiple of 8 below N
+      for (int n = 0; n < g.N; n += 8) {
+        if (!gemm_col_uses_bias(g, n)) continue;
+        lo = std::min<int64_t>(lo, n);
+        hi = std::max<int64_t>(hi, std::min<int64_t>(n + 8, g.N));
+      }
+    }
+  }
+  *first = hi > 0 ? lo : 0;
+  *last = hi;
+}
+
 int launch_big_tile(const GemmArgs& g, int mode, hipStream_t stream) {
   if (!g.A || !g.B || !g.C) return AF3_ERR_BAD_ARG;
   if (mode != big_tile_mode(g) && !(mode == BIG_PLAIN && contract_supported(g))) return AF3_ERR_BAD_ARG;
   if (mode < BIG_PLAIN || mode > BIG_SWIGLU) return AF3_ERR_BAD_ARG;
+  if (mode == BIG_COLUMN_OPS && g.bias) {
+    // the epilogue fetches the bias in groups of four per lane: nothing it touches may lie outside the array
+    int64_t first, last;
+    gemm_bias_span(g, true, &first, &last);
+    if (first < 0 || last > g.bias_len) return AF3_ERR_BAD_ARG;
+  }
   const int64_t tiles_n = (g.N + CN - 1) / CN;
   const int64_t total4 = (int64_t)((g.M + 255) / 256) * tiles_n * g.batch;
   const int64_t total3 = (int64_t)((g.M + 191) / 192) * tiles_n * g.batch;

@@ -213,7 +213,7 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
   for (int e = 0; e < 8; ++e) bias[e] = 0.f;
   if (g.epi == EPI_SEGMENTED) {
     op = (g.seg_ops >> (4 * (n / g.seg_len))) & 15;  // seg_len % 8 == 0: a chunk never straddles segments
-    if (op == SEG_BIAS_SCALE && g.bias)
+    if (gemm_col_uses_bias(g, n))
 #pragma unroll
       for (int e = 0; e < 8; ++e) if (e < nv) bias[e] = g.bias[n + e];
   } else if (g.bias) {
@@ -299,19 +299,23 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
 
 }  // namespace
 
+// Products of at least 120 tiles of 256x256 go to the large-tile kernel where
+// one of its epilogues fits: from there on the 128x128 tiles no longer fit
+// the chip in one round (two workgroups per CU) and the large tile, with
+// half the fragment reads per MFMA, is 1.3 to 1.45 times faster;
+// below, the two kernels are within a few percent of each other and the
+// small tile wins where it fills more CUs.
+int gemm_big_tile_choice(const GemmArgs& g) {
+  constexpr int64_t BIG_TILE_MIN_TILES = 120;
+  const int64_t tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * g.batch;
+  return g.M > 128 && g.N > 128 && tiles >= BIG_TILE_MIN_TILES ? big_tile_mode(g) : -1;
+}
+
 int launch_gemm_nt(const GemmArgs& g_in, hipStream_t stream) {
   GemmArgs g = g_in;
   if (g.M <= 0 || g.N <= 0 || g.K <= 0 || g.batch <= 0) return AF3_ERR_BAD_ARG;
   {
-    // Products of at least 120 tiles of 256x256 go to the large-tile kernel where
-    // one of its epilogues fits: from there on the 128x128 tiles no longer fit
-    // the chip in one round (two workgroups per CU) and the large tile, with
-    // half the fragment reads per MFMA, is 1.3 to 1.45 times faster;
-    // below, the two kernels are within a few percent of each other and the
-    // small tile wins where it fills more CUs.
-    constexpr int64_t BIG_TILE_MIN_TILES = 120;
-    const int64_t tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * g.batch;
-    const int big = g.M > 128 && g.N > 128 && tiles >= BIG_TILE_MIN_TILES ? big_tile_mode(g) : -1;
+    const int big = gemm_big_tile_choice(g);
     if (big >= 0) return launch_big_tile(g, big, stream);
   }
   if ((g.K & 7) || (g.lda & 7) || (g.ldb & 7) || (g.sA & 7) || (g.sB & 7)) return AF3_ERR_BAD_ARG;
@@ -319,6 +323,11 @@ int launch_gemm_nt(const GemmArgs& g_in, hipStream_t stream) {
   if (g.epi == EPI_SWIGLU && ((g.N & 63) || g.out_f32)) return AF3_ERR_BAD_ARG;
   if (g.epi == EPI_SEGMENTED && (g.seg_len <= 0 || (g.seg_len & 7))) return AF3_ERR_BAD_ARG;
   if (g.gate && g.gate_rows <= 0) return AF3_ERR_BAD_ARG;
+  if (g.bias) {
+    int64_t first, last;
+    gemm_bias_span(g, false, &first, &last);
+    if (first < 0 || last > g.bias_len) return AF3_ERR_BAD_ARG;
+  }
   if (g.regroup32 && (g.epi != EPI_PLAIN || g.batch != 1 || (g.M & 31) || (g.N & 31))) return AF3_ERR_BAD_ARG;
   // 16/32-byte stores need aligned rows; otherwise the epilogue stores element-wise
   const int esz = g.out_f32 ? 4 : 2;

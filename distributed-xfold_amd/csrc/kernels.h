@@ -16,7 +16,8 @@ struct GemmArgs {
   int out_f32 = 0;
   int epi = EPI_PLAIN;
   float alpha = 1.f;            // PLAIN: (acc + bias) * alpha ; SEG_BIAS_SCALE likewise
-  const float* bias = nullptr;  // [N]
+  const float* bias = nullptr;  // indexed by output column: entries 0 .. bias_len - 1 exist
+  int64_t bias_len = 0;         // a launch whose epilogue would read past it is refused (gemm_bias_span)
   int act_sigmoid = 0;          // PLAIN only
   int seg_len = 0, seg_ops = 0; // SEGMENTED: op of column segment s in bits [4s, 4s+4)
   const float* gate = nullptr;  // GATE_RES: multiply by gate[m % gate_rows][n]
@@ -33,6 +34,24 @@ struct GemmArgs {
   int regroup32 = 0;
 };
 int launch_gemm_nt(const GemmArgs& g, hipStream_t stream);
+// Which bias entries a launch reads.  Column c takes bias[c] when the epilogue is not segmented, or
+// when c lies in a segment whose op is SEG_BIAS_SCALE; the kernels read whole groups of entries
+// (gemm_nt_kernel up to 8 from a multiple of 8, the large tile 4 from a multiple of 4, the last
+// group pulled back to end at N).  The device code takes its addresses from these functions, the
+// host takes the extent it checks against bias_len from them: one formula for both.
+__host__ __device__ inline bool gemm_col_uses_bias(const GemmArgs& g, int col) {
+  if (!g.bias) return false;
+  if (g.epi != EPI_SEGMENTED) return true;
+  return ((g.seg_ops >> (4 * (col / g.seg_len))) & 15) == SEG_BIAS_SCALE;
+}
+// large tile: the 4 entries a lane fetches for columns colb .. colb + 3 of its wave (colb may lie past N)
+__host__ __device__ inline bool big_tile_bias_quad(const GemmArgs& g, int colb, int* first) {
+  *first = (colb < g.N - 4 ? colb : g.N - 4);
+  return gemm_col_uses_bias(g, colb < g.N - 1 ? colb : g.N - 1);
+}
+// Half-open range [first, last) of bias entries the launch of `g` reads (big: on the large tile);
+// first == last: none.
+void gemm_bias_span(const GemmArgs& g, bool big, int64_t* first, int64_t* last);
 // contract.hip: the same product, plain bf16 output, 256x256 tiles (large M, N)
 bool contract_supported(const GemmArgs& g);
 int launch_contract(const GemmArgs& g, hipStream_t stream);
@@ -41,6 +60,8 @@ int launch_contract(const GemmArgs& g, hipStream_t stream);
 // kernel instance that can take `g`, or -1
 int big_tile_mode(const GemmArgs& g);
 int launch_big_tile(const GemmArgs& g, int mode, hipStream_t stream);
+// the large-tile instance launch_gemm_nt hands `g` to, or -1: the 128x128-tile kernel
+int gemm_big_tile_choice(const GemmArgs& g);
 
 // ---------------------------------------------------------------- rowops.hip
 // y = LN(x) [* weight + bias] ; then, if scale: y = sigmoid(scale[r]) * y + shift[r]

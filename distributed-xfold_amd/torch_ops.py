@@ -69,11 +69,25 @@ _libs = []          # torch.library.Library objects must stay alive
 _registered = False
 
 
-def _cached(tensors, build):
-    """`build()` once per set of source tensors.  An entry holds weak references to its sources and
-    is only good while they are the very same tensor objects, unmodified (`_version`): an address alone
-    may have been handed to another tensor in the meantime."""
-    key = tuple((id(t), t._version) for t in tensors)
+def _version_of(t):
+    """The tensor's modification counter, or None where it has none to offer (tensors created under
+    torch.inference_mode() refuse to tell)."""
+    try:
+        return t._version
+    except RuntimeError:
+        return None
+
+
+def _cached(role, tensors, build):
+    """`build()` once per (role, set of source tensors).  `role` names what is built: the same tensor may
+    reach two builders (an fp32 copy here, a repacked bf16 weight there) and each needs its own entry.  An
+    entry holds weak references to its sources and is only good while they are the very same tensor objects,
+    unmodified (`_version`): an address alone may have been handed to another tensor in the meantime.
+    Sources without a version counter are not cached."""
+    versions = tuple(_version_of(t) for t in tensors)
+    if any(v is None for v in versions):
+        return build()
+    key = (role,) + tuple((id(t), v) for t, v in zip(tensors, versions))
     hit = _CACHE.get(key)
     if hit is not None and all(r() is t for r, t in zip(hit[0], tensors)):
         return hit[1]
@@ -89,11 +103,11 @@ def clear_cache() -> None:
 
 
 def _f32(t: torch.Tensor) -> torch.Tensor:
-    return _cached((t,), lambda: t.detach().to(torch.float32).contiguous())
+    return _cached("f32", (t,), lambda: t.detach().to(torch.float32).contiguous())
 
 
 def _bf16(t: torch.Tensor) -> torch.Tensor:
-    return _cached((t,), lambda: t.detach().to(torch.bfloat16).contiguous())
+    return _cached("bf16", (t,), lambda: t.detach().to(torch.bfloat16).contiguous())
 
 
 def _linear_weight(w_chd: torch.Tensor) -> torch.Tensor:
@@ -102,11 +116,21 @@ def _linear_weight(w_chd: torch.Tensor) -> torch.Tensor:
 
 
 def _key_mask(bias: torch.Tensor, batch: int, seq: int) -> torch.Tensor:
-    """`1e9 * (mask - 1)` of shape [B or 1, 1, 1, S] back to the 0/1 mask [B, S]."""
-    m = (bias.reshape(-1, seq) > -5e8).to(torch.float32)
-    if m.shape[0] not in (1, batch):
-        raise ValueError(f"bias: expected [{batch}, 1, 1, {seq}] or [1, 1, 1, {seq}], got {tuple(bias.shape)}")
-    return m.expand(batch, seq).contiguous()
+    """The operators' additive `bias` argument, `1e9 * (mask - 1)` of shape [B or 1, 1, 1, S]
+    (d_attention.py:63, d_diffusion_transformer.py:206), back to the 0/1 key mask [B, S] the kernels take.
+    The kernels replace a masked key's logit by -1e9 and add nothing to the others, so any other additive
+    value cannot be honoured: a tensor that holds anything but 0 and -1e9 is refused.  One reduction on
+    the device per tensor version (the result is cached with the mask)."""
+    def build():
+        flat = bias.detach().reshape(-1, seq).to(torch.float32)
+        if flat.shape[0] not in (1, batch):
+            raise ValueError(f"bias: expected [{batch}, 1, 1, {seq}] or [1, 1, 1, {seq}], got {tuple(bias.shape)}")
+        # (-1e9 as fp32 holds it, or as a bf16 / fp16-free cast chain may have rounded it: within 2^-8)
+        if not bool(((flat == 0) | ((flat + 1e9).abs() <= 4e6)).all()):
+            raise ValueError("bias: only the key-mask form 1e9 * (mask - 1), i.e. values 0 and -1e9, is supported "
+                             "on the GPU path; other additive biases belong in nonbatched_bias")
+        return (flat == 0).to(torch.float32).expand(batch, seq).contiguous()
+    return _cached(("key_mask", batch, seq), (bias,), build)
 
 
 def _activations(x: torch.Tensor) -> torch.Tensor:
@@ -129,7 +153,7 @@ def traingle_multiplication_forward(act, mask, equation_flag, left_norm_input_we
                   for h in (0, 1) for lo in (0, 64)]
         return torch.stack(chunks).to(torch.bfloat16).contiguous()
 
-    w_pg = _cached((projection_weight, gate_weight), pack)
+    w_pg = _cached("trimul_proj_gate", (projection_weight, gate_weight), pack)
     n = act.shape[0]
     return ops.triangle_multiplication(
         _activations(act).contiguous(), mask.reshape(n, -1), int(equation_flag), _f32(left_norm_input_weight),
@@ -150,8 +174,8 @@ def grid_self_attn_forward(q_data, bias, nonbatched_bias, query_w, key_w, value_
         return torch.stack([_linear_weight(w) for w in (query_w, key_w, value_w, gating_w)]) \
             .to(torch.bfloat16).contiguous()
 
-    w_qkvg = _cached((query_w, key_w, value_w, gating_w), pack)
-    w_out = _cached((output_w,), lambda: output_w.detach().reshape(-1, output_w.shape[-1]).t()
+    w_qkvg = _cached("grid_qkvg", (query_w, key_w, value_w, gating_w), pack)
+    w_out = _cached("attn_output_w", (output_w,), lambda: output_w.detach().reshape(-1, output_w.shape[-1]).t()
                     .to(torch.bfloat16).contiguous())
     nb = nonbatched_bias.to(torch.float32).contiguous() if nonbatched_bias.numel() else None
     return ops.grid_self_attn(_activations(q_data).contiguous(), _key_mask(bias, b, s), False, None, None, None, nb,
@@ -168,8 +192,8 @@ def batch_diffusion_self_attention_forward(q_data, bias, nonbatched_bias, query_
         return torch.cat([_linear_weight(w) for w in (query_w, key_w, value_w, gating_w)], dim=0) \
             .to(torch.bfloat16).contiguous()
 
-    w_qkvg = _cached((query_w, key_w, value_w, gating_w), pack)
-    q_b = _cached((query_b,), lambda: query_b.detach().reshape(-1).to(torch.float32).contiguous()) \
+    w_qkvg = _cached("self_qkvg", (query_w, key_w, value_w, gating_w), pack)
+    q_b = _cached("query_b", (query_b,), lambda: query_b.detach().reshape(-1).to(torch.float32).contiguous()) \
         if query_b.numel() else None
     nb = nonbatched_bias.to(torch.float32).contiguous() if nonbatched_bias.numel() else None
     out = ops.batch_diffusion_self_attention(q_data.to(torch.bfloat16).contiguous(), _key_mask(bias, b, s), nb,
@@ -184,11 +208,11 @@ def batch_diffusion_cross_attention_forward(q_data, m_data, batched_bias, query_
     b, sq, c = q_data.shape
     sk = m_data.shape[1]
     num_head = query_w.shape[1]
-    w_qg = _cached((query_w, gating_w), lambda: torch.cat([_linear_weight(query_w), _linear_weight(gating_w)], dim=0)
+    w_qg = _cached("cross_qg", (query_w, gating_w), lambda: torch.cat([_linear_weight(query_w), _linear_weight(gating_w)], dim=0)
                    .to(torch.bfloat16).contiguous())
-    w_kv = _cached((key_w, value_w), lambda: torch.cat([_linear_weight(key_w), _linear_weight(value_w)], dim=0)
+    w_kv = _cached("cross_kv", (key_w, value_w), lambda: torch.cat([_linear_weight(key_w), _linear_weight(value_w)], dim=0)
                    .to(torch.bfloat16).contiguous())
-    q_b = _cached((query_b,), lambda: query_b.detach().reshape(-1).to(torch.float32).contiguous()) \
+    q_b = _cached("query_b", (query_b,), lambda: query_b.detach().reshape(-1).to(torch.float32).contiguous()) \
         if query_b.numel() else None
     logits = batched_bias.to(torch.float32).reshape(-1, batched_bias.shape[-3], sq, sk)
     logits = logits.expand(logits.shape[0], num_head, sq, sk).contiguous()
@@ -208,9 +232,9 @@ def transition_forward(act, transition1, transition2, layernorm_weight, layernor
         raise ValueError("transition_forward on the GPU: 128 channels")
     from .nn.base import pack_swiglu
     hidden = transition2.shape[0]
-    w1 = _cached((transition1,), lambda: pack_swiglu(transition1.detach().t(), 64).to(torch.bfloat16)
+    w1 = _cached("transition1", (transition1,), lambda: pack_swiglu(transition1.detach().t(), 64).to(torch.bfloat16)
                  .reshape(hidden // 64, 128, 128).contiguous())
-    w2 = _cached((transition2,), lambda: transition2.detach().t().to(torch.bfloat16).contiguous())
+    w2 = _cached("transition2", (transition2,), lambda: transition2.detach().t().to(torch.bfloat16).contiguous())
     x = _activations(act).contiguous()
     return ops.transition128(x.view(-1, c), _f32(layernorm_weight), _f32(layernorm_bias), w1, w2,
                              residual=False).view(act.shape)

@@ -405,6 +405,21 @@ int af3_linear_forward(
     const void* residual, int res_dtype, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Diagnostic, no counterpart in the reference.  The dense kernels fetch a
+ * column bias in groups (eight entries on the 128x128 tile, four per lane on the
+ * 256x256 tile, the last group pulled back to end at column n), and a segmented
+ * epilogue (the q-k-v-gate projection of the attentions: segments of seg_len
+ * columns, op of segment s in bits [4s, 4s+4) of seg_ops, 1 = biased and
+ * scaled) only touches the entries of the segments that use the bias.
+ * af3_linear_bias_span reports the half-open range [*first, *last) of entries
+ * a product x[m,k] W[n,k]^T with a bias would read on the kernel that takes it
+ * (seg_len = 0: one bias per column, as af3_linear_forward), computed by the
+ * function the launch path itself checks the caller's extent with; no GPU is
+ * needed.
+ */
+int af3_linear_bias_span(int64_t m, int n, int k, int seg_len, int seg_ops, int64_t* first, int64_t* last);
+
+/* ---------------------------------------------------------------------------
  * Kernel-level entry points: the two MFMA-bound inner kernels on their own,
  * so that a caller (the benchmark's roofline leg, a profiler) can time exactly
  * one launch.  They are the inner stages of the operators above.

@@ -83,6 +83,37 @@ def test_null_and_bad_arguments_are_rejected_without_a_gpu(pkg):
                                                    None, 0, 8, None, 0, None) == -1
 
 
+def _bias_span(lib, m, n, k, seg_len=0, seg_ops=0):
+    first, last = ctypes.c_int64(-1), ctypes.c_int64(-1)
+    assert lib.af3_linear_bias_span(m, n, k, seg_len, seg_ops, ctypes.byref(first), ctypes.byref(last)) == 0
+    return first.value, last.value
+
+
+def test_bias_entries_a_launch_reads_stay_inside_the_callers_array(pkg):
+    """The dense kernels fetch the column bias in groups; the launch path refuses a product whose groups
+    would reach past the extent the caller vouches for.  The span comes from the formula the device
+    code takes its addresses from.  Shapes: the q-k-v-gate projection of
+    tests/test_gpu_big_tile.py::test_self_attention_projection_segments (5 x 768 tokens, 768 channels:
+    the 256x256 tile; its bias covers the 768 query columns only), one sample of it (128x128 tile),
+    and plain biased products with ragged column counts on both tiles."""
+    lib = pkg.lib.load()
+    BIAS_SCALE, PLAIN, SIGMOID = 1, 0, 2
+    qkvg = BIAS_SCALE | (PLAIN << 4) | (PLAIN << 8) | (SIGMOID << 12)
+    for m in (5 * 768, 768):                       # large tile / small tile
+        assert _bias_span(lib, m, 4 * 768, 768, 768, qkvg) == (0, 768)
+    # queries and gates of the atom cross-attention: 2 x 128 columns, bias for the first 128
+    assert _bias_span(lib, 5 * 576 * 32, 256, 128, 128, BIAS_SCALE | (SIGMOID << 4)) == (0, 128)
+    # a biased segment further right reaches further: the launch path compares this with the extent
+    assert _bias_span(lib, 5 * 768, 4 * 768, 768, 768, PLAIN | (BIAS_SCALE << 8)) == (2 * 768, 3 * 768)
+    # unsegmented: exactly the n columns, whatever the tile and however ragged n is
+    for m, n, k in ((3850, 2824, 200), (5000, 3400, 72), (300, 2824, 200), (100, 40, 64), (4096, 2560, 768)):
+        assert _bias_span(lib, m, n, k) == (0, n), (m, n, k)
+    # no segment uses the bias: nothing is read
+    first, last = _bias_span(lib, 5 * 768, 4 * 768, 768, 768, PLAIN | (SIGMOID << 12))
+    assert first == last
+    assert lib.af3_linear_bias_span(0, 8, 8, 0, 0, None, None) == -1
+
+
 def test_gathered_cross_attention_and_regrouped_store_reject_bad_arguments(pkg):
     lib = pkg.lib.load()
     one = 1 << 20     # a non-null dummy address: every check below fails before it is touched

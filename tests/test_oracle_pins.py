@@ -470,6 +470,30 @@ def test_pairformer_block_wiring():
     assert torch.allclose(only_pair, z, atol=1e-12)
 
 
+def test_pairformer_stack_threads_pair_and_single_through_its_blocks():
+    """d_alphafold3.py:242-244: block i + 1 takes BOTH outputs of block i (a stack that re-fed the
+    input single, dropped a block or applied them in another order fails), and the distinct weights of
+    the blocks do not commute."""
+    g = gen(23)
+    N = 5
+    blocks = [O.cast_params(O.make_pairformer_block_params(g, std=0.1), D) for _ in range(2)]
+    pair, single = randn(g, N, N, 128), randn(g, N, 384)
+    seq_mask = torch.tensor([1, 1, 1, 1, 0], dtype=D)
+    pair_mask = seq_mask[:, None] * seq_mask[None, :]
+    got_pair, got_single = O.pairformer_stack(pair, pair_mask, single, seq_mask, blocks)
+    p1, s1 = O.pairformer_block(pair, pair_mask, single, seq_mask, blocks[0])
+    p2, s2 = O.pairformer_block(p1, pair_mask, s1, seq_mask, blocks[1])
+    assert torch.equal(got_pair, p2) and torch.equal(got_single, s2)
+    # the mistakes the pin is there for give visibly different answers
+    _, s_stale = O.pairformer_block(p1, pair_mask, single, seq_mask, blocks[1])
+    r1, t1 = O.pairformer_block(pair, pair_mask, single, seq_mask, blocks[1])
+    r2, _ = O.pairformer_block(r1, pair_mask, t1, seq_mask, blocks[0])
+    assert not torch.allclose(s_stale, s2, atol=1e-6) and not torch.allclose(r2, p2, atol=1e-6)
+    assert not torch.allclose(p1, p2, atol=1e-6)
+    one_pair, one_single = O.pairformer_stack(pair, pair_mask, single, seq_mask, blocks[:1])
+    assert torch.equal(one_pair, p1) and torch.equal(one_single, s1)
+
+
 def test_diffusion_transformer_wiring_and_logit_layout():
     g = gen(20)
     N, c, cs, cp, H, nb, sbs = 5, 16, 8, 6, 4, 4, 2

@@ -94,6 +94,39 @@ def test_repacked_weights_follow_their_source_tensor(pkg):
     assert len(seen) < 50
 
 
+def test_cache_entries_are_per_role_and_survive_inference_mode(pkg):
+    """One tensor that reaches two builders gets one entry per builder (an fp32 copy is not a bf16 copy),
+    and tensors made under torch.inference_mode(), which have no version counter, are simply not cached."""
+    from distributed_xfold_amd import torch_ops
+    torch_ops.clear_cache()
+    a = torch.arange(8, dtype=torch.float64)
+    f, b = torch_ops._f32(a), torch_ops._bf16(a)
+    assert f.dtype == torch.float32 and b.dtype == torch.bfloat16
+    assert torch_ops._f32(a) is f and torch_ops._bf16(a) is b
+    with torch.inference_mode():
+        t = torch.ones(8, dtype=torch.bfloat16)
+        got = torch_ops._f32(t)
+        assert got.dtype == torch.float32 and float(got.sum()) == 8.0
+        assert torch_ops._key_mask(torch.zeros(1, 1, 1, 4), 2, 4).shape == (2, 4)
+
+
+def test_operator_bias_must_be_a_key_mask(pkg):
+    """The operators' `bias` argument is the additive key mask 1e9 * (mask - 1) (Alpha_Attention.cpp:182-185,
+    built at d_attention.py:63 and d_diffusion_transformer.py:206).  The kernels take it as a 0/1 mask; any
+    other additive value would be dropped, so it is refused instead."""
+    from distributed_xfold_amd import torch_ops
+    mask = torch.tensor([[1., 1., 0., 1.], [0., 1., 1., 1.]])
+    bias = (1e9 * (mask - 1))[:, None, None, :]
+    assert torch.equal(torch_ops._key_mask(bias, 2, 4), mask)
+    assert torch.equal(torch_ops._key_mask(bias.bfloat16(), 2, 4), mask)          # -1e9 as bf16 rounds it
+    assert torch.equal(torch_ops._key_mask(bias[:1], 3, 4), mask[:1].expand(3, 4))
+    for bad in (bias + 0.5, bias * 0.5, torch.full((2, 1, 1, 4), -3.0)):
+        with pytest.raises(ValueError, match="key-mask form"):
+            torch_ops._key_mask(bad, 2, 4)
+    with pytest.raises(ValueError, match="expected"):
+        torch_ops._key_mask(bias, 3, 4)
+
+
 # ------------------------------------------------------------------ GPU: the operators as the reference calls them
 gpu = pytest.mark.gpu
 
