@@ -117,6 +117,7 @@ static int triangle_multiplication_impl(
 
   TriMulArgs a;
   a.lw = ln_width(valid_channels);
+  a.valid_c = valid_channels;
   a.pair = act; a.mask = mask; a.out = out;
   a.io_f32 = io_dtype == AF3_F32; a.N = (int)n; a.Np = (int)np;
   a.outgoing = equation_flag == 0; a.residual = residual != 0;
@@ -132,7 +133,8 @@ static int triangle_multiplication_impl(
   g.A = a.outgoing ? a_buf : b_buf;
   g.B = a.outgoing ? b_buf : a_buf;
   g.C = t_buf;
-  g.M = g.N = (int)n; g.K = (int)np; g.batch = C_PAIR;
+  // (the hidden layer has as many channels as the pair tensor: the padded ones are zero and are left out)
+  g.M = g.N = (int)n; g.K = (int)np; g.batch = valid_channels;
   g.lda = g.ldb = g.ldc = np;
   g.sA = g.sB = g.sC = n * np;
   rc = contraction(g, s);

@@ -115,6 +115,7 @@ inline LnWidth ln_width(int valid) {
 
 struct TriMulArgs {
   LnWidth lw;
+  int valid_c = 128;  // hidden channels 0 .. valid_c - 1 are real: the others are never contracted and count as zero
   const void* pair = nullptr;   // [N][N][128]
   const float* mask = nullptr;  // [N][N] 0/1 or null
   void* out = nullptr;          // [N][N][128]; may alias pair when residual

@@ -217,8 +217,10 @@ __global__ __launch_bounds__(256, 2) void trimul_epilogue_kernel(TriMulArgs a) {
   const int j_chunk = t.r0 + pc * 8 < a.Np ? t.r0 + pc * 8 : t.r0;
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
+    // (channels past the valid ones were not contracted: their rows hold whatever the workspace held;
+    // the load goes to a valid channel's row instead and is replaced by zeros below)
     const int c = it * 16 + crow;
-    rt[it] = *reinterpret_cast<const u32x4*>(a.t_buf + ((int64_t)c * a.N + t.o) * a.Np + j_chunk);
+    rt[it] = *reinterpret_cast<const u32x4*>(a.t_buf + ((int64_t)(c < a.valid_c ? c : 0) * a.N + t.o) * a.Np + j_chunk);
   }
 
   // 1. output gate from the LayerNorm-ed input: sigmoid(LN(x) Wgl^T), T form, kept in registers
@@ -245,7 +247,8 @@ __global__ __launch_bounds__(256, 2) void trimul_epilogue_kernel(TriMulArgs a) {
   // transposing 2-byte scatter would put a whole wave on two banks.
   bf16_t* sT = sX;
 #pragma unroll
-  for (int it = 0; it < 8; ++it) *reinterpret_cast<u32x4*>(sT + (it * 16 + crow) * LDX + pc * 8) = rt[it];
+  for (int it = 0; it < 8; ++it)
+    *reinterpret_cast<u32x4*>(sT + (it * 16 + crow) * LDX + pc * 8) = it * 16 + crow < a.valid_c ? rt[it] : u32x4{0u, 0u, 0u, 0u};
   wr.store(sW, tid);
   if (tid < C) {
     sP[tid] = a.ln_c_w[tid];
