@@ -384,6 +384,18 @@ int af3_batch_diffusion_self_attention_forward_static(
                             num_head, out, out_dtype, batch, seq, channels, qkvg, static_cast<hipStream_t>(stream));
 }
 
+// ---------------------------------------------------- masked row softmax, narrow fp32 layers
+int af3_masked_softmax_rows_forward(const float* logits, const float* key_mask, uint16_t* out, int64_t rows,
+                                    int64_t cols, int64_t out_ld, af3_stream_t stream) {
+  if (cols <= 0 || cols > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  return launch_softmax_rows(logits, key_mask, out, rows, (int)cols, out_ld, static_cast<hipStream_t>(stream));
+}
+
+int af3_narrow_linear_f32_forward(const float* x, const float* w, const float* residual, float* y, int64_t rows,
+                                  int k, int n_out, int relu_input, af3_stream_t stream) {
+  return launch_narrow_linear_f32(x, w, residual, y, rows, k, n_out, relu_input, static_cast<hipStream_t>(stream));
+}
+
 // -------------------------------------------------------------------- transpose
 int af3_transpose_bf16_forward(const uint16_t* in, uint16_t* out, int64_t rows, int64_t cols, af3_stream_t stream) {
   return launch_transpose(in, out, rows, cols, static_cast<hipStream_t>(stream));

@@ -95,6 +95,12 @@ int launch_gather_rows_add(const bf16_t* src, const int* rows, const bf16_t* add
 int launch_ln_project3_gather(const bf16_t* x, const int* rows, const float* ln_w, const float* w, float* out,
                               int64_t batch, int64_t n_src, int64_t n_out, int channels, hipStream_t stream);
 int launch_transpose(const bf16_t* in, bf16_t* out, int64_t rows, int64_t cols, hipStream_t stream);
+// y[r][k] = softmax_k(x[r][k] + 1e9 (mask[k] - 1)) as bf16, x [rows][cols] fp32, y rows ldy apart (the tail zero)
+int launch_softmax_rows(const float* x, const float* mask, bf16_t* y, int64_t rows, int cols, int64_t ldy,
+                        hipStream_t stream);
+// y[r][:] = (res ? res[r][:] : 0) + W relu?(x[r][:]), fp32, W [n_out][k], n_out 16 or 3, k % 4 == 0, k <= 128
+int launch_narrow_linear_f32(const float* x, const float* w, const float* res, float* y, int64_t rows, int k, int n_out,
+                             int relu_in, hipStream_t stream);
 
 // -------------------------------------------------------------- pair_tile.hip
 // Residual-stream tensors (`pair`, `out`, `x`) are bf16 or fp32 (io_f32).

@@ -329,6 +329,62 @@ __global__ __launch_bounds__(256) void ln_project3_gather_kernel(const bf16_t* _
   dst[0] = o0; dst[1] = o1; dst[2] = o2;
 }
 
+// ----------------------------------------------------------------------------
+// softmax over the rows of a [rows][cols] fp32 array with an additive key mask -> bf16.
+// One wave per row, three passes over the row (it stays in the caches): maximum, sum of
+// exponentials, normalised values.  y[r][k] = softmax_k(x[r][k] + 1e9 (mask[k] - 1)),
+// columns cols .. ldy - 1 of y are zero.
+// ----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const float* __restrict__ x, const float* __restrict__ mask,
+                                                          bf16_t* __restrict__ y, int64_t rows, int cols, int64_t ldy) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const float* xr = x + r * cols;
+  auto logit = [&](int k) { return xr[k] + (mask ? 1e9f * (mask[k] - 1.f) : 0.f); };
+  float m = -__builtin_huge_valf();
+  for (int k = lane; k < cols; k += 64) m = fmaxf(m, logit(k));
+  m = wave_max(m);
+  float s = 0.f;
+  for (int k = lane; k < cols; k += 64) s += __expf(logit(k) - m);
+  s = wave_sum(s);
+  const float inv = 1.f / s;
+  bf16_t* yr = y + r * ldy;
+  for (int k = lane; k < ldy; k += 64) yr[k] = k < cols ? f2bf(__expf(logit(k) - m) * inv) : (bf16_t)0;
+}
+
+// ----------------------------------------------------------------------------
+// Narrow fp32 layers of the atom conditioning: y[r][:] = (res ? res[r][:] : 0) + W f(x[r][:]),
+// f = relu or the identity, W [NOUT][k] with NOUT = 16 or 3 outputs and k a multiple of 4 up to
+// 128.  One thread per row, the weights in LDS, plain fp32 FMAs (these layers set up per-batch
+// conditioning in fp32; they are far too narrow for the matrix units).
+// ----------------------------------------------------------------------------
+template <int NOUT>
+__global__ __launch_bounds__(256) void narrow_linear_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                               const float* __restrict__ res, float* __restrict__ y,
+                                                               int64_t rows, int k, int relu_in) {
+  __shared__ __attribute__((aligned(16))) float sW[NOUT * 128];
+  for (int i = threadIdx.x; i < NOUT * k; i += 256) sW[i] = w[i];
+  __syncthreads();
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= rows) return;
+  float acc[NOUT];
+#pragma unroll
+  for (int o = 0; o < NOUT; ++o) acc[o] = res ? res[r * NOUT + o] : 0.f;
+  const float* xr = x + r * k;
+  for (int c = 0; c < k; c += 4) {
+    f32x4 v = *reinterpret_cast<const f32x4*>(xr + c);
+    if (relu_in) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
+#pragma unroll
+    for (int o = 0; o < NOUT; ++o) {
+      const f32x4 ww = *reinterpret_cast<const f32x4*>(sW + o * k + c);
+      acc[o] = fmaf(v.x, ww.x, fmaf(v.y, ww.y, fmaf(v.z, ww.z, fmaf(v.w, ww.w, acc[o]))));
+    }
+  }
+#pragma unroll
+  for (int o = 0; o < NOUT; ++o) y[r * NOUT + o] = acc[o];
+}
+
 }  // namespace
 
 int launch_gather_rows_add(const bf16_t* src, const int* rows, const bf16_t* add, bf16_t* out, int64_t batch,
@@ -399,5 +455,27 @@ int launch_transpose(const bf16_t* in, bf16_t* out, int64_t rows, int64_t cols, 
   const int64_t blocks = ((rows + TT - 1) / TT) * ((cols + TT - 1) / TT);
   if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
   hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, in, out, rows, cols);
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+int launch_softmax_rows(const float* x, const float* mask, bf16_t* y, int64_t rows, int cols, int64_t ldy,
+                        hipStream_t stream) {
+  if (!x || !y || rows <= 0 || cols <= 0 || ldy < cols) return AF3_ERR_BAD_ARG;
+  const int64_t blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  hipLaunchKernelGGL(softmax_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, mask, y, rows, cols, ldy);
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+int launch_narrow_linear_f32(const float* x, const float* w, const float* res, float* y, int64_t rows, int k, int n_out,
+                             int relu_in, hipStream_t stream) {
+  if (!x || !w || !y || rows <= 0 || k <= 0 || k > 128 || (k & 3)) return AF3_ERR_BAD_ARG;
+  if (n_out != 16 && n_out != 3) return AF3_ERR_UNSUPPORTED;
+  if ((uintptr_t)x & 15) return AF3_ERR_BAD_ARG;
+  const int64_t blocks = (rows + 255) / 256;
+  if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  const dim3 grid((unsigned)blocks), block(256);
+  if (n_out == 16) hipLaunchKernelGGL(narrow_linear_f32_kernel<16>, grid, block, 0, stream, x, w, res, y, rows, k, relu_in);
+  else hipLaunchKernelGGL(narrow_linear_f32_kernel<3>, grid, block, 0, stream, x, w, res, y, rows, k, relu_in);
   return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }

@@ -19,7 +19,6 @@ from typing import Any, Optional
 
 import torch
 import torch.nn as nn
-import torch.nn.functional as F
 
 from .. import check, ops
 from .atom_layout import GatherInfo, convert
@@ -27,16 +26,19 @@ from .base import HipModule, bf16, drop_mesh, f32, in_check_mode
 from .diffusion_transformer import DiffusionCrossAttTransformer
 
 
-def _lin(x: torch.Tensor, layer: nn.Linear) -> torch.Tensor:
-    """fp32 product with a narrow weight (K of 1 or 3 as explicit FMAs)."""
+def _lin(x: torch.Tensor, layer: nn.Linear, relu_input: bool = False, residual=None) -> torch.Tensor:
+    """fp32 product with a narrow weight: K of 1 or 3 as explicit FMAs, the 128 -> 16 / 16 -> 16 /
+    128 -> 3 layers on the narrow fp32 kernel (optionally relu on the way in, a residual on the way out)."""
     w = layer.weight.float()
     x = x.float()
     if w.shape[1] <= 4:
+        if relu_input:
+            x = torch.relu(x)
         out = x[..., 0:1] * w[:, 0]
         for j in range(1, w.shape[1]):
             out = out + x[..., j:j + 1] * w[:, j]
-        return out
-    return F.linear(x, w)
+        return out if residual is None else out + residual
+    return ops.narrow_linear_f32(x.contiguous(), w.contiguous(), relu_input, residual)
 
 
 def _ln_lin(x: torch.Tensor, norm: nn.LayerNorm, layer: nn.Linear, ln_w, w_bf16) -> torch.Tensor:
@@ -135,9 +137,8 @@ class AtomCrossAttEncoder(HipModule):
         for j in range(4):
             act = act + wn[j][chars[..., j]]
         act = act * m[:, :, None]
-        r = torch.relu(act)
-        pair_act = (_lin(r, self.single_to_pair_cond_row)[:, :, None, :]
-                    + _lin(r, self.single_to_pair_cond_col)[:, None, :, :])
+        pair_act = (_lin(act, self.single_to_pair_cond_row, relu_input=True)[:, :, None, :]
+                    + _lin(act, self.single_to_pair_cond_col, relu_input=True)[:, None, :, :])
         pos = rs.positions.float()
         d = pos[:, :, None, :] - pos[:, None, :, :]
         pair_act = pair_act + _lin(d, self.embed_pair_offsets)
@@ -158,8 +159,8 @@ class AtomCrossAttEncoder(HipModule):
             q_cond = q_cond + convert(aca.tokens_to_queries, ts, (-2,))
         k_cond = convert(aca.queries_to_keys, q_cond, (-3, -2))
         k_mask = convert(aca.queries_to_keys, q_mask, (-2, -1))
-        pair_act = (_lin(torch.relu(q_cond), self.single_to_pair_cond_row_1)[:, :, None, :]
-                    + _lin(torch.relu(k_cond), self.single_to_pair_cond_col_1)[:, None, :, :])
+        pair_act = (_lin(q_cond, self.single_to_pair_cond_row_1, relu_input=True)[:, :, None, :]
+                    + _lin(k_cond, self.single_to_pair_cond_col_1, relu_input=True)[:, None, :, :])
         if trunk_pair_cond is not None:
             tp = _ln_lin(trunk_pair_cond, self.lnorm_trunk_pair_cond, self.embed_trunk_pair_cond,
                          p.get("tp_ln"), p.get("tp_w"))
@@ -179,9 +180,10 @@ class AtomCrossAttEncoder(HipModule):
         pair_act = pair_act + _lin(off, self.embed_pair_offsets_1) * valid
         pair_act = pair_act + _lin(1.0 / (1 + (off * off).sum(-1, keepdim=True)), self.embed_pair_distances_1) * valid
         pair_act = pair_act + _lin(valid, self.embed_pair_offsets_valid)
-        h = _lin(torch.relu(pair_act), self.pair_mlp_1)
-        h = _lin(torch.relu(h), self.pair_mlp_2)
-        pair_act = (pair_act + _lin(torch.relu(h), self.pair_mlp_3)).contiguous()
+        pair_act = pair_act.contiguous()
+        h = _lin(pair_act, self.pair_mlp_1, relu_input=True)
+        h = _lin(h, self.pair_mlp_2, relu_input=True)
+        pair_act = _lin(h, self.pair_mlp_3, relu_input=True, residual=pair_act)
         q_cond, k_cond = q_cond.contiguous(), k_cond.contiguous()
         tcond = None
         if not in_check_mode():
@@ -351,5 +353,5 @@ class AtomCrossAttDecoder(HipModule):
             q_act = check._ln(q_act.contiguous(), self.atom_features_layer_norm)
         else:
             q_act = ops.layer_norm(q_act.contiguous(), p["ln_w"])
-        upd = F.linear(q_act.float(), self.atom_features_to_position_update.weight.float())
+        upd = _lin(q_act, self.atom_features_to_position_update)
         return convert(aca.queries_to_token_atoms, upd, (-3, -2))

@@ -133,8 +133,8 @@ class MSAAttention(HipModule):
         h, d = self.num_head, self.value_dim
         x = ops.layer_norm(msa.contiguous(), p["ln_w"], p["ln_b"])
         logits = ops.pair_logits(pair.contiguous(), p["pn_w"], p["pn_b"], p["w_logits"], h)     # [h, q, k] fp32
-        logits += 1e9 * (msa_mask.float().max(dim=0).values - 1.0)
-        w = _pad_last(torch.softmax(logits, dim=-1).to(torch.bfloat16)).contiguous()              # [h, q, k]
+        # softmax over the keys of logits + 1e9 (key mask - 1), bf16, rows padded to a multiple of 8
+        w = ops.masked_softmax_rows(logits, msa_mask.float().max(dim=0).values.contiguous())        # [h, q, k]
         if n % 8 == 0 and (a * n) % 8 == 0 and c % 8 == 0:
             # Everything with the tokens innermost: the value and gate projections are taken
             # transposed (weights as the left operand), [(h, d), (row, k)], which is per head the

@@ -450,6 +450,42 @@ def transpose2d(x):
     return out
 
 
+def masked_softmax_rows(logits, key_mask, pad_to: int = 8):
+    """softmax over the last axis of fp32 `logits` [..., rows, cols] plus the additive key mask
+    1e9 * (key_mask - 1) (key_mask [cols] 0/1 or None) -> bf16 [..., rows, ld], ld = cols rounded up to
+    `pad_to`, tail columns zero (af3_masked_softmax_rows_forward)."""
+    lib = _L.load()
+    _gpu(logits, "logits", torch.float32)
+    cols = logits.shape[-1]
+    rows = logits.numel() // cols
+    maskf = _mask_f32(key_mask, (cols,), "key_mask")
+    ld = (cols + pad_to - 1) // pad_to * pad_to
+    out = torch.empty(logits.shape[:-1] + (ld,), dtype=torch.bfloat16, device=logits.device)
+    rc = lib.af3_masked_softmax_rows_forward(_p(logits), _p(maskf), _p(out), rows, cols, ld, _stream(logits.device))
+    _L.check(rc, "af3_masked_softmax_rows_forward")
+    return out
+
+
+def narrow_linear_f32(x, w, relu_input: bool = False, residual=None):
+    """y = (residual or 0) + relu?(x) @ w.T in fp32 for the narrow layers of the atom conditioning:
+    x [..., k] fp32, w [n_out, k] fp32 with n_out 16 or 3 and k a multiple of 4 up to 128
+    (af3_narrow_linear_f32_forward)."""
+    lib = _L.load()
+    _gpu(x, "x", torch.float32)
+    _gpu(w, "w", torch.float32)
+    n_out, k = w.shape
+    if x.shape[-1] != k:
+        raise ValueError(f"x: last axis {x.shape[-1]} != {k}")
+    rows = x.numel() // k
+    out = torch.empty(x.shape[:-1] + (n_out,), dtype=torch.float32, device=x.device)
+    if residual is not None:
+        _gpu(residual, "residual", torch.float32, out.shape)
+    rc = lib.af3_narrow_linear_f32_forward(_p(x), _p(w), _p(residual), _p(out), rows, k, n_out, int(bool(relu_input)),
+                                           _stream(x.device))
+    _L.check(rc, "af3_narrow_linear_f32_forward")
+    return out
+
+
 def batched_nt_product(a, b, out=None):
     """out[i] = a[i] @ b[i].T for a [batch, m, k], b [batch, n, k] bf16 (af3_batched_nt_product_forward)."""
     lib = _L.load()

@@ -405,6 +405,27 @@ int af3_linear_forward(
     const void* residual, int res_dtype, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Softmax of the MSA pair-weighted averaging (nn/d_attention.py:131-133): the
+ * pair logits [heads * N][N] fp32 plus the additive key mask 1e9 (mask - 1)
+ * (key_mask [N] fp32 0/1, or NULL), normalised over the keys, as bf16 with rows
+ * out_ld >= cols elements apart and the tail columns zero (the layout the
+ * averaging product reads).
+ */
+int af3_masked_softmax_rows_forward(const float* logits, const float* key_mask, uint16_t* out, int64_t rows,
+                                    int64_t cols, int64_t out_ld, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * The narrow fp32 layers of the atom conditioning (nn/d_atom_cross_attention.py:
+ * 139-140, 161-162, 182-184: single-to-pair conditioning 128 -> 16 and the three
+ * 16 -> 16 layers of the pair MLP; :407-411: the 128 -> 3 position update):
+ *   y[r] = (residual ? residual[r] : 0) + W f(x[r]),  f = relu (relu_input) or identity,
+ * x [rows,k] fp32, W [n_out,k] fp32 (nn.Linear layout), n_out 16 or 3, k a multiple
+ * of 4 up to 128, y and residual [rows,n_out] fp32.  Plain fp32 FMAs.
+ */
+int af3_narrow_linear_f32_forward(const float* x, const float* w, const float* residual, float* y, int64_t rows,
+                                  int k, int n_out, int relu_input, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Diagnostic, no counterpart in the reference.  The dense kernels fetch a
  * column bias in groups (eight entries on the 128x128 tile, four per lane on the
  * 256x256 tile, the last group pulled back to end at column n), and a segmented

@@ -163,6 +163,43 @@ def test_layer_norm_and_adaln(gpu_pkg, c):
     assert_within_bf16_ulp("adaln", got, want, ulps=1.01, atol=1e-5)
 
 
+@pytest.mark.parametrize("rows,cols", [(8 * 37, 37), (8 * 130, 130), (16, 4100)])
+def test_masked_softmax_rows(gpu_pkg, rows, cols):
+    """Softmax of the MSA pair-weighted averaging (nn/d_attention.py:131-133): logits plus the additive
+    key mask, normalised over the keys, bf16 out with zero tail columns."""
+    note(f"test_masked_softmax_rows rows={rows} cols={cols}")
+    g = gen(rows + cols)
+    logits = torch.randn(rows, cols, generator=g) * 3.0
+    mask = (torch.rand(cols, generator=g) > 0.3).float()
+    mask[0] = 1.0
+    got = gpu_pkg.ops.masked_softmax_rows(logits.to(dev()), mask.to(dev()))
+    ld = (cols + 7) // 8 * 8
+    assert got.shape == (rows, ld) and got.dtype == torch.bfloat16
+    want = torch.softmax(logits.double() + 1e9 * (mask.double() - 1.0), dim=-1)
+    assert_within_bf16_ulp("softmax", got[:, :cols], want, ulps=1.01, atol=1e-7)
+    assert float(got[:, cols:].float().abs().max()) == 0.0 if ld > cols else True
+    assert float(got[:, :cols].float().cpu()[:, mask == 0].abs().max()) == 0.0      # masked keys: exactly zero
+    none = gpu_pkg.ops.masked_softmax_rows(logits.to(dev()), None)
+    assert_within_bf16_ulp("softmax, no mask", none[:, :cols], torch.softmax(logits.double(), dim=-1), ulps=1.01, atol=1e-7)
+
+
+@pytest.mark.parametrize("rows,k,n_out", [(1000, 128, 16), (4097, 16, 16), (300, 128, 3)])
+def test_narrow_linear_f32(gpu_pkg, rows, k, n_out):
+    """The narrow fp32 layers of the atom conditioning (nn/d_atom_cross_attention.py:139-140, 161-162,
+    182-184, 407-411): plain fp32 arithmetic, so the float64 product is met to fp32 rounding (the
+    largest error over the maximum value, sums of up to 128 terms: a few 1e-6)."""
+    note(f"test_narrow_linear_f32 rows={rows} k={k} n_out={n_out}")
+    g = gen(rows + k)
+    x, w = torch.randn(rows, k, generator=g), torch.randn(n_out, k, generator=g) * 0.3
+    res = torch.randn(rows, n_out, generator=g)
+    d = dev()
+    assert O.rel_err(gpu_pkg.ops.narrow_linear_f32(x.to(d), w.to(d)).cpu(), x.double() @ w.double().T) < 1e-5
+    got = gpu_pkg.ops.narrow_linear_f32(x.to(d), w.to(d), relu_input=True, residual=res.to(d))
+    assert O.rel_err(got.cpu(), res.double() + torch.relu(x.double()) @ w.double().T) < 1e-5
+    with pytest.raises(gpu_pkg.lib.Af3Error):
+        gpu_pkg.ops.narrow_linear_f32(x.to(d), torch.randn(8, k).to(d))             # 8 outputs: not built
+
+
 # ----------------------------------------------------------------- pair path
 @pytest.mark.parametrize("rows,factor", [(300, 4), (128, 2), (1000, 4)])
 def test_transition128(gpu_pkg, rows, factor):
