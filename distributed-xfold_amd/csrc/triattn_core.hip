@@ -45,7 +45,6 @@
 // Key tiles whose 64 keys are masked in every row of the wave are left out (their
 // probabilities are exactly zero); a row whose keys are ALL masked gets the reference's exact
 // answer, the mean of V, directly.
-#include <cstdlib>
 #include <type_traits>
 
 #include "common.h"
@@ -667,14 +666,8 @@ int launch_triattn_flash(const TriAttnArgs& a, hipStream_t stream) {
   const int QT = (a.N + QW - 1) / QW;
   const int nkt = (a.N + KT - 1) / KT;
   // Two rows per wave once that still leaves every CU several workgroups, one row below that
-  // (and when the per-key mask codes of two rows would not fit the 64 KB of LDS a launch gets
-  // without opting in to more).  AF3_TRIATTN_ROWS=1|2 overrides the choice (for tests).
+  // (and when the per-key mask codes of two rows would not fit the LDS share of a workgroup).
   int R = (int64_t)((a.N + 1) / 2) * H * QT >= 2048 ? 2 : 1;
-  static const int forced = [] {
-    const char* e = getenv("AF3_TRIATTN_ROWS");
-    return e ? atoi(e) : 0;
-  }();
-  if (forced == 1 || forced == 2) R = forced;
   // static LDS: K / V buffers, small arrays; dynamic: the mask codes.  Two workgroups must fit a
   // CU's 160 KB.
   const size_t stat2 = 8 * TILE_BYTES + 512;

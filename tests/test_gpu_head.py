@@ -138,10 +138,12 @@ def test_full_size_head_properties(gpu_pkg):
     with gpu_pkg.nn.check_mode():
         sc32, pc32 = head.pre_conditioning(gb, ge, t, True)
         ref = head(noisy[:1].contiguous(), t[0], gb, ge, sc32[0], pc32)
-    compare("single_cond, bf16 vs fp32 check", sc, sc32, 1e-2, 8e-2)
-    compare("pair_cond, bf16 vs fp32 check", pc, pc32, 1e-2, 8e-2)
+    # caps at 1.25 x the measured figures (rms / max over the rms of the check mode's result: conditioning
+    # 1.8e-3 / 1.0e-2, update after 24 + 6 blocks of bf16 intermediates 8.9e-3 / 5.5e-2)
+    compare("single_cond, bf16 vs fp32 check", sc, sc32, 2.5e-3, 1.3e-2)
+    compare("pair_cond, bf16 vs fp32 check", pc, pc32, 2.5e-3, 1.3e-2)
     skip = 256.0 / (float(t) ** 2 + 256.0) * noisy[:1] * am[None, ..., None]
-    compare("update, bf16 vs fp32 check", out[:1] - skip, ref - skip, 2e-2, 2e-1)
+    compare("update, bf16 vs fp32 check", out[:1] - skip, ref - skip, 1.2e-2, 7e-2)
 
 
 def test_per_atom_key_path_matches_the_gathered_key_tensor_path(gpu_pkg):
