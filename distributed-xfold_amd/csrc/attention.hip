@@ -29,7 +29,13 @@ constexpr float LOG2E = 1.4426950408889634f;
 // per-key code staged in LDS next to the K tile
 constexpr int KEY_MASKED = 1, KEY_PAD = 2, KEY_BEYOND = 4;
 
-template <int KSTEPS, int DVT, int NW>
+// FAST: keys are rows of K / V as they stand (no row table) and the pair bias is present and 16-byte
+// addressable.  Then every address of the key-tile loop is a wave-uniform base that advances by a
+// constant per tile plus a per-lane offset that never changes, and the bias quads are loaded straight
+// into the registers in which the matrix unit accumulates K Q^T on top of them: no address arithmetic
+// and no bias additions in the loop.  The last tile of a key count that is not a multiple of 64 takes
+// the clamped addresses of the general form.
+template <int KSTEPS, int DVT, int NW, bool FAST>
 // at least two waves per SIMD: the register allocator then keeps everything in
 // the 256 architectural VGPRs instead of parking loop state in accumulation
 // registers, which would leave a single wave per SIMD
@@ -45,11 +51,25 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hh = lane >> 5, j = lane & 31;
   const int xaddr = half_swap_addr();
-  // blockIdx.x = (q_tile * H + head) * B + batch: workgroups in flight together
-  // share one (head, q-tile) slab of the pair bias across many batch rows.
-  const int b = blockIdx.x % a.B;
-  const int h = (blockIdx.x / a.B) % a.H;
-  const int q0 = (blockIdx.x / (a.B * a.H)) * (NW * 32) + wave * 32;
+  // Batch entries that share a slab of a non-batched pair bias must meet in one L2 for that slab to be
+  // fetched from memory once: workgroup ids are dealt round-robin to the 8 XCDs, each with an L2 of its
+  // own, so id -> (xcd, slot) -> logical id gives every XCD a contiguous range of logical ids, and
+  // logical = (q_tile * H + head) * B + batch has the sharing entries as its fastest index.
+  int b, h, q0;
+  if (a.bias_mod > 0) {
+    // (windows of a few keys: the workgroups are short and the bias slabs small; plain order)
+    if ((int)blockIdx.x >= a.n_blocks) return;
+    b = blockIdx.x % a.B;
+    h = (blockIdx.x / a.B) % a.H;
+    q0 = (blockIdx.x / (a.B * a.H)) * (NW * 32) + wave * 32;
+  } else {
+    const int per_xcd = (gridDim.x + 7) >> 3;
+    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= a.n_blocks) return;  // workgroup-uniform, before any barrier
+    b = logical % a.B;
+    h = (logical / a.B) % a.H;
+    q0 = (logical / (a.B * a.H)) * (NW * 32) + wave * 32;
+  }
   const int d = a.d;
   const int qi = min(q0 + j, a.Sq - 1);  // clamped for loads; stores are guarded
   const bool q_ok = q0 + j < a.Sq;
@@ -83,40 +103,62 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   //   K: chunk id = key * (KD/8) + c, c fastest (one key row is contiguous)
   //   V: chunk id = c * KT + key, key fastest, so that the transposing 2-byte
   //      LDS stores of a wave walk along a V^T row instead of down a column
+  // The K chunks of a tile and then its V chunks form one list of 2 KCH entries that the threads share out
+  // evenly: thread t moves entries t, t + NT, ..  (head dimension 48 with 256 threads: three each, the
+  // middle one a K chunk for waves 0 and 1 and a V chunk for waves 2 and 3; whether an entry is K or V is
+  // uniform over a wave because KCH is a multiple of 64).
   constexpr int KCH = KT * (KD / 8);
-  constexpr int NLD = (KCH + NT - 1) / NT;
-  u32x4 rk[NLD], rv[NLD];
-  bool k_row_ok[NLD], v_row_ok[NLD];
+  static_assert((2 * KCH) % NT == 0, "the chunk list divides evenly");
+  constexpr int NL = 2 * KCH / NT;
+  u32x4 rc[NL];
+  bool row_ok[NL];
   float rkm = 1.f, rkp = 1.f;  // key mask / key padding flag of key tid (threads 0..63)
   const int bb = a.bias_mod > 0 ? b % a.bias_mod : b;  // batch index of bias / padding masks
   const int* krows = a.key_rows ? a.key_rows + (int64_t)bb * a.Sk : nullptr;
   const float* kmask = a.key_mask ? a.key_mask + (int64_t)b * a.km_sb : nullptr;
   const float* kpad = a.kpad ? a.kpad + (int64_t)bb * a.kp_sb : nullptr;
   int k0_loaded = 0;
-  // Rows of the K / V chunks this thread moves.  With key_rows they are looked
+  // entry i of this thread: K chunk (key = e / (KD/8), c = e % (KD/8)) or V chunk (key = e % KT, c = e / KT)
+  bool is_v[NL];
+  int ch_key[NL], ch_c[NL];
+  // FAST: byte offset of the chunk from the first key row of a tile (the launcher has checked that 64 rows
+  // of K or V span less than 2 GB)
+  uint32_t choff[NL];
+#pragma unroll
+  for (int i = 0; i < NL; ++i) {
+    const int e = tid + i * NT;
+    is_v[i] = e >= KCH;
+    ch_key[i] = is_v[i] ? (e - KCH) % KT : e / (KD / 8);
+    ch_c[i] = is_v[i] ? (e - KCH) / KT : e % (KD / 8);
+    choff[i] = (uint32_t)(ch_key[i] * (is_v[i] ? a.v_ss : a.k_ss) + (ch_c[i] < dch ? ch_c[i] : 0) * 8) * 2u;
+  }
+  // Rows of the chunks this thread moves.  With key_rows they are looked
   // up one tile before the chunks themselves are requested, so that a tile
   // costs one memory round trip, not two in a row.
-  int krow_i[NLD], vrow_i[NLD];
+  int row_i[NL];
   auto gidx = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      const int idx = min(tid + i * NT, KCH - 1);
-      const int key = min(k0 + idx / (KD / 8), a.Sk - 1), vkey = min(k0 + idx % KT, a.Sk - 1);
-      krow_i[i] = krows ? krows[key] : key;
-      vrow_i[i] = krows ? krows[vkey] : vkey;
+    for (int i = 0; i < NL; ++i) {
+      const int key = min(k0 + ch_key[i], a.Sk - 1);
+      row_i[i] = krows ? krows[key] : key;
     }
   };
   auto gload = [&](int k0) {
     k0_loaded = k0;
+    if (FAST && k0 + KT <= a.Sk) {  // (workgroup-uniform)
+      const char* kb = reinterpret_cast<const char*>(kg + (int64_t)k0 * a.k_ss);
+      const char* vb = reinterpret_cast<const char*>(vg + (int64_t)k0 * a.v_ss);
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      const int idx = min(tid + i * NT, KCH - 1);
-      const int c = idx % (KD / 8), vc = idx / KT;
-      const int krow = krow_i[i], vrow = vrow_i[i];
-      k_row_ok[i] = krow >= 0;
-      rk[i] = *reinterpret_cast<const u32x4*>(kg + (int64_t)max(krow, 0) * a.k_ss + (c < dch ? c : 0) * 8);
-      v_row_ok[i] = vrow >= 0;
-      rv[i] = *reinterpret_cast<const u32x4*>(vg + (int64_t)max(vrow, 0) * a.v_ss + (vc < dch ? vc : 0) * 8);
+      for (int i = 0; i < NL; ++i) rc[i] = *reinterpret_cast<const u32x4*>((is_v[i] ? vb : kb) + choff[i]);
+    } else {
+      if constexpr (FAST) gidx(k0);
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {
+        const int row = row_i[i];
+        row_ok[i] = row >= 0;
+        rc[i] = *reinterpret_cast<const u32x4*>((is_v[i] ? vg : kg) + (int64_t)max(row, 0) * (is_v[i] ? a.v_ss : a.k_ss) +
+                                                (ch_c[i] < dch ? ch_c[i] : 0) * 8);
+      }
     }
     if (tid < KT) {
       const int key = min(k0 + tid, a.Sk - 1);
@@ -127,21 +169,18 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   auto sstore = [&](int buf) {
     const u32x4 z = {0, 0, 0, 0};
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      const int idx = tid + i * NT;
-      if (idx >= KCH) continue;
-      const int key = idx / (KD / 8), c = idx % (KD / 8);
-      *reinterpret_cast<u32x4*>(&sK[buf][key * LDK + c * 8]) =
-          (k0_loaded + key < a.Sk && c < dch && k_row_ok[i]) ? rk[i] : z;
-      const int vkey = idx % KT, vc = idx / KT;
-      if (vc * 8 < DVT * 32) {
-        const bool ok = k0_loaded + vkey < a.Sk && vc < dch && v_row_ok[i];
-        const uint32_t w4[4] = {rv[i].x, rv[i].y, rv[i].z, rv[i].w};
+    for (int i = 0; i < NL; ++i) {
+      const int key = ch_key[i], c = ch_c[i];
+      const bool ok = k0_loaded + key < a.Sk && c < dch && (FAST || row_ok[i]);  // (FAST: rows are never negative)
+      const u32x4 vv = ok ? rc[i] : z;
+      if (!is_v[i]) {
+        *reinterpret_cast<u32x4*>(&sK[buf][key * LDK + c * 8]) = vv;
+      } else if (c * 8 < DVT * 32) {
+        const uint32_t w4[4] = {vv.x, vv.y, vv.z, vv.w};
+        bf16_t* dst = &sVt[buf][(c * 8) * LDV + key];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const bf16_t x = (bf16_t)((e & 1) ? (w4[e >> 1] >> 16) : (w4[e >> 1] & 0xffffu));
-          sVt[buf][(vc * 8 + e) * LDV + vkey] = ok ? x : (bf16_t)0;
-        }
+        for (int e = 0; e < 8; ++e)
+          dst[e * LDV] = (bf16_t)((e & 1) ? (w4[e >> 1] >> 16) : (w4[e >> 1] & 0xffffu));
       }
     }
     if (tid < KT) {  // wave 0, all of it (KT = 64)
@@ -164,39 +203,54 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   for (int t = 0; t < DVT; ++t)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
-  float m_run = NEG_INF, l_run = 0.f;  // running maximum in natural units
+  float m_run = NEG_INF, l_run = 0.f;  // softmax base (a maximum seen so far) in natural units, and row sum
 
   // Pair bias (fp32, one row per query): the 8 quads of a 64-key tile are
   // fetched one tile ahead, unconditionally, from addresses clamped into the
   // row (a clamped quad belongs to keys >= Sk, which are masked anyway).
-  const float* bias_row = a.bias ? a.bias + (int64_t)bb * a.bias_sb + (int64_t)h * a.bias_sh + (int64_t)qi * a.bias_sq : nullptr;
+  const float* bias_plane = a.bias ? a.bias + (int64_t)bb * a.bias_sb + (int64_t)h * a.bias_sh : nullptr;  // (uniform)
+  const float* bias_row = a.bias ? bias_plane + (int64_t)qi * a.bias_sq : nullptr;
   const bool q_is_pad = a.qpad ? (a.qpad[(int64_t)bb * a.qp_sb + qi] == 0.f) : false;
-  const bool bias_vec = a.bias && a.Sk >= 4 && ((a.bias_sq & 3) == 0) && ((a.bias_sb & 3) == 0) &&
-                        ((a.bias_sh & 3) == 0) && ((a.bias_squad & 3) == 0) && (((uintptr_t)a.bias & 15) == 0);
+  const bool bias_vec = FAST || (a.bias && a.Sk >= 4 && ((a.bias_sq & 3) == 0) && ((a.bias_sb & 3) == 0) &&
+                                 ((a.bias_sh & 3) == 0) && ((a.bias_squad & 3) == 0) && (((uintptr_t)a.bias & 15) == 0));
   // key k of the row: at k (row-major) or, with quads of four keys as the outer
   // index, at (k / 4) * bias_squad + k % 4
   const int64_t quad_step = a.bias_squad ? a.bias_squad : 4;
   const int last_quad = (a.Sk - 1) & ~3;
-  f32x4 rbias[2][4];
-#pragma unroll
-  for (int u = 0; u < 2; ++u)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) rbias[u][g] = f32x4{0.f, 0.f, 0.f, 0.f};
-  auto gload_bias = [&](int k0) {
+  // FAST: this lane's byte offset from the tile's first quad of the bias plane (checked by the launcher to fit)
+  const uint32_t bias_lane = (uint32_t)((int64_t)qi * a.bias_sq + hh * quad_step) * 4u;
+  // the quads of tile k0 into `dst`, laid out like the score accumulators:
+  // dst[u][4g + e] = bias(query, key k0 + 32u + 8g + 4hh + e)
+  // `part` < 0: all eight quads; 0..3: the two quads (u = part / 2, g = 2 (part % 2) + {0, 1}) only
+  auto gload_bias = [&](f32x16 (&dst)[2], int k0, int part = -1) {
     if (!bias_vec) return;  // workgroup-uniform
+    const bool fast_addr = FAST && k0 + KT <= a.Sk;
+    const char* bt = reinterpret_cast<const char*>(bias_plane + (int64_t)(k0 >> 2) * quad_step);
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int g = 0; g < 4; ++g)
-        rbias[u][g] = *reinterpret_cast<const f32x4*>(
-            bias_row + (int64_t)(min(k0 + u * 32 + 8 * g + 4 * hh, last_quad) >> 2) * quad_step);
+      for (int g = 0; g < 4; ++g) {
+        if (part >= 0 && (u != (part >> 1) || (g >> 1) != (part & 1))) continue;
+        f32x4 v;
+        if (fast_addr) v = *reinterpret_cast<const f32x4*>(bt + (int64_t)(8 * u + 2 * g) * quad_step * 4 + bias_lane);
+        else v = *reinterpret_cast<const f32x4*>(bias_row + (int64_t)(min(k0 + u * 32 + 8 * g + 4 * hh, last_quad) >> 2) * quad_step);
+        dst[u][4 * g] = v.x; dst[u][4 * g + 1] = v.y; dst[u][4 * g + 2] = v.z; dst[u][4 * g + 3] = v.w;
+      }
   };
 
   const int nkt = (a.Sk + KT - 1) / KT;
-  gidx(0);
+  // Two register sets of 2 x 16 values.  FAST: they alternate between the tiles, the set of tile kt + 1
+  // receives that tile's bias while tile kt is worked on and is then accumulated on by the matrix unit.
+  // Otherwise one set holds the scores and the other the prefetched bias, copied over before the products.
+  f32x16 setA[2], setB[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) setA[u][r] = setB[u][r] = 0.f;
+  if constexpr (!FAST) gidx(0);
   gload(0);
-  gidx(KT);
-  gload_bias(0);
+  if constexpr (!FAST) gidx(KT);
+  gload_bias(FAST ? setA : setB, 0);
   // the output gate of the lane's query: asked for now, used after the last tile
   u32x2 gate_w[DVT][4];
 #pragma unroll
@@ -210,41 +264,51 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   sstore(0);
   lds_barrier();
 
-  for (int kt = 0; kt < nkt; ++kt) {
+  // One key tile.  FAST: `s` holds the tile's bias, `other` takes the next tile's.  Otherwise `other`
+  // holds this tile's bias, is copied to `s`, and then takes the next tile's.
+  auto tile = [&](int kt, f32x16 (&s)[2], f32x16 (&other)[2]) {
     const int buf = kt & 1;
     const int k0 = kt * KT;
     // next tile's K / V chunks (their rows are known) and the rows of the one after
     gload((kt + 1) * KT);
-    gidx((kt + 2) * KT);
+    if constexpr (!FAST) gidx((kt + 2) * KT);
+    // FAST: the next tile's bias is requested in four pieces spread over this tile (below).  A wave that
+    // issues a burst of loads sits at them until the CU's address unit, which takes 16 to 64 cycles per wave
+    // instruction and serves eight waves, has accepted them all; spread out, the unit works through them
+    // while the wave computes.
+    auto bias_piece = [&](int part) {
+      if constexpr (FAST) {
+        __builtin_amdgcn_sched_barrier(0);
+        gload_bias(other, (kt + 1) * KT, part);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
     // both 32-key halves through the matrix unit first (two independent chains);
     // s[u][4g + e] = logit(query j, key k0 + 32u + 8g + 4hh + e)
-    f32x16 s[2];
+    // (either form starts the accumulation from the bias, so both give the same bits)
+    if constexpr (!FAST) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[u][r] = 0.f;
+        for (int g = 0; g < 4; ++g)
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks)
-        s[u] = mfma32(lds_frag(sK[buf], LDK, u * 32, ks * 16, lane), qf[ks], s[u]);
+          for (int e = 0; e < 4; ++e) {
+            float bv = 0.f;
+            if (bias_vec) bv = other[u][4 * g + e];
+            else if (bias_row) {
+              const int kc = min(k0 + u * 32 + 8 * g + 4 * hh + e, a.Sk - 1);
+              bv = bias_row[(int64_t)(kc >> 2) * quad_step + (kc & 3)];
+            }
+            s[u][4 * g + e] = bv;
+          }
+      gload_bias(other, (kt + 1) * KT);  // the next tile's bias into the registers just read
     }
-    // bias, then the next tile's bias into the registers just freed
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        if (bias_vec) {
-          s[u][4 * g] += rbias[u][g].x; s[u][4 * g + 1] += rbias[u][g].y;
-          s[u][4 * g + 2] += rbias[u][g].z; s[u][4 * g + 3] += rbias[u][g].w;
-        } else if (bias_row) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int key = k0 + u * 32 + 8 * g + 4 * hh + e;
-            const int kc = min(key, a.Sk - 1);
-            s[u][4 * g + e] += bias_row[(int64_t)(kc >> 2) * quad_step + (kc & 3)];
-          }
-        }
-      }
-    gload_bias((kt + 1) * KT);
+      for (int ks = 0; ks < KSTEPS; ++ks)
+        s[u] = mfma32(lds_frag(sK[buf], LDK, u * 32, ks * 16, lane), qf[ks], s[u]);
+    bias_piece(0);
     // Masks from the per-key codes; most tiles carry none (a workgroup-uniform
     // test skips the block).  The logits stay in natural units: the maximum
     // does not care, and exp2 takes fma(s, log2 e, -m log2 e).  (For a row
@@ -280,7 +344,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
     const float t9c = fmaxf(fmaxf(t3[6], t3[7]), t3[8]), t9d = fmaxf(t3[9], t3[10]);
     float mx = fmaxf(fmaxf(fmaxf(t9a, t9b), t9c), t9d);
     mx = fmaxf(mx, half_swap(xaddr, mx));
-    const float m_new = fmaxf(m_run, mx);
+    bias_piece(1);
+    // The base of the exponentials follows the maximum lazily: it moves only when a tile's maximum
+    // exceeds it by more than BASE_SLACK (weights then reach e^BASE_SLACK at most, far inside fp32 and
+    // bf16 range; the normalisation at the end takes the common factor out again), so that most tiles
+    // leave the output accumulators alone.  The first tile moves it from -inf to its maximum.
+    constexpr float BASE_SLACK = 8.f;
+    const float m_new = mx - m_run > BASE_SLACK ? mx : m_run;
     const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);  // 0 on the first tile (m_run = -inf, m_new finite)
     m_run = m_new;
     const float m2 = m_new * LOG2E;
@@ -293,6 +363,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
 #pragma unroll
         for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[u][8 * half + e], LOG2E, -m2));
         pf[u][half] = as_frag(pack8(pv));
+        if (half == 1) bias_piece(2 + u);
       }
     // row sums of the ROUNDED probabilities on the matrix unit (ones * P), so
     // that the weights that multiply V sum to exactly one after normalisation
@@ -327,6 +398,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
         }
     if (kt + 1 < nkt) sstore(buf ^ 1);
     lds_barrier();
+  };
+  if constexpr (FAST) {
+    for (int kt = 0; kt < nkt; kt += 2) {
+      tile(kt, setA, setB);
+      if (kt + 1 < nkt) tile(kt + 1, setB, setA);
+    }
+  } else {
+    for (int kt = 0; kt < nkt; ++kt) tile(kt, setA, setB);
   }
 
   const float inv = 1.f / l_run;  // the ones * P sums cover both half-waves' keys
@@ -368,11 +447,34 @@ int launch_nw(const FlashArgs& a, hipStream_t stream) {
   // workgroups to cover the chip; below that, two waves per workgroup spread
   // the work over twice as many CUs.
   const int nw = a.Sq <= 32 ? 1 : (((a.Sq + 127) / 128) * heads < 256 ? 2 : 4);
-  const int64_t blocks = (int64_t)((a.Sq + nw * 32 - 1) / (nw * 32)) * heads;
-  if (blocks <= 0 || blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
-  if (nw == 1) hipLaunchKernelGGL((flash_kernel<KSTEPS, DVT, 1>), dim3((unsigned)blocks), dim3(64), 0, stream, a);
-  else if (nw == 2) hipLaunchKernelGGL((flash_kernel<KSTEPS, DVT, 2>), dim3((unsigned)blocks), dim3(128), 0, stream, a);
-  else hipLaunchKernelGGL((flash_kernel<KSTEPS, DVT, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  const int64_t n_blocks = (int64_t)((a.Sq + nw * 32 - 1) / (nw * 32)) * heads;
+  if (n_blocks <= 0 || n_blocks > 0x7ffffff0) return AF3_ERR_BAD_ARG;
+  FlashArgs fa = a;
+  fa.n_blocks = (int)n_blocks;
+  const dim3 grid((unsigned)((n_blocks + 7) / 8 * 8));  // whole rounds over the 8 XCDs; the surplus ids return at once
+  // The form with fixed per-lane offsets: no row table, a bias that can be fetched 16 bytes at a time, and
+  // offsets inside a key tile / a bias plane that fit 32 bits.
+  const int64_t quad_step = a.bias_squad ? a.bias_squad : 4;
+  const bool fast = !a.key_rows && a.bias && a.Sk >= 4 && (a.bias_sq & 3) == 0 && (a.bias_sb & 3) == 0 &&
+                    (a.bias_sh & 3) == 0 && (a.bias_squad & 3) == 0 && ((uintptr_t)a.bias & 15) == 0 &&
+                    a.k_ss > 0 && a.v_ss > 0 && a.k_ss < (1 << 22) && a.v_ss < (1 << 22) && a.bias_sq >= 0 &&
+                    quad_step > 0 && (int64_t)a.Sq * a.bias_sq + quad_step < (1 << 28);
+  // (with a single wave, or with head dimension 48 and fewer than four waves, to share the K / V staging
+  // registers between, the second register set of that form no longer fits: those take the general form)
+#define AF3_FLASH_LAUNCH(NW_)                                                                                   \
+  do {                                                                                                          \
+    if constexpr (NW_ == 4 || (KSTEPS < 3 && NW_ == 2)) {                                                       \
+      if (fast) {                                                                                               \
+        hipLaunchKernelGGL((flash_kernel<KSTEPS, DVT, NW_, true>), grid, dim3(NW_ * 64), 0, stream, fa);        \
+        break;                                                                                                  \
+      }                                                                                                         \
+    }                                                                                                           \
+    hipLaunchKernelGGL((flash_kernel<KSTEPS, DVT, NW_, false>), grid, dim3(NW_ * 64), 0, stream, fa);           \
+  } while (0)
+  if (nw == 1) AF3_FLASH_LAUNCH(1);
+  else if (nw == 2) AF3_FLASH_LAUNCH(2);
+  else AF3_FLASH_LAUNCH(4);
+#undef AF3_FLASH_LAUNCH
   return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }
 
@@ -388,7 +490,7 @@ int launch_flash_attention(const FlashArgs& a, hipStream_t stream) {
       ((uintptr_t)a.out & 15))
     return AF3_ERR_BAD_ARG;
   if ((a.qpad == nullptr) != (a.kpad == nullptr)) return AF3_ERR_BAD_ARG;
-  if (a.key_rows && (a.bias_mod <= 0 || a.B % a.bias_mod)) return AF3_ERR_BAD_ARG;
+  if (a.bias_mod < 0 || (a.bias_mod > 0 && a.B % a.bias_mod) || (a.key_rows && a.bias_mod <= 0)) return AF3_ERR_BAD_ARG;
   if (a.bias_squad && (a.bias_sq != 4 || (a.bias_squad & 3))) return AF3_ERR_BAD_ARG;
   if (a.d == 48) return launch_nw<3, 2>(a, stream);
   if (a.d == 16) return launch_nw<1, 1>(a, stream);

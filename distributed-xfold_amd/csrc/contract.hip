@@ -545,13 +545,15 @@ int launch_big_tile(const GemmArgs& g, int mode, hipStream_t stream) {
               ? prop.multiProcessorCount
               : 256;
   }
-  const bool flat = mode == BIG_PLAIN && ((total3 + cus - 1) / cus) * 7 < ((total4 + cus - 1) / cus) * 8;
+  const bool flat = ((total3 + cus - 1) / cus) * 7 < ((total4 + cus - 1) / cus) * 8;
   const int64_t total = flat ? total3 : total4;
   if (total > 0x3fffffff) return AF3_ERR_BAD_ARG;
   // persistent workgroups, one per CU (a multiple of 8: ids are dealt round-robin to the 8 XCDs)
   const int64_t blocks = std::min<int64_t>((total + 7) / 8 * 8, std::max(cus / 8 * 8, 8));
   const dim3 grid((unsigned)blocks), block(256);
-  if (flat) hipLaunchKernelGGL((contract_kernel<BIG_PLAIN, 3>), grid, block, 0, stream, g);
+  if (flat && mode == BIG_PLAIN) hipLaunchKernelGGL((contract_kernel<BIG_PLAIN, 3>), grid, block, 0, stream, g);
+  else if (flat && mode == BIG_COLUMN_OPS) hipLaunchKernelGGL((contract_kernel<BIG_COLUMN_OPS, 3>), grid, block, 0, stream, g);
+  else if (flat) hipLaunchKernelGGL((contract_kernel<BIG_SWIGLU, 3>), grid, block, 0, stream, g);
   else if (mode == BIG_PLAIN) hipLaunchKernelGGL(contract_kernel<BIG_PLAIN>, grid, block, 0, stream, g);
   else if (mode == BIG_COLUMN_OPS) hipLaunchKernelGGL(contract_kernel<BIG_COLUMN_OPS>, grid, block, 0, stream, g);
   else hipLaunchKernelGGL(contract_kernel<BIG_SWIGLU>, grid, block, 0, stream, g);

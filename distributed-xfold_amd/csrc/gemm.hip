@@ -22,7 +22,8 @@ constexpr int LDT = BK + 8;  // padded LDS row (bf16 elements): 144 B keeps 16-B
 
 constexpr int LDC_S = BN + 4;  // fp32 staging row stride of the C tile
 
-template <bool OUT_F32>
+// K_TAIL: K is not a multiple of the slab depth, so chunks past K have to be zeroed on their way to LDS.
+template <bool OUT_F32, bool K_TAIL>
 __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
   // A/B slabs, double buffered; after the k loop the same memory stages the C tile
   __shared__ __attribute__((aligned(16))) bf16_t smem[2 * (BM + BN) * LDT];
@@ -81,8 +82,8 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = ld_row + 32 * i;
-      *reinterpret_cast<u32x4*>(smem + buf * STAGE + row * LDT + ld_kc) = k_ok[set] ? ra[set][i] : z;
-      *reinterpret_cast<u32x4*>(smem + buf * STAGE + (BM + row) * LDT + ld_kc) = k_ok[set] ? rb[set][i] : z;
+      *reinterpret_cast<u32x4*>(smem + buf * STAGE + row * LDT + ld_kc) = !K_TAIL || k_ok[set] ? ra[set][i] : z;
+      *reinterpret_cast<u32x4*>(smem + buf * STAGE + (BM + row) * LDT + ld_kc) = !K_TAIL || k_ok[set] ? rb[set][i] : z;
     }
   };
 
@@ -122,16 +123,26 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(fa[i], fb[j], acc[i][j]);
     }
-    // fragment reads four ahead of the MFMAs that use them
+    // The next slab (requested one stage ago) goes into the other LDS buffer, which nobody reads during
+    // this stage, while the matrix unit works: its eight stores are dealt out between the MFMAs of the
+    // second half, behind the fragment reads (issued four ahead of the MFMAs that use them).  Unconditional,
+    // so that it stays in one basic block with them: after the last slab it stores a clamped re-read that
+    // nobody uses (the C tile is staged over it only after the barrier below).
+    sstore(par ^ 1, par ^ 1);
     __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-    for (int i = 0; i < 12; ++i) {
+    for (int i = 0; i < 4; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    }
     __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
     __builtin_amdgcn_sched_barrier(0);
-    if (kt + 1 < nk) sstore(par ^ 1, par ^ 1);
     lds_barrier();
   };
   for (int kt = 0; kt < nk; kt += 2) {
@@ -338,7 +349,10 @@ int launch_gemm_nt(const GemmArgs& g_in, hipStream_t stream) {
   const int64_t blocks = (total + 7) / 8 * 8;
   if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
   dim3 grid((unsigned)blocks);
-  if (g.out_f32) hipLaunchKernelGGL(gemm_nt_kernel<true>, grid, dim3(256), 0, stream, g);
-  else hipLaunchKernelGGL(gemm_nt_kernel<false>, grid, dim3(256), 0, stream, g);
+  const bool k_tail = (g.K % BK) != 0;
+  if (g.out_f32 && k_tail) hipLaunchKernelGGL((gemm_nt_kernel<true, true>), grid, dim3(256), 0, stream, g);
+  else if (g.out_f32) hipLaunchKernelGGL((gemm_nt_kernel<true, false>), grid, dim3(256), 0, stream, g);
+  else if (k_tail) hipLaunchKernelGGL((gemm_nt_kernel<false, true>), grid, dim3(256), 0, stream, g);
+  else hipLaunchKernelGGL((gemm_nt_kernel<false, false>), grid, dim3(256), 0, stream, g);
   return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }

@@ -206,6 +206,7 @@ struct FlashArgs {
   // of the K / V table of sample b / bias_mod (k_sb / v_sb: table stride); a
   // negative row is a key with zero K and V.  Null: key s is row s of batch b.
   const int* key_rows = nullptr;
+  int n_blocks = 0;  // workgroups that have work (set by the launcher; the grid is rounded up to a multiple of 8)
 };
 int launch_flash_attention(const FlashArgs& a, hipStream_t stream);
 
