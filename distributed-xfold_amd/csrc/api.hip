@@ -396,6 +396,22 @@ int af3_narrow_linear_f32_forward(const float* x, const float* w, const float* r
   return launch_narrow_linear_f32(x, w, residual, y, rows, k, n_out, relu_input, static_cast<hipStream_t>(stream));
 }
 
+int af3_pair_cond_init_forward(const void* pair, int pair_dtype, float in_scale, const int32_t* asym_id,
+                               const int32_t* residue_index, const int32_t* token_index, const int32_t* entity_id,
+                               const int32_t* sym_id, int max_relative_idx, int max_relative_chain, const float* ln_w,
+                               const uint16_t* w_pair, const float* g_hot, const float* g_sum, float* out, int64_t n,
+                               af3_stream_t stream) {
+  if (bad_dtype(pair_dtype) || n <= 0 || n > 0x7fff) return AF3_ERR_BAD_ARG;
+  PairCondInitArgs a;
+  a.pair = pair; a.io_f32 = pair_dtype == AF3_F32; a.N = (int)n; a.in_scale = in_scale;
+  a.asym_id = asym_id; a.residue_index = residue_index; a.token_index = token_index; a.entity_id = entity_id;
+  a.sym_id = sym_id;
+  a.max_rel_idx = max_relative_idx; a.max_rel_chain = max_relative_chain;
+  a.n_rel = 4 * max_relative_idx + 2 * max_relative_chain + 7;
+  a.ln_w = ln_w; a.w_pair = w_pair; a.g_hot = g_hot; a.g_sum = g_sum; a.out = out;
+  return launch_pair_cond_init(a, static_cast<hipStream_t>(stream));
+}
+
 // -------------------------------------------------------------------- transpose
 int af3_transpose_bf16_forward(const uint16_t* in, uint16_t* out, int64_t rows, int64_t cols, af3_stream_t stream) {
   return launch_transpose(in, out, rows, cols, static_cast<hipStream_t>(stream));

@@ -156,6 +156,23 @@ struct AttnProjArgs {
 };
 int launch_attn_proj(const AttnProjArgs& a, hipStream_t s);
 
+// pair_cond = Linear(LayerNorm([pair | relative encoding of the token pair])) without the concatenated
+// tensor (pair_tile.hip).  The relative encoding has n_rel = 4 max_rel_idx + 2 max_rel_chain + 7 one-hot
+// channels; g_hot[h][o] = ln_w[128 + h] * W[o][128 + h] and g_sum[o] = sum_h g_hot[h][o].
+struct PairCondInitArgs {
+  const void* pair = nullptr;  // [N][N][128], fp32 or bf16
+  int io_f32 = 1, N = 0;
+  float in_scale = 1.f;        // the pair values are multiplied by this first
+  const int *asym_id = nullptr, *residue_index = nullptr, *token_index = nullptr, *entity_id = nullptr, *sym_id = nullptr;  // [N]
+  int max_rel_idx = 32, max_rel_chain = 2, n_rel = 139;
+  const float* ln_w = nullptr;     // [128] LayerNorm weights of the pair channels
+  const bf16_t* w_pair = nullptr;  // [128][128] projection weights of the pair channels
+  const float* g_hot = nullptr;    // [n_rel][128]
+  const float* g_sum = nullptr;    // [128]
+  float* out = nullptr;            // [N][N][128] fp32
+};
+int launch_pair_cond_init(const PairCondInitArgs& a, hipStream_t s);
+
 struct AttnOutArgs {
   LnWidth lw;
   const bf16_t* og = nullptr;  // [(b*N + s)][ld_og] attention output, normalised, not yet gated

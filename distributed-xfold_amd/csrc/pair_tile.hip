@@ -644,6 +644,114 @@ __global__ __launch_bounds__(256, 2) void transition_kernel(TransitionArgs a) {
   store_tile_f32<TIO>(sS, t, reinterpret_cast<TIO*>(a.out), a.residual ? x : nullptr, tid);
 }
 
+// ============================================================================
+// diffusion conditioning: pair_cond = Linear(LayerNorm([pair | relative encoding]))
+// ============================================================================
+// The 267 input channels of a pixel (i, j) are the 128 pair channels and 139 one-hot channels of the
+// relative encoding: clipped residue offset inside a chain (2r + 2 classes), clipped token offset inside a
+// residue (2r + 2), same entity (1), clipped chain-copy offset inside an entity (2c + 2); r = 32, c = 2.
+// The concatenated tensor is never made.  A pixel holds n1 = 3 + same_entity ones, so its LayerNorm
+// statistics are mean = (sum x + n1) / 267, E[x^2] = (sum x^2 + n1) / 267, and with the weight rows of the
+// one-hot channels h folded with their LayerNorm weights, G[h][o] = ln_w[h] W[o][h],
+//   out[o] = sum_{c < 128} LN(x)_c W[o][c]  +  rstd * (sum_{hot h} G[h][o]  -  mean * sum_h G[h][o]).
+// The first term is the tile product of the other kernels here (LayerNorm-ed pixels as bf16 fragments);
+// the second is four rows of a 139 x 128 fp32 table per pixel, added in fp32.
+template <typename TIO>
+__global__ __launch_bounds__(256, 2) void pair_cond_init_kernel(PairCondInitArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t smem[2 * TM * LDX];
+  bf16_t* sX = smem;
+  bf16_t* sW = smem + TM * LDX;
+  float* sS = reinterpret_cast<float*>(smem);
+  __shared__ float sRstd[TM], sMeanRstd[TM];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const Tile t = make_tile(a.N, false);
+  const TIO* x = reinterpret_cast<const TIO*>(a.pair);
+  using E = Elem<TIO>;
+  constexpr int NB = E::kBatch;
+  const int chunk = tid & 15, prow = tid >> 4;
+  const int i = t.o;
+  const int ent_i = a.entity_id[i];
+  const float inv_c = 1.f / (float)(C + a.n_rel);
+
+  WChunkRegs wr;
+  wr.load(a.w_pair, tid);
+  float w[8];
+  load_param8(a.ln_w + chunk * 8, 1.f, w);
+#pragma unroll
+  for (int base = 0; base < 8; base += NB) {
+    typename E::Raw raw[NB];
+    int ent_j[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int p = (base + b) * 16 + prow;
+      const int pc = t.valid(p) ? p : 0;
+      raw[b] = E::load_raw(x + t.pix(pc) * C + chunk * 8);
+      ent_j[b] = a.entity_id[t.r0 + pc];
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int p = (base + b) * 16 + prow;
+      float v[8], o[8];
+      E::unpack_raw(raw[b], v);
+      float s = 0.f, q = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { v[e] *= a.in_scale; s += v[e]; q = fmaf(v[e], v[e], q); }
+      const float n1 = 3.f + (ent_j[b] == ent_i ? 1.f : 0.f);
+      const float mean = (group16_sum(s) + n1) * inv_c;
+      const float var = fmaxf(fmaf(group16_sum(q) + n1, inv_c, -mean * mean), 0.f);
+      const float rstd = rsqrtf(var + LN_EPS);
+      const float shift = -mean * rstd;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = fmaf(v[e], rstd, shift) * w[e];
+      u32x4 pk = pack8(o);
+      if (!t.valid(p)) pk = u32x4{0u, 0u, 0u, 0u};
+      *reinterpret_cast<u32x4*>(sX + p * LDX + chunk * 8) = pk;
+      if (chunk == 0) { sRstd[p] = rstd; sMeanRstd[p] = mean * rstd; }
+    }
+  }
+  wr.store(sW, tid);
+  lds_barrier();
+  bf16x8 xf[8];
+  load_x_frags(sX, wave, lane, xf);
+  f32x16 acc[4];
+  mfma_chunk<true, 4>(xf, sW, lane, acc);
+
+  // the lane's pixel: its four hot rows of the table
+  const int px = wave * 32 + (lane & 31), hh = lane >> 5;
+  const int j = t.r0 + (t.valid(px) ? px : 0);
+  const int r = a.max_rel_idx, c2 = a.max_rel_chain;
+  const bool same_chain = a.asym_id[i] == a.asym_id[j];
+  const int dres = a.residue_index[i] - a.residue_index[j];
+  const int h_res = same_chain ? min(max(dres + r, 0), 2 * r) : 2 * r + 1;
+  const int h_tok = (same_chain && dres == 0) ? min(max(a.token_index[i] - a.token_index[j] + r, 0), 2 * r) : 2 * r + 1;
+  const bool same_ent = a.entity_id[j] == ent_i;
+  const int h_sym = same_ent ? min(max(a.sym_id[i] - a.sym_id[j] + c2, 0), 2 * c2) : 2 * c2 + 1;
+  const float* g0 = a.g_hot + (int64_t)h_res * C;
+  const float* g1 = a.g_hot + (int64_t)(2 * r + 2 + h_tok) * C;
+  const float* g2 = a.g_hot + (int64_t)(4 * r + 4) * C;              // same entity
+  const float* g3 = a.g_hot + (int64_t)(4 * r + 5 + h_sym) * C;
+  const float ent_f = same_ent ? 1.f : 0.f;
+  const float rstd = sRstd[px], mrstd = sMeanRstd[px];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int ch = nt * 32 + 8 * g + 4 * hh;
+      const f32x4 v0 = *reinterpret_cast<const f32x4*>(g0 + ch), v1 = *reinterpret_cast<const f32x4*>(g1 + ch);
+      const f32x4 v2 = *reinterpret_cast<const f32x4*>(g2 + ch), v3 = *reinterpret_cast<const f32x4*>(g3 + ch);
+      const f32x4 so = *reinterpret_cast<const f32x4*>(a.g_sum + ch);
+      const float hot[4] = {v0.x + v1.x + ent_f * v2.x + v3.x, v0.y + v1.y + ent_f * v2.y + v3.y,
+                            v0.z + v1.z + ent_f * v2.z + v3.z, v0.w + v1.w + ent_f * v2.w + v3.w};
+      const float sum[4] = {so.x, so.y, so.z, so.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[nt][4 * g + e] += rstd * hot[e] - mrstd * sum[e];
+    }
+  lds_barrier();
+  stage_t_f32(acc, sS, wave, lane);
+  lds_barrier();
+  store_tile_f32<float>(sS, t, a.out, nullptr, tid);
+}
+
 template <typename K, typename A>
 int launch_tiles(K kern, const A& a, int64_t n_outer, int N, hipStream_t stream) {
   const int64_t tiles = n_outer * ((N + TM - 1) / TM);
@@ -687,6 +795,17 @@ int launch_attn_out(const AttnOutArgs& a, hipStream_t s) {
     return AF3_ERR_BAD_ARG;
   return a.io_f32 ? launch_tiles(attn_out_kernel<float>, a, a.N, a.N, s)
                   : launch_tiles(attn_out_kernel<bf16_t>, a, a.N, a.N, s);
+}
+int launch_pair_cond_init(const PairCondInitArgs& a, hipStream_t s) {
+  if (a.N <= 0 || !a.pair || !a.out || !a.w_pair || !a.ln_w || !a.g_hot || !a.g_sum || !a.asym_id || !a.residue_index ||
+      !a.token_index || !a.entity_id || !a.sym_id)
+    return AF3_ERR_BAD_ARG;
+  if (a.max_rel_idx < 0 || a.max_rel_chain < 0 || a.n_rel != 4 * a.max_rel_idx + 2 * a.max_rel_chain + 7) return AF3_ERR_BAD_ARG;
+  if (!aligned16(a.pair) || !aligned16(a.out) || !aligned16(a.w_pair) || !aligned16(a.g_hot) || !aligned16(a.g_sum) ||
+      !aligned16(a.ln_w))
+    return AF3_ERR_BAD_ARG;
+  return a.io_f32 ? launch_tiles(pair_cond_init_kernel<float>, a, a.N, a.N, s)
+                  : launch_tiles(pair_cond_init_kernel<bf16_t>, a, a.N, a.N, s);
 }
 int launch_transition(const TransitionArgs& a, hipStream_t s) {
   // x is [rows][128]; handled as `rows` positions in one long row

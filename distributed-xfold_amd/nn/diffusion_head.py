@@ -148,7 +148,13 @@ class DiffusionHead(HipModule):
         return bf16(F.pad(w.detach().float(), (0, (-k) % 8)))
 
     def _pack(self):
+        # first layer of the pair conditioning (ops.pair_cond_init): the pair channels' LayerNorm weights and
+        # projection columns, and the one-hot channels' columns folded with their LayerNorm weights
+        cp = self.pair_channel
+        wp, gp = self.pair_cond_initial_projection.weight.detach().float(), self.pair_cond_initial_norm.weight.detach().float()
+        g_hot = (wp[:, cp:] * gp[cp:]).t().contiguous()
         return dict(w_pair0=self._pad_k(self.pair_cond_initial_projection.weight),
+                    pair_ln=f32(gp[:cp]), w_pair=bf16(wp[:, :cp]), g_hot=f32(g_hot), g_sum=f32(g_hot.sum(0)),
                     w_single0=self._pad_k(self.single_cond_initial_projection.weight),
                     noise_ln=f32(self.noise_embedding_initial_norm.weight),
                     w_noise=bf16(self.noise_embedding_initial_projection.weight),
@@ -172,13 +178,25 @@ class DiffusionHead(HipModule):
         for the noise levels [T] of all steps."""
         p = self.packed()
         single = use_conditioning * embeddings["single"].float()
-        pair = use_conditioning * embeddings["pair"].float()
-        rel = create_relative_encoding(batch.token_features, 32, 2).to(pair.dtype)
-        f2d = torch.cat([pair, rel], dim=-1)
         f1d = torch.cat([single, embeddings["target_feat"].float()], dim=-1)
-        pair_cond = self._norm_project(f2d, self.pair_cond_initial_norm, self.pair_cond_initial_projection,
-                                       p["w_pair0"])
-        del f2d, rel
+        if in_check_mode() or p["g_hot"].shape[0] != 139:
+            pair = use_conditioning * embeddings["pair"].float()
+            rel = create_relative_encoding(batch.token_features, 32, 2).to(pair.dtype)
+            f2d = torch.cat([pair, rel], dim=-1)
+            pair_cond = self._norm_project(f2d, self.pair_cond_initial_norm, self.pair_cond_initial_projection,
+                                           p["w_pair0"])
+            del f2d, rel
+        else:
+            # one kernel: the relative encoding is one-hot, so its LayerNorm statistics and its share of the
+            # projection follow from the token indices; the [N, N, 267] tensor is never made
+            tf = batch.token_features
+            ids = tuple(getattr(tf, k).to(torch.int32).contiguous()
+                        for k in ("asym_id", "residue_index", "token_index", "entity_id", "sym_id"))
+            pair_in = embeddings["pair"]
+            if pair_in.dtype not in (torch.float32, torch.bfloat16):
+                pair_in = pair_in.float()
+            pair_cond = ops.pair_cond_init(pair_in.contiguous(), ids, p["pair_ln"], p["w_pair"], p["g_hot"], p["g_sum"],
+                                           in_scale=float(use_conditioning), max_relative_idx=32, max_relative_chain=2)
         pair_cond = self._transition(self.pair_transition_0, pair_cond)
         pair_cond = self._transition(self.pair_transition_1, pair_cond)
         noise = self.fourier_embeddings(0.25 * torch.log(noise_level.float() / SIGMA_DATA))

@@ -486,6 +486,34 @@ def narrow_linear_f32(x, w, relu_input: bool = False, residual=None):
     return out
 
 
+def pair_cond_init(pair, token_ids, ln_w, w_pair, g_hot, g_sum, in_scale: float = 1.0,
+                   max_relative_idx: int = 32, max_relative_chain: int = 2):
+    """Linear(LayerNorm([pair | relative encoding])) in one pass (af3_pair_cond_init_forward).
+    pair [N, N, 128] fp32 or bf16; token_ids = (asym_id, residue_index, token_index, entity_id, sym_id), each
+    [N] int32; ln_w [128] fp32; w_pair [128, 128] bf16; g_hot [4 r + 2 c + 7, 128] fp32 and g_sum [128] fp32
+    as DiffusionHead packs them.  Returns [N, N, 128] fp32."""
+    lib = _L.load()
+    _gpu(pair, "pair", None)
+    n = pair.shape[0]
+    if pair.dim() != 3 or pair.shape[1] != n or pair.shape[2] != 128:
+        raise ValueError(f"pair: expected [N, N, 128], got {tuple(pair.shape)}")
+    if len(token_ids) != 5:
+        raise ValueError("token_ids: (asym_id, residue_index, token_index, entity_id, sym_id)")
+    for name, t in zip(("asym_id", "residue_index", "token_index", "entity_id", "sym_id"), token_ids):
+        _gpu(t, name, torch.int32, (n,))
+    n_rel = 4 * max_relative_idx + 2 * max_relative_chain + 7
+    _gpu(ln_w, "ln_w", torch.float32, (128,))
+    _gpu(w_pair, "w_pair", torch.bfloat16, (128, 128))
+    _gpu(g_hot, "g_hot", torch.float32, (n_rel, 128))
+    _gpu(g_sum, "g_sum", torch.float32, (128,))
+    out = torch.empty((n, n, 128), dtype=torch.float32, device=pair.device)
+    rc = lib.af3_pair_cond_init_forward(_p(pair), _dt(pair), float(in_scale), *[_p(t) for t in token_ids],
+                                        int(max_relative_idx), int(max_relative_chain), _p(ln_w), _p(w_pair),
+                                        _p(g_hot), _p(g_sum), _p(out), n, _stream(pair.device))
+    _L.check(rc, "af3_pair_cond_init_forward")
+    return out
+
+
 def batched_nt_product(a, b, out=None):
     """out[i] = a[i] @ b[i].T for a [batch, m, k], b [batch, n, k] bf16 (af3_batched_nt_product_forward)."""
     lib = _L.load()

@@ -426,6 +426,30 @@ int af3_narrow_linear_f32_forward(const float* x, const float* w, const float* r
                                   int k, int n_out, int relu_input, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Pair conditioning of the diffusion head, first layer
+ * (nn/d_diffusion_head.py:104-116: features_2d = [pair | relative encoding],
+ * pair_cond = pair_cond_initial_projection(pair_cond_initial_norm(features_2d))),
+ * in one pass and without the concatenated [n,n,267] tensor.  The relative
+ * encoding of the token pair (i, j) is one-hot: clipped residue offset inside a
+ * chain (2 r + 2 classes, the last for different chains), clipped token offset
+ * inside a residue (2 r + 2), same entity (1), clipped chain-copy offset inside an
+ * entity (2 c + 2); r = max_relative_idx, c = max_relative_chain, n_rel = 4 r + 2 c + 7
+ * channels after the 128 of `pair`.
+ *   pair      [n,n,128] fp32 or bf16 (pair_dtype), multiplied by in_scale first
+ *   asym_id .. sym_id   [n] int32 token features
+ *   ln_w      [128] fp32: LayerNorm weights of the pair channels (the norm has no bias)
+ *   w_pair    [128,128] bf16: projection weights of the pair channels, W[:, :128]
+ *   g_hot     [n_rel,128] fp32: g_hot[h][o] = ln_w[128 + h] * W[o][128 + h]
+ *   g_sum     [128] fp32: sum over h of g_hot[h][o]
+ *   out       [n,n,128] fp32
+ */
+int af3_pair_cond_init_forward(const void* pair, int pair_dtype, float in_scale, const int32_t* asym_id,
+                               const int32_t* residue_index, const int32_t* token_index, const int32_t* entity_id,
+                               const int32_t* sym_id, int max_relative_idx, int max_relative_chain, const float* ln_w,
+                               const uint16_t* w_pair, const float* g_hot, const float* g_sum, float* out, int64_t n,
+                               af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Diagnostic, no counterpart in the reference.  The dense kernels fetch a
  * column bias in groups (eight entries on the 128x128 tile, four per lane on the
  * 256x256 tile, the last group pulled back to end at column n), and a segmented

@@ -75,6 +75,42 @@ def test_pre_conditioning_and_head_against_oracle(gpu_pkg, n, blocks):
                 compare(f"update, step {step}, {mode}", got.double().cpu() - skip, want - skip, rms_tol, max_tol)
 
 
+@pytest.mark.parametrize("n,in_dtype", [(150, torch.float32), (96, torch.bfloat16)])
+def test_pair_conditioning_first_layer_kernel(gpu_pkg, n, in_dtype):
+    """ops.pair_cond_init against LayerNorm + projection of the explicit [pair | relative encoding] tensor
+    in float64, on token features that reach every branch of the encoding: several chains, residues of
+    several tokens (same residue, different token index), offsets beyond the clipping range, chain copies
+    of one entity and chains of different entities."""
+    print(f"test_pair_conditioning_first_layer_kernel n={n} {in_dtype}", flush=True)
+    from types import SimpleNamespace
+    g = gen(300 + n)
+    ri = lambda lo, hi: torch.randint(lo, hi, (n,), generator=g)
+    tf = SimpleNamespace(asym_id=ri(1, 4), residue_index=ri(0, 90) // ri(1, 3).clamp(max=2), token_index=ri(0, 80),
+                         entity_id=ri(1, 3), sym_id=ri(1, 7))
+    tf.residue_index[: n // 3] = tf.residue_index[0]      # a long residue: many tokens share it
+    tf.asym_id[: n // 3] = tf.asym_id[0]
+    pair = O.round_bf16(torch.randn(n, n, 128, generator=g) * 2 + 0.5)
+    ln_w = 1 + 0.2 * torch.randn(267, generator=g)
+    w = O.round_bf16(torch.randn(128, 267, generator=g) * 0.1)
+    scale = 0.75
+    f2d = torch.cat([scale * pair.double(), H.create_relative_encoding(tf).double()], dim=-1)
+    want = torch.nn.functional.layer_norm(f2d, (267,), ln_w.double(), None, 1e-5) @ w.double().T
+    ids = tuple(getattr(tf, k).to(torch.int32).to(dev()) for k in ("asym_id", "residue_index", "token_index", "entity_id", "sym_id"))
+    g_hot = (w[:, 128:].float() * ln_w[128:]).t().contiguous()
+    got = gpu_pkg.ops.pair_cond_init(pair.to(in_dtype).to(dev()), ids, ln_w[:128].contiguous().to(dev()),
+                                     w[:, :128].contiguous().bfloat16().to(dev()), g_hot.to(dev()), g_hot.sum(0).to(dev()),
+                                     in_scale=scale)
+    compare("pair conditioning, first layer", got, want, 3.5e-3, 2e-2)
+    # pair channels switched off: what is left is the one-hot share (fp32 table rows) and the pair channels'
+    # LayerNorm shift; a wrong table row would show at the size of the output itself
+    f2d0 = torch.cat([0 * pair.double(), H.create_relative_encoding(tf).double()], dim=-1)
+    want0 = torch.nn.functional.layer_norm(f2d0, (267,), ln_w.double(), None, 1e-5) @ w.double().T
+    got0 = gpu_pkg.ops.pair_cond_init(pair.to(in_dtype).to(dev()), ids, ln_w[:128].contiguous().to(dev()),
+                                      w[:, :128].contiguous().bfloat16().to(dev()), g_hot.to(dev()), g_hot.sum(0).to(dev()),
+                                      in_scale=0.0)
+    compare("pair conditioning, one-hot share alone", got0, want0, 3e-4, 1e-3)
+
+
 def test_state_reuse_is_exact_and_samples_are_independent(gpu_pkg):
     g, batch, p, emb, pos, head = case(gpu_pkg, 16, 4, seed=31, samples=3)
     gb, ge = batch.to(dev()), on_gpu(emb)
