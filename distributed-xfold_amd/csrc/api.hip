@@ -396,6 +396,25 @@ int af3_narrow_linear_f32_forward(const float* x, const float* w, const float* r
   return launch_narrow_linear_f32(x, w, residual, y, rows, k, n_out, relu_input, static_cast<hipStream_t>(stream));
 }
 
+int af3_atom_pair_cond_forward(const float* row, const float* col, const float* token_pair, const int32_t* query_token,
+                               const int32_t* key_token, int64_t n_token, const float* query_pos, const float* key_pos,
+                               const int32_t* query_uid, const int32_t* key_uid, const float* w_offsets,
+                               const float* w_distances, const float* w_valid, const float* w_mlp1, const float* w_mlp2,
+                               const float* w_mlp3, float* out, int64_t subsets, int64_t queries, int64_t keys,
+                               af3_stream_t stream) {
+  if (queries > 0x7fffffff || keys > 0x7fffffff || n_token > 0x7fff) return AF3_ERR_BAD_ARG;
+  return launch_atom_pair_cond(row, col, token_pair, query_token, key_token, (int)n_token, query_pos, key_pos, query_uid,
+                               key_uid, w_offsets, w_distances, w_valid, w_mlp1, w_mlp2, w_mlp3, out, subsets, (int)queries,
+                               (int)keys, static_cast<hipStream_t>(stream));
+}
+
+int af3_atom_pair_logits_forward(const float* pair_cond, const float* ln_w, const float* w, float* out, int64_t subsets,
+                                 int64_t queries, int64_t keys, int num_blocks, int num_head, af3_stream_t stream) {
+  if (queries <= 0 || keys <= 0) return AF3_ERR_BAD_ARG;
+  return launch_atom_pair_logits(pair_cond, ln_w, w, out, subsets, queries * keys, num_blocks, num_head,
+                                 static_cast<hipStream_t>(stream));
+}
+
 int af3_pair_cond_init_forward(const void* pair, int pair_dtype, float in_scale, const int32_t* asym_id,
                                const int32_t* residue_index, const int32_t* token_index, const int32_t* entity_id,
                                const int32_t* sym_id, int max_relative_idx, int max_relative_chain, const float* ln_w,

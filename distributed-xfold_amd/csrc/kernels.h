@@ -101,6 +101,12 @@ int launch_softmax_rows(const float* x, const float* mask, bf16_t* y, int64_t ro
 // y[r][:] = (res ? res[r][:] : 0) + W relu?(x[r][:]), fp32, W [n_out][k], n_out 16 or 3, k % 4 == 0, k <= 128
 int launch_narrow_linear_f32(const float* x, const float* w, const float* res, float* y, int64_t rows, int k, int n_out,
                              int relu_in, hipStream_t stream);
+int launch_atom_pair_logits(const float* x, const float* ln_w, const float* w, float* out, int64_t n_groups, int64_t group,
+                            int n_blocks, int n_head, hipStream_t stream);
+int launch_atom_pair_cond(const float* row, const float* col, const float* tp, const int* tq, const int* tk, int n_tok,
+                          const float* q_pos, const float* k_pos, const int* q_uid, const int* k_uid, const float* w_off,
+                          const float* w_dist, const float* w_valid, const float* w1, const float* w2, const float* w3,
+                          float* out, int64_t subsets, int queries, int keys, hipStream_t stream);
 
 // -------------------------------------------------------------- pair_tile.hip
 // Residual-stream tensors (`pair`, `out`, `x`) are bf16 or fp32 (io_f32).

@@ -385,6 +385,138 @@ __global__ __launch_bounds__(256) void narrow_linear_f32_kernel(const float* __r
   for (int o = 0; o < NOUT; ++o) y[r * NOUT + o] = acc[o];
 }
 
+
+// ----------------------------------------------------------------------------
+// Pair logits of the windowed atom transformer: per row of 16 conditioning channels a LayerNorm (weight, no
+// bias) and a 16 -> n_out projection, n_out = blocks x heads, each output written to its own
+// [block][subset][head][query][key] plane: the layout the attention kernel reads its bias in.  Rows are
+// (subset, query, key) in this order, `group` = queries x keys rows per subset.  One thread per row, fp32.
+// ----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void atom_pair_logits_kernel(const float* __restrict__ x, const float* __restrict__ ln_w,
+                                                               const float* __restrict__ w, float* __restrict__ out,
+                                                               int64_t rows, int64_t group, int64_t n_groups, int n_blocks,
+                                                               int n_head) {
+  __shared__ __attribute__((aligned(16))) float sW[32 * 16];
+  const int n_out = n_blocks * n_head;
+  // the LayerNorm weight goes into the projection: (xhat * g) . w = xhat . (g * w)
+  for (int i = threadIdx.x; i < n_out * 16; i += 256) sW[i] = w[i] * ln_w[i & 15];
+  __syncthreads();
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= rows) return;
+  float v[16];
+#pragma unroll
+  for (int c = 0; c < 16; c += 4) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(x + r * 16 + c);
+    v[c] = t.x; v[c + 1] = t.y; v[c + 2] = t.z; v[c + 3] = t.w;
+  }
+  float mean = 0.f;
+#pragma unroll
+  for (int c = 0; c < 16; ++c) mean += v[c];
+  mean *= 1.f / 16;
+  float var = 0.f;
+#pragma unroll
+  for (int c = 0; c < 16; ++c) { v[c] -= mean; var = fmaf(v[c], v[c], var); }
+  const float rstd = rsqrtf(var * (1.f / 16) + LN_EPS);
+  const int64_t s = r / group, qk = r - s * group;
+  for (int o = 0; o < n_out; ++o) {
+    float acc = 0.f;
+#pragma unroll
+    for (int c = 0; c < 16; c += 4) {
+      const f32x4 ww = *reinterpret_cast<const f32x4*>(sW + o * 16 + c);
+      acc = fmaf(v[c], ww.x, fmaf(v[c + 1], ww.y, fmaf(v[c + 2], ww.z, fmaf(v[c + 3], ww.w, acc))));
+    }
+    const int blk = o / n_head, h = o - blk * n_head;
+    out[(((int64_t)blk * n_groups + s) * n_head + h) * group + qk] = acc * rstd;
+  }
+}
+
+
+// ----------------------------------------------------------------------------
+// Pair conditioning of the windowed atom attention, one pass per (subset, query, key):
+//   a = row[s,q] + col[s,k] + [both atoms exist] tp[token(s,q), token(s,k)]
+//       + valid * (W_off (pos_q - pos_k) + W_dist / (1 + |pos_q - pos_k|^2)) + valid * w_valid,
+//   valid = the two atoms share a reference frame (uid_q == uid_k),
+//   out = a + W3 relu(W2 relu(W1 relu(a)))                      (16 channels, fp32 throughout).
+// One thread per (s, q, k), the weights in LDS.  Every term used to be a pass of its own over the
+// [S, Q, K, 16] tensor.
+// ----------------------------------------------------------------------------
+struct AtomPairCondArgs {
+  const float *row, *col;           // [S*Q][16], [S*K][16]
+  const float* tp;                  // [n_tok*n_tok][16] or null
+  const int *tq, *tk;               // token of query atom (s,q) / key atom (s,k), negative: no atom
+  const float *q_pos, *k_pos;       // [S*Q][3], [S*K][3]
+  const int *q_uid, *k_uid;
+  const float *w_off, *w_dist, *w_valid, *w1, *w2, *w3;  // [16][3], [16], [16], [16][16] x 3
+  float* out;
+  int64_t S;
+  int Q, K, n_tok;
+};
+
+__global__ __launch_bounds__(256) void atom_pair_cond_kernel(AtomPairCondArgs a) {
+  __shared__ __attribute__((aligned(16))) float sW[3 * 256 + 16 * 4 + 16 + 16];
+  float* sOff = sW + 768;   // [16][4]: w_off rows padded to four
+  float* sDist = sOff + 64;
+  float* sValid = sDist + 16;
+  for (int i = threadIdx.x; i < 768; i += 256) sW[i] = (i < 256 ? a.w1 : i < 512 ? a.w2 : a.w3)[i & 255];
+  if (threadIdx.x < 64) sOff[threadIdx.x] = (threadIdx.x & 3) < 3 ? a.w_off[(threadIdx.x >> 2) * 3 + (threadIdx.x & 3)] : 0.f;
+  if (threadIdx.x < 16) { sDist[threadIdx.x] = a.w_dist[threadIdx.x]; sValid[threadIdx.x] = a.w_valid[threadIdx.x]; }
+  __syncthreads();
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= a.S * a.Q * a.K) return;
+  const int k = (int)(r % a.K);
+  const int64_t sq = r / a.K, sk = (sq / a.Q) * a.K + k;
+  float v[16];
+#pragma unroll
+  for (int c = 0; c < 16; c += 4) {
+    const f32x4 x = *reinterpret_cast<const f32x4*>(a.row + sq * 16 + c), y = *reinterpret_cast<const f32x4*>(a.col + sk * 16 + c);
+    v[c] = x.x + y.x; v[c + 1] = x.y + y.y; v[c + 2] = x.z + y.z; v[c + 3] = x.w + y.w;
+  }
+  if (a.tp) {
+    const int tq = a.tq[sq], tk = a.tk[sk];
+    if (tq >= 0 && tk >= 0) {
+      const float* t = a.tp + ((int64_t)tq * a.n_tok + tk) * 16;
+#pragma unroll
+      for (int c = 0; c < 16; c += 4) {
+        const f32x4 x = *reinterpret_cast<const f32x4*>(t + c);
+        v[c] += x.x; v[c + 1] += x.y; v[c + 2] += x.z; v[c + 3] += x.w;
+      }
+    }
+  }
+  if (a.q_uid[sq] == a.k_uid[sk]) {
+    const float dx = a.q_pos[sq * 3] - a.k_pos[sk * 3], dy = a.q_pos[sq * 3 + 1] - a.k_pos[sk * 3 + 1],
+                dz = a.q_pos[sq * 3 + 2] - a.k_pos[sk * 3 + 2];
+    const float inv = 1.0f / (1.0f + (dx * dx + dy * dy + dz * dz));
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      const f32x4 w = *reinterpret_cast<const f32x4*>(sOff + 4 * c);
+      v[c] += fmaf(dz, w.z, fmaf(dy, w.y, dx * w.x)) + inv * sDist[c] + sValid[c];
+    }
+  }
+  // three 16 x 16 layers with a relu on the way in; the residual is the unactivated a
+  auto layer = [&](const float* w, const float* in, float* out) {
+#pragma unroll
+    for (int o = 0; o < 16; ++o) {
+      float acc = 0.f;
+#pragma unroll
+      for (int c = 0; c < 16; c += 4) {
+        const f32x4 ww = *reinterpret_cast<const f32x4*>(w + o * 16 + c);
+        acc = fmaf(fmaxf(in[c], 0.f), ww.x, fmaf(fmaxf(in[c + 1], 0.f), ww.y,
+                   fmaf(fmaxf(in[c + 2], 0.f), ww.z, fmaf(fmaxf(in[c + 3], 0.f), ww.w, acc))));
+      }
+      out[o] = acc;
+    }
+  };
+  float h1[16], h2[16];
+  layer(sW, v, h1);
+  layer(sW + 256, h1, h2);
+  layer(sW + 512, h2, h1);
+#pragma unroll
+  for (int c = 0; c < 16; c += 4) {
+    const f32x4 o = {v[c] + h1[c], v[c + 1] + h1[c + 1], v[c + 2] + h1[c + 2], v[c + 3] + h1[c + 3]};
+    *reinterpret_cast<f32x4*>(a.out + r * 16 + c) = o;
+  }
+}
+
 }  // namespace
 
 int launch_gather_rows_add(const bf16_t* src, const int* rows, const bf16_t* add, bf16_t* out, int64_t batch,
@@ -477,5 +609,34 @@ int launch_narrow_linear_f32(const float* x, const float* w, const float* res, f
   const dim3 grid((unsigned)blocks), block(256);
   if (n_out == 16) hipLaunchKernelGGL(narrow_linear_f32_kernel<16>, grid, block, 0, stream, x, w, res, y, rows, k, relu_in);
   else hipLaunchKernelGGL(narrow_linear_f32_kernel<3>, grid, block, 0, stream, x, w, res, y, rows, k, relu_in);
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+int launch_atom_pair_logits(const float* x, const float* ln_w, const float* w, float* out, int64_t n_groups, int64_t group,
+                            int n_blocks, int n_head, hipStream_t stream) {
+  if (!x || !ln_w || !w || !out || n_groups <= 0 || group <= 0 || n_blocks <= 0 || n_head <= 0) return AF3_ERR_BAD_ARG;
+  if (n_blocks * n_head > 32) return AF3_ERR_UNSUPPORTED;
+  if ((uintptr_t)x & 15) return AF3_ERR_BAD_ARG;
+  const int64_t rows = n_groups * group, blocks = (rows + 255) / 256;
+  if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  hipLaunchKernelGGL(atom_pair_logits_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, ln_w, w, out, rows, group,
+                     n_groups, n_blocks, n_head);
+  return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+int launch_atom_pair_cond(const float* row, const float* col, const float* tp, const int* tq, const int* tk, int n_tok,
+                          const float* q_pos, const float* k_pos, const int* q_uid, const int* k_uid, const float* w_off,
+                          const float* w_dist, const float* w_valid, const float* w1, const float* w2, const float* w3,
+                          float* out, int64_t subsets, int queries, int keys, hipStream_t stream) {
+  if (!row || !col || !q_pos || !k_pos || !q_uid || !k_uid || !w_off || !w_dist || !w_valid || !w1 || !w2 || !w3 || !out)
+    return AF3_ERR_BAD_ARG;
+  if (subsets <= 0 || queries <= 0 || keys <= 0) return AF3_ERR_BAD_ARG;
+  if (tp && (!tq || !tk || n_tok <= 0)) return AF3_ERR_BAD_ARG;
+  if (((uintptr_t)row & 15) || ((uintptr_t)col & 15) || ((uintptr_t)tp & 15) || ((uintptr_t)out & 15)) return AF3_ERR_BAD_ARG;
+  AtomPairCondArgs a{row, col, tp, tq, tk, q_pos, k_pos, q_uid, k_uid, w_off, w_dist, w_valid, w1, w2, w3, out,
+                     subsets, queries, keys, n_tok};
+  const int64_t blocks = (subsets * queries * keys + 255) / 256;
+  if (blocks > 0x7fffffff) return AF3_ERR_BAD_ARG;
+  hipLaunchKernelGGL(atom_pair_cond_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a);
   return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }

@@ -55,6 +55,9 @@ SIGNATURES = {
     "af3_triangle_contraction_forward": (_i, [_vp, _vp, _vp, _i64, _vp]),
     "af3_masked_softmax_rows_forward": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "af3_narrow_linear_f32_forward": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
+    "af3_atom_pair_cond_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                        _i64, _i64, _i64, _vp]),
+    "af3_atom_pair_logits_forward": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i, _i, _vp]),
     "af3_pair_cond_init_forward": (_i, [_vp, _i, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
     "af3_linear_bias_span": (_i, [_i64, _i, _i, _i, _i, _vp, _vp]),
     "af3_grid_attention_core_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),

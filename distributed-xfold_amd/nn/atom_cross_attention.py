@@ -159,31 +159,48 @@ class AtomCrossAttEncoder(HipModule):
             q_cond = q_cond + convert(aca.tokens_to_queries, ts, (-2,))
         k_cond = convert(aca.queries_to_keys, q_cond, (-3, -2))
         k_mask = convert(aca.queries_to_keys, q_mask, (-2, -1))
-        pair_act = (_lin(q_cond, self.single_to_pair_cond_row_1, relu_input=True)[:, :, None, :]
-                    + _lin(k_cond, self.single_to_pair_cond_col_1, relu_input=True)[:, None, :, :])
-        if trunk_pair_cond is not None:
-            tp = _ln_lin(trunk_pair_cond, self.lnorm_trunk_pair_cond, self.embed_trunk_pair_cond,
-                         p.get("tp_ln"), p.get("tp_w"))
-            n_tok = tp.shape[0]
-            t2q, t2k = aca.tokens_to_queries, aca.tokens_to_keys
-            idx = n_tok * t2q.gather_idxs[:, :, None] + t2k.gather_idxs[:, None, :]
-            msk = t2q.gather_mask[:, :, None] & t2k.gather_mask[:, None, :]
-            pair_act = pair_act + tp.reshape(n_tok * n_tok, -1)[idx] * msk[..., None].float()
         rs = batch.ref_structure
         q_pos = convert(aca.token_atoms_to_queries, rs.positions.float(), (-3, -2))
         q_uid = convert(aca.token_atoms_to_queries, rs.ref_space_uid, (-2, -1))
         k_pos = convert(aca.queries_to_keys, q_pos, (-3, -2))
         # :279-283: the keys' uid is gathered from the token-atom layout with the query-layout gather
         k_uid = convert(aca.queries_to_keys, rs.ref_space_uid, (-2, -1))
-        valid = (q_uid[:, :, None] == k_uid[:, None, :]).float()[..., None]
-        off = q_pos[:, :, None, :] - k_pos[:, None, :, :]
-        pair_act = pair_act + _lin(off, self.embed_pair_offsets_1) * valid
-        pair_act = pair_act + _lin(1.0 / (1 + (off * off).sum(-1, keepdim=True)), self.embed_pair_distances_1) * valid
-        pair_act = pair_act + _lin(valid, self.embed_pair_offsets_valid)
-        pair_act = pair_act.contiguous()
-        h = _lin(pair_act, self.pair_mlp_1, relu_input=True)
-        h = _lin(h, self.pair_mlp_2, relu_input=True)
-        pair_act = _lin(h, self.pair_mlp_3, relu_input=True, residual=pair_act)
+        row = _lin(q_cond, self.single_to_pair_cond_row_1, relu_input=True)
+        col = _lin(k_cond, self.single_to_pair_cond_col_1, relu_input=True)
+        tp = None
+        if trunk_pair_cond is not None:
+            tp = _ln_lin(trunk_pair_cond, self.lnorm_trunk_pair_cond, self.embed_trunk_pair_cond,
+                         p.get("tp_ln"), p.get("tp_w"))
+        t2q, t2k = aca.tokens_to_queries, aca.tokens_to_keys
+        if in_check_mode():
+            pair_act = row[:, :, None, :] + col[:, None, :, :]
+            if tp is not None:
+                n_tok = tp.shape[0]
+                idx = n_tok * t2q.gather_idxs[:, :, None] + t2k.gather_idxs[:, None, :]
+                msk = t2q.gather_mask[:, :, None] & t2k.gather_mask[:, None, :]
+                pair_act = pair_act + tp.reshape(n_tok * n_tok, -1)[idx] * msk[..., None].float()
+            valid = (q_uid[:, :, None] == k_uid[:, None, :]).float()[..., None]
+            off = q_pos[:, :, None, :] - k_pos[:, None, :, :]
+            pair_act = pair_act + _lin(off, self.embed_pair_offsets_1) * valid
+            pair_act = pair_act + _lin(1.0 / (1 + (off * off).sum(-1, keepdim=True)), self.embed_pair_distances_1) * valid
+            pair_act = pair_act + _lin(valid, self.embed_pair_offsets_valid)
+            pair_act = pair_act.contiguous()
+            h = _lin(pair_act, self.pair_mlp_1, relu_input=True)
+            h = _lin(h, self.pair_mlp_2, relu_input=True)
+            pair_act = _lin(h, self.pair_mlp_3, relu_input=True, residual=pair_act)
+        else:
+            # every term above and the three-layer MLP in one pass over the [S, 32, 128, 16] tensor
+            i32 = lambda t: t.to(torch.int32).contiguous()
+            tq = tk = None
+            if tp is not None:
+                tq = i32(torch.where(t2q.gather_mask, t2q.gather_idxs, -1))
+                tk = i32(torch.where(t2k.gather_mask, t2k.gather_idxs, -1))
+                tp = tp.float().contiguous()
+            w = lambda layer: layer.weight.detach().float().contiguous()
+            pair_act = ops.atom_pair_cond(row.contiguous(), col.contiguous(), tp, tq, tk, q_pos.float().contiguous(),
+                                          k_pos.float().contiguous(), i32(q_uid), i32(k_uid), w(self.embed_pair_offsets_1),
+                                          w(self.embed_pair_distances_1), w(self.embed_pair_offsets_valid),
+                                          w(self.pair_mlp_1), w(self.pair_mlp_2), w(self.pair_mlp_3))
         q_cond, k_cond = q_cond.contiguous(), k_cond.contiguous()
         tcond = None
         if not in_check_mode():

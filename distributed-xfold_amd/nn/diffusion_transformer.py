@@ -413,6 +413,7 @@ class DiffusionCrossAttTransformer(HipModule):
                 wg.append(az.adaptive_zero_cond.weight)
                 bg.append(az.adaptive_zero_cond.bias)
         return dict(ln_w=f32(self.pair_input_layer_norm.weight), w=bf16(self.pair_logits_projection.weight),
+                    w_f32=f32(self.pair_logits_projection.weight),
                     w_ss_q=bf16(torch.cat(wq, dim=0)), b_ss_q=f32(torch.cat(bq)),
                     w_ss_k=bf16(torch.cat(wk, dim=0)), b_ss_k=f32(torch.cat(bk)),
                     w_gate=bf16(torch.cat(wg, dim=0)), b_gate=f32(torch.cat(bg)))
@@ -455,10 +456,15 @@ class DiffusionCrossAttTransformer(HipModule):
             key_rows = torch.where(gmask.bool(), idx, torch.full_like(idx, -1)).to(torch.int32).contiguous()
             key_rows._af3_checked_rows = n_atoms
             keys_single_cond = queries_single_cond          # per atom
-        pair_act = ops.layer_norm(pair_cond.contiguous(), p["ln_w"])
-        logits = ops.linear(pair_act, p["w"], out_dtype=torch.float32)           # [S, Q, K, (b h)]
-        s, q, k, _ = logits.shape
-        logits = logits.reshape(s, q, k, self.num_blocks, self.num_head).permute(3, 0, 4, 1, 2).contiguous()
+        if pair_cond.dtype == torch.float32 and pair_cond.dim() == 4 and pair_cond.shape[-1] == 16 \
+                and self.num_blocks * self.num_head <= 32:
+            # LayerNorm, projection and the split into [block][S][head][Q][K] planes in one fp32 pass
+            logits = ops.atom_pair_logits(pair_cond.contiguous(), p["ln_w"], p["w_f32"], self.num_blocks, self.num_head)
+        else:
+            pair_act = ops.layer_norm(pair_cond.contiguous(), p["ln_w"])
+            logits = ops.linear(pair_act, p["w"], out_dtype=torch.float32)           # [S, Q, K, (b h)]
+            s, q, k, _ = logits.shape
+            logits = logits.reshape(s, q, k, self.num_blocks, self.num_head).permute(3, 0, 4, 1, 2).contiguous()
         c = self.c_query
         cq = queries_single_cond.contiguous()
         ck = keys_single_cond.contiguous()

@@ -486,6 +486,63 @@ def narrow_linear_f32(x, w, relu_input: bool = False, residual=None):
     return out
 
 
+def atom_pair_cond(row, col, token_pair, query_token, key_token, query_pos, key_pos, query_uid, key_uid,
+                   w_offsets, w_distances, w_valid, w_mlp1, w_mlp2, w_mlp3):
+    """The [S, Q, K, 16] pair conditioning of the windowed atom attention with its three-layer MLP in one
+    pass (af3_atom_pair_cond_forward).  row [S, Q, 16], col [S, K, 16], token_pair [N, N, 16] or None,
+    query_token [S, Q] / key_token [S, K] int32 (negative: empty slot), positions [S, Q, 3] / [S, K, 3],
+    uids int32, weights fp32 in nn.Linear layout."""
+    lib = _L.load()
+    _gpu(row, "row", torch.float32)
+    s, q, _ = row.shape
+    k = col.shape[1]
+    _gpu(col, "col", torch.float32, (s, k, 16))
+    n_tok = 0
+    if token_pair is not None:
+        _gpu(token_pair, "token_pair", torch.float32)
+        n_tok = token_pair.shape[0]
+        if tuple(token_pair.shape) != (n_tok, n_tok, 16):
+            raise ValueError(f"token_pair: expected [N, N, 16], got {tuple(token_pair.shape)}")
+        _gpu(query_token, "query_token", torch.int32, (s, q))
+        _gpu(key_token, "key_token", torch.int32, (s, k))
+        if int(query_token.max()) >= n_tok or int(key_token.max()) >= n_tok:
+            raise ValueError("token index beyond token_pair")
+    _gpu(query_pos, "query_pos", torch.float32, (s, q, 3))
+    _gpu(key_pos, "key_pos", torch.float32, (s, k, 3))
+    _gpu(query_uid, "query_uid", torch.int32, (s, q))
+    _gpu(key_uid, "key_uid", torch.int32, (s, k))
+    _gpu(w_offsets, "w_offsets", torch.float32, (16, 3))
+    _gpu(w_distances, "w_distances", torch.float32, (16, 1))
+    _gpu(w_valid, "w_valid", torch.float32, (16, 1))
+    for name, w in (("w_mlp1", w_mlp1), ("w_mlp2", w_mlp2), ("w_mlp3", w_mlp3)):
+        _gpu(w, name, torch.float32, (16, 16))
+    out = torch.empty((s, q, k, 16), dtype=torch.float32, device=row.device)
+    rc = lib.af3_atom_pair_cond_forward(_p(row), _p(col), _p(token_pair), _p(query_token), _p(key_token), n_tok,
+                                        _p(query_pos), _p(key_pos), _p(query_uid), _p(key_uid), _p(w_offsets),
+                                        _p(w_distances), _p(w_valid), _p(w_mlp1), _p(w_mlp2), _p(w_mlp3), _p(out), s, q, k,
+                                        _stream(row.device))
+    _L.check(rc, "af3_atom_pair_cond_forward")
+    return out
+
+
+def atom_pair_logits(pair_cond, ln_w, w, num_blocks: int, num_head: int):
+    """LayerNorm (weight, no bias) and 16 -> blocks x heads projection of the atom pair conditioning, written as
+    the [blocks, S, heads, Q, K] fp32 bias planes of the windowed attention (af3_atom_pair_logits_forward).
+    pair_cond [S, Q, K, 16] fp32; ln_w [16] fp32; w [blocks * heads, 16] fp32."""
+    lib = _L.load()
+    _gpu(pair_cond, "pair_cond", torch.float32)
+    if pair_cond.dim() != 4 or pair_cond.shape[-1] != 16:
+        raise ValueError(f"pair_cond: expected [S, Q, K, 16], got {tuple(pair_cond.shape)}")
+    s, q, k, _ = pair_cond.shape
+    _gpu(ln_w, "ln_w", torch.float32, (16,))
+    _gpu(w, "w", torch.float32, (num_blocks * num_head, 16))
+    out = torch.empty((num_blocks, s, num_head, q, k), dtype=torch.float32, device=pair_cond.device)
+    rc = lib.af3_atom_pair_logits_forward(_p(pair_cond), _p(ln_w), _p(w), _p(out), s, q, k, int(num_blocks), int(num_head),
+                                          _stream(pair_cond.device))
+    _L.check(rc, "af3_atom_pair_logits_forward")
+    return out
+
+
 def pair_cond_init(pair, token_ids, ln_w, w_pair, g_hot, g_sum, in_scale: float = 1.0,
                    max_relative_idx: int = 32, max_relative_chain: int = 2):
     """Linear(LayerNorm([pair | relative encoding])) in one pass (af3_pair_cond_init_forward).

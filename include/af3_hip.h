@@ -426,6 +426,39 @@ int af3_narrow_linear_f32_forward(const float* x, const float* w, const float* r
                                   int k, int n_out, int relu_input, af3_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Pair conditioning of the windowed atom attention
+ * (nn/d_atom_cross_attention.py:231-311: row + column conditioning, the trunk pair
+ * conditioning of the two atoms' tokens, offset / distance / validity embeddings of
+ * atoms in one reference frame, then the three-layer MLP with its residual), one
+ * pass per (subset, query, key), 16 channels, fp32:
+ *   a   = row[s,q] + col[s,k] + [both atoms exist] token_pair[query_token[s,q], key_token[s,k]]
+ *         + valid (W_off d + W_dist / (1 + |d|^2) + w_valid),  d = query_pos[s,q] - key_pos[s,k],
+ *         valid = query_uid[s,q] == key_uid[s,k]
+ *   out = a + W3 relu(W2 relu(W1 relu(a)))
+ * row [subsets,queries,16], col [subsets,keys,16], token_pair [n_token,n_token,16] (or
+ * null: no such term), query_token / key_token int32 (negative: no atom in the slot),
+ * positions [.,3], uids int32, weights in nn.Linear layout ([16,3], [16,1], [16,1],
+ * [16,16] x 3, no bias), out [subsets,queries,keys,16].
+ */
+int af3_atom_pair_cond_forward(const float* row, const float* col, const float* token_pair, const int32_t* query_token,
+                               const int32_t* key_token, int64_t n_token, const float* query_pos, const float* key_pos,
+                               const int32_t* query_uid, const int32_t* key_uid, const float* w_offsets,
+                               const float* w_distances, const float* w_valid, const float* w_mlp1, const float* w_mlp2,
+                               const float* w_mlp3, float* out, int64_t subsets, int64_t queries, int64_t keys,
+                               af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Pair logits of the windowed atom transformer for all its blocks
+ * (nn/d_diffusion_transformer.py:510-520: pair_input_layer_norm, then
+ * pair_logits_projection, then the split into blocks and heads), one pass, fp32:
+ *   pair_cond [subsets,queries,keys,16] fp32, ln_w [16] fp32 (the norm has no bias),
+ *   w [num_blocks*num_head,16] fp32 (nn.Linear layout, no bias; at most 32 rows),
+ *   out [num_blocks,subsets,num_head,queries,keys] fp32.
+ */
+int af3_atom_pair_logits_forward(const float* pair_cond, const float* ln_w, const float* w, float* out, int64_t subsets,
+                                 int64_t queries, int64_t keys, int num_blocks, int num_head, af3_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Pair conditioning of the diffusion head, first layer
  * (nn/d_diffusion_head.py:104-116: features_2d = [pair | relative encoding],
  * pair_cond = pair_cond_initial_projection(pair_cond_initial_norm(features_2d))),

@@ -111,6 +111,54 @@ def test_pair_conditioning_first_layer_kernel(gpu_pkg, n, in_dtype):
     compare("pair conditioning, one-hot share alone", got0, want0, 3e-4, 1e-3)
 
 
+@pytest.mark.parametrize("with_tp", [True, False])
+def test_atom_pair_conditioning_kernel(gpu_pkg, with_tp):
+    """ops.atom_pair_cond against the same sum of terms and three-layer MLP written out in float64."""
+    print(f"test_atom_pair_conditioning_kernel with_tp={with_tp}", flush=True)
+    g = gen(512)
+    S, Q, K, n_tok = 5, 32, 128, 11
+    r = lambda *shape: torch.randn(*shape, generator=g)
+    row, col, tp = r(S, Q, 16), r(S, K, 16), r(n_tok, n_tok, 16)
+    tq = torch.randint(-1, n_tok, (S, Q), generator=g)
+    tk = torch.randint(-1, n_tok, (S, K), generator=g)
+    q_pos, k_pos = r(S, Q, 3) * 3, r(S, K, 3) * 3
+    q_uid, k_uid = torch.randint(0, 4, (S, Q), generator=g), torch.randint(0, 4, (S, K), generator=g)
+    w_off, w_dist, w_valid = r(16, 3), r(16, 1), r(16, 1)
+    w1, w2, w3 = r(16, 16) * 0.4, r(16, 16) * 0.4, r(16, 16) * 0.4
+    d = lambda t: t.double()
+    a = d(row)[:, :, None, :] + d(col)[:, None, :, :]
+    if with_tp:
+        live = ((tq >= 0)[:, :, None] & (tk >= 0)[:, None, :])[..., None].double()
+        a = a + d(tp)[tq.clamp(min=0)[:, :, None], tk.clamp(min=0)[:, None, :]] * live
+    valid = (q_uid[:, :, None] == k_uid[:, None, :]).double()[..., None]
+    off = d(q_pos)[:, :, None, :] - d(k_pos)[:, None, :, :]
+    a = a + (off @ d(w_off).T + (1.0 / (1 + (off * off).sum(-1, keepdim=True))) @ d(w_dist).T + d(w_valid)[:, 0]) * valid
+    h = torch.relu(a) @ d(w1).T
+    h = torch.relu(h) @ d(w2).T
+    want = a + torch.relu(h) @ d(w3).T
+    t = lambda x: x.to(dev())
+    i32 = lambda x: x.to(torch.int32).to(dev())
+    got = gpu_pkg.ops.atom_pair_cond(t(row), t(col), t(tp) if with_tp else None, i32(tq) if with_tp else None,
+                                     i32(tk) if with_tp else None, t(q_pos), t(k_pos), i32(q_uid), i32(k_uid),
+                                     t(w_off), t(w_dist), t(w_valid), t(w1), t(w2), t(w3))
+    compare("atom pair conditioning", got, want, 2e-6, 2e-5)
+
+
+def test_atom_pair_logits_kernel(gpu_pkg):
+    """ops.atom_pair_logits against LayerNorm + projection + the block / head split in float64."""
+    print("test_atom_pair_logits_kernel", flush=True)
+    g = gen(411)
+    S, Q, K, blocks, heads = 7, 32, 128, 3, 4
+    x = torch.randn(S, Q, K, 16, generator=g) * 3 + 1
+    ln_w = 1 + 0.3 * torch.randn(16, generator=g)
+    w = torch.randn(blocks * heads, 16, generator=g)
+    want = torch.nn.functional.layer_norm(x.double(), (16,), ln_w.double(), None, 1e-5) @ w.double().T
+    want = want.reshape(S, Q, K, blocks, heads).permute(3, 0, 4, 1, 2)
+    got = gpu_pkg.ops.atom_pair_logits(x.to(dev()), ln_w.to(dev()), w.to(dev()), blocks, heads)
+    assert tuple(got.shape) == (blocks, S, heads, Q, K)
+    compare("atom pair logits", got, want, 2e-6, 2e-5)
+
+
 def test_state_reuse_is_exact_and_samples_are_independent(gpu_pkg):
     g, batch, p, emb, pos, head = case(gpu_pkg, 16, 4, seed=31, samples=3)
     gb, ge = batch.to(dev()), on_gpu(emb)
