@@ -495,6 +495,21 @@ def test_kernel_level_contraction(gpu_pkg, n):
     assert_within_bf16_ulp("contraction", t[:, :, :n].cpu(), want.cpu(), ulps=1.01, atol=1e-3)
 
 
+def test_kernel_level_contraction_at_the_target_token_count(gpu_pkg):
+    """N = 1536 (4608 blocks of 256 x 256: 18 per persistent workgroup), compared on the device 16
+    channels at a time."""
+    note("test_kernel_level_contraction_at_the_target_token_count")
+    n = 1536
+    g = gen(n)
+    a = rb(torch.randn(128, n, n, generator=g)).to(dev())
+    b = rb(torch.randn(128, n, n, generator=g)).to(dev())
+    t = gpu_pkg.ops.triangle_contraction(a.bfloat16(), b.bfloat16())
+    for c0 in range(0, 128, 16):
+        want = torch.bmm(a[c0:c0 + 16].double(), b[c0:c0 + 16].double().transpose(1, 2))
+        bad = (t[c0:c0 + 16].double() - want).abs() > 1.01 * 2.0 ** -8 * want.abs() + 1e-3
+        assert not bool(bad.any()), f"channels {c0}..: {int(bad.sum())} elements beyond 1.01 bf16 ulp"
+
+
 @pytest.mark.parametrize("batch,m,n,k", [
     (8, 2048, 1792, 16),      # less than one 32-deep slab of k, 448 tiles: several per workgroup
     (3, 2300, 1100, 40),      # partial tiles on both edges and a k tail
