@@ -8,8 +8,10 @@
 // between the two lane halves.  The same registers, rounded to bf16, are
 // directly the B fragments of O^T += V^T P^T (the MFMA k index is a summation
 // index, so the key order inside a fragment is free as long as the V^T
-// fragment uses the same order).  K and V^T tiles of 64 keys are staged in LDS,
-// double-buffered, and shared by the workgroup's waves.
+// fragment uses the same order).  K and V tiles of 64 keys are staged in LDS row
+// by row as they lie in memory, double-buffered and shared by the workgroup's
+// waves; the V^T fragments come out of the transposing LDS read of this target
+// (ds_read_b64_tr_b16), so nothing is transposed on the way in.
 //
 // Logit = q.k (q pre-scaled) + pair_bias[h][q][k]; then
 //   key_mask:  keys with mask 0 are REPLACED by -1e9 (so a fully masked row is
@@ -23,8 +25,13 @@
 namespace {
 
 constexpr int KT = 64;        // keys per LDS tile
-constexpr int LDV = KT + 4;   // sVt row stride (bf16): 34 dwords, 32 rows' 8-byte reads hit 32 bank pairs
 constexpr float NEG_INF = -__builtin_huge_valf();
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef short v8s __attribute__((ext_vector_type(8)));
+// ds_read_b64_tr_b16: four 16-bit elements per lane, transposed within each group of 16 lanes
+__device__ __forceinline__ v4s lds_read_tr16(const bf16_t* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)p);
+}
 constexpr float LOG2E = 1.4426950408889634f;
 // per-key code staged in LDS next to the K tile
 constexpr int KEY_MASKED = 1, KEY_PAD = 2, KEY_BEYOND = 4;
@@ -38,13 +45,16 @@ constexpr int KEY_MASKED = 1, KEY_PAD = 2, KEY_BEYOND = 4;
 template <int KSTEPS, int DVT, int NW, bool FAST>
 // at least two waves per SIMD: the register allocator then keeps everything in
 // the 256 architectural VGPRs instead of parking loop state in accumulation
-// registers, which would leave a single wave per SIMD
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) void flash_kernel(FlashArgs a) {
+// registers, which would leave a single wave per SIMD (the one-wave workgroup of
+// head dimension 48 stages twelve chunks per thread and is given the whole register file)
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(KSTEPS == 3 && NW == 1 ? 1 : 2)))
+void flash_kernel(FlashArgs a) {
   constexpr int KD = KSTEPS * 16;  // padded q/k head dim
   constexpr int LDK = KD + 8;      // sK row stride (bf16)
   constexpr int NT = NW * 64;
   __shared__ __attribute__((aligned(16))) bf16_t sK[2][KT * LDK];
-  __shared__ __attribute__((aligned(16))) bf16_t sVt[2][DVT * 32 * LDV];
+  constexpr int LDV = DVT * 32 + 8;  // sV row stride (bf16): V rows as they are, padded to the 32 DVT columns the products read
+  __shared__ __attribute__((aligned(16))) bf16_t sV[2][KT * LDV];
   __shared__ __attribute__((aligned(16))) int sCode[2][KT];
   __shared__ int sAnyCode[2];  // whether any key of the staged tile carries a code
 
@@ -100,9 +110,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   // from a clamped address, and nothing is decided from a loaded value before
   // the LDS store one tile later: a load under a lane mask, or a value
   // inspected right after its load, costs a full memory round trip per tile.
-  //   K: chunk id = key * (KD/8) + c, c fastest (one key row is contiguous)
-  //   V: chunk id = c * KT + key, key fastest, so that the transposing 2-byte
-  //      LDS stores of a wave walk along a V^T row instead of down a column
+  //   chunk id = key * (KD/8) + c, c fastest (one key row is contiguous), for K and for V alike: both go to
+  //   LDS row by row as they lie in memory
   // The K chunks of a tile and then its V chunks form one list of 2 KCH entries that the threads share out
   // evenly: thread t moves entries t, t + NT, ..  (head dimension 48 with 256 threads: three each, the
   // middle one a K chunk for waves 0 and 1 and a V chunk for waves 2 and 3; whether an entry is K or V is
@@ -118,7 +127,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   const float* kmask = a.key_mask ? a.key_mask + (int64_t)b * a.km_sb : nullptr;
   const float* kpad = a.kpad ? a.kpad + (int64_t)bb * a.kp_sb : nullptr;
   int k0_loaded = 0;
-  // entry i of this thread: K chunk (key = e / (KD/8), c = e % (KD/8)) or V chunk (key = e % KT, c = e / KT)
+  // entry i of this thread: chunk e (K) or e - KCH (V) of its tile, key = chunk / (KD/8), c = chunk % (KD/8)
   bool is_v[NL];
   int ch_key[NL], ch_c[NL];
   // FAST: byte offset of the chunk from the first key row of a tile (the launcher has checked that 64 rows
@@ -128,8 +137,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   for (int i = 0; i < NL; ++i) {
     const int e = tid + i * NT;
     is_v[i] = e >= KCH;
-    ch_key[i] = is_v[i] ? (e - KCH) % KT : e / (KD / 8);
-    ch_c[i] = is_v[i] ? (e - KCH) / KT : e % (KD / 8);
+    const int ch = is_v[i] ? e - KCH : e;
+    ch_key[i] = ch / (KD / 8);
+    ch_c[i] = ch % (KD / 8);
     choff[i] = (uint32_t)(ch_key[i] * (is_v[i] ? a.v_ss : a.k_ss) + (ch_c[i] < dch ? ch_c[i] : 0) * 8) * 2u;
   }
   // Rows of the chunks this thread moves.  With key_rows they are looked
@@ -173,15 +183,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
       const int key = ch_key[i], c = ch_c[i];
       const bool ok = k0_loaded + key < a.Sk && c < dch && (FAST || row_ok[i]);  // (FAST: rows are never negative)
       const u32x4 vv = ok ? rc[i] : z;
-      if (!is_v[i]) {
-        *reinterpret_cast<u32x4*>(&sK[buf][key * LDK + c * 8]) = vv;
-      } else if (c * 8 < DVT * 32) {
-        const uint32_t w4[4] = {vv.x, vv.y, vv.z, vv.w};
-        bf16_t* dst = &sVt[buf][(c * 8) * LDV + key];
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          dst[e * LDV] = (bf16_t)((e & 1) ? (w4[e >> 1] >> 16) : (w4[e >> 1] & 0xffffu));
-      }
+      if (!is_v[i]) *reinterpret_cast<u32x4*>(&sK[buf][key * LDK + c * 8]) = vv;
+      else *reinterpret_cast<u32x4*>(&sV[buf][key * LDV + c * 8]) = vv;
     }
     if (tid < KT) {  // wave 0, all of it (KT = 64)
       const int code = (k0_loaded + tid >= a.Sk ? KEY_BEYOND : 0) | (rkm == 0.f ? KEY_MASKED : 0) | (rkp == 0.f ? KEY_PAD : 0);
@@ -190,13 +193,15 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
       if (tid == 0) sAnyCode[buf] = any ? 1 : 0;
     }
   };
-  // V^T rows that no chunk covers (head dim padding: rows KD .. 32 DVT - 1 of
-  // either buffer) must read as zero
+  // V columns that no chunk covers (head dimension padding: columns KD .. 32 DVT - 1 of either buffer) must
+  // read as zero
   if constexpr (KD < DVT * 32) {
-    constexpr int PAD_WORDS = (DVT * 32 - KD) * LDV / 2;
-    for (int idx = tid; idx < 2 * PAD_WORDS; idx += NT)
-      reinterpret_cast<uint32_t*>(&sVt[idx / PAD_WORDS][KD * LDV])[idx % PAD_WORDS] = 0u;
-  }  // (no tile store touches these rows; the barrier after the first tile's stores orders them too)
+    constexpr int PAD = DVT * 32 - KD;  // a multiple of 16
+    for (int idx = tid; idx < 2 * KT * (PAD / 2); idx += NT) {
+      const int row = idx / (PAD / 2), w = idx % (PAD / 2);
+      reinterpret_cast<uint32_t*>(&sV[row / KT][(row % KT) * LDV + KD])[w] = 0u;
+    }
+  }  // (no tile store touches these columns; the barrier after the first tile's stores orders them too)
 
   f32x16 o[DVT];
 #pragma unroll
@@ -382,20 +387,25 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
         for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
     }
     // O^T[dd][query] += sum_key V^T[dd][key] P^T[key][query]; fragment element e
-    // of lane-half hh in k-step `half` is key 32u + 16*half + 8*(e>>2) + 4*hh + (e&3)
+    // of lane-half hh in k-step `half` is key 32u + 16*half + 8*(e>>2) + 4*hh + (e&3).  V lies in LDS as it
+    // lies in memory, [key][dd]; the transposing LDS read hands each lane of a group of 16 one column of a
+    // 4-row x 16-column block (lane i of the group points at row i / 4, columns 4 (i % 4) .. of the block
+    // and receives column i of its four rows): rows = four consecutive keys, columns = the group's 16 dd.
+    {
+      const int i16 = lane & 15;
+      const bf16_t* vbase = &sV[buf][(4 * hh + (i16 >> 2)) * LDV + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3)];
 #pragma unroll
-    for (int t = 0; t < DVT; ++t)
+      for (int t = 0; t < DVT; ++t)
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+        for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const bf16_t* vp = &sVt[buf][(t * 32 + j) * LDV + u * 32 + 16 * half + 4 * hh];
-          const u32x2 lo = *reinterpret_cast<const u32x2*>(vp);
-          const u32x2 hi = *reinterpret_cast<const u32x2*>(vp + 8);
-          u32x4 vv;
-          vv.x = lo.x; vv.y = lo.y; vv.z = hi.x; vv.w = hi.y;
-          o[t] = mfma32(as_frag(vv), pf[u][half], o[t]);
-        }
+          for (int half = 0; half < 2; ++half) {
+            const bf16_t* vp = vbase + (u * 32 + 16 * half) * LDV + t * 32;
+            const v4s lo = lds_read_tr16(vp), hi = lds_read_tr16(vp + 8 * LDV);
+            o[t] = mfma32(as_frag(__builtin_bit_cast(u32x4, v8s{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w})),
+                          pf[u][half], o[t]);
+          }
+    }
     if (kt + 1 < nkt) sstore(buf ^ 1);
     lds_barrier();
   };
