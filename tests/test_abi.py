@@ -176,6 +176,26 @@ def test_gathered_relu_mean_rejects_bad_arguments(pkg):
     assert lib.af3_atom_position_features_forward(one, one, one, one, one, 0, 1, 8, 8, 100, None) == -1    # channels % 8
 
 
+def test_conditioning_kernels_reject_bad_arguments(pkg):
+    """The per-batch conditioning entry points of the diffusion head check their arguments before any launch."""
+    lib = pkg.lib.load()
+    one = 1 << 20
+    ids = (one, one, one, one, one)
+    ok_tail = (32, 2, one, one, one, one, one, 16, None)
+    assert lib.af3_pair_cond_init_forward(None, 0, 1.0, *ids, *ok_tail) == -1                        # no pair tensor
+    assert lib.af3_pair_cond_init_forward(one, 5, 1.0, *ids, *ok_tail) == -1                         # dtype
+    assert lib.af3_pair_cond_init_forward(one, 0, 1.0, one, one, None, one, one, *ok_tail) == -1     # a token feature missing
+    assert lib.af3_pair_cond_init_forward(one, 0, 1.0, *ids, 32, 2, one, one, one, one, one, 0, None) == -1    # n = 0
+    assert lib.af3_pair_cond_init_forward(one + 4, 0, 1.0, *ids, *ok_tail) == -1                     # misaligned
+    assert lib.af3_atom_pair_logits_forward(one, one, one, None, 4, 32, 128, 3, 4, None) == -1       # no output
+    assert lib.af3_atom_pair_logits_forward(one, one, one, one, 4, 32, 128, 9, 4, None) != 0         # more than 32 planes
+    assert lib.af3_atom_pair_logits_forward(one, one, one, one, 4, 0, 128, 3, 4, None) == -1         # no queries
+    w = (one, one, one, one, one, one)
+    assert lib.af3_atom_pair_cond_forward(one, None, None, None, None, 0, one, one, one, one, *w, one, 4, 32, 128, None) == -1
+    assert lib.af3_atom_pair_cond_forward(one, one, one, None, one, 8, one, one, one, one, *w, one, 4, 32, 128, None) == -1  # token table missing
+    assert lib.af3_atom_pair_cond_forward(one, one, None, None, None, 0, one, one, one, one, *w, one, 0, 32, 128, None) == -1
+
+
 def test_new_modules_share_the_reference_parameter_names(pkg):
     from oracle import af3_head_oracle as H
     from oracle import af3_msa_oracle as M
