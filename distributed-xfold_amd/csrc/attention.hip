@@ -53,7 +53,11 @@ void flash_kernel(FlashArgs a) {
   constexpr int LDK = KD + 8;      // sK row stride (bf16)
   constexpr int NT = NW * 64;
   __shared__ __attribute__((aligned(16))) bf16_t sK[2][KT * LDK];
-  constexpr int LDV = DVT * 32 + 8;  // sV row stride (bf16): V rows as they are, padded to the 32 DVT columns the products read
+  // sV row stride (bf16): V rows as they are, padded to the 32 DVT columns the products read.  A transposing
+  // read touches 8 rows x 64 bytes; with a row stride of 16 or 48 dwords modulo the 64 banks (32 or 96
+  // elements) these tile the banks exactly twice, the minimum for its 512 bytes.
+  constexpr int LDV = DVT == 1 ? 32 : 96;
+  static_assert(LDV >= DVT * 32, "a row holds every column the products read");
   __shared__ __attribute__((aligned(16))) bf16_t sV[2][KT * LDV];
   __shared__ __attribute__((aligned(16))) int sCode[2][KT];
   __shared__ int sAnyCode[2];  // whether any key of the staged tile carries a code
